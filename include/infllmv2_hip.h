@@ -1,0 +1,136 @@
+/*
+ * C ABI of libinfllmv2_hip.so — gfx950 (MI355X) kernels for the InfLLM-V2 two-stage sparse
+ * attention path.
+ *
+ * Every function takes plain device pointers, sizes and a HIP stream handle (passed as void*,
+ * null = the default stream), launches asynchronously on that stream, allocates nothing and
+ * returns 0 on success.  A non-zero return means nothing was launched by the failing step;
+ * infllmv2_last_error() then holds a message (thread-local).  "uint64" masks are the int64
+ * tensors of the reference (bit 63 set = negative value).
+ *
+ * Each declaration cites the interface of the reference (paths relative to the reference
+ * checkout) that it replaces.  Where the reference's pybind function takes at::Tensor arguments
+ * the tensor is flattened here into pointer + sizes + strides, and outputs/scratch that the
+ * reference allocates internally are passed in by the caller.
+ */
+#ifndef INFLLMV2_HIP_H
+#define INFLLMV2_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define INFLLMV2_ABI_VERSION 1
+
+/* ---- library ------------------------------------------------------------------------------ */
+
+const char* infllmv2_last_error(void);
+int infllmv2_abi_version(void);
+/* 0 iff `device` is a gfx950 GPU.  Replaces the sm80/sm90 gate of
+ * csrc/flash_attn/flash_api.cpp:546-550. */
+int infllmv2_check_device(int device);
+
+/* ---- block-mask bit operations -------------------------------------------------------------- */
+
+/* csrc/entry.cu:78-96 `topk_to_uint64` (kernel csrc/topk_to_uint64.cuh:10-76).
+ * topk_idx (rows, k) int32, result (rows, n_uint64_per_row); entries < 0 are skipped. */
+int infllmv2_topk_to_uint64(void* stream, const int32_t* topk_idx, uint64_t* result, int64_t rows,
+                            int k, int k_blocks, int n_uint64_per_row);
+
+/* csrc/entry.cu:98-114 `uint64_to_bool` (kernel csrc/uint64_to_bool.cuh:10-66).
+ * result (rows, last_dim_size) bytes of 0/1. */
+int infllmv2_uint64_to_bool(void* stream, const uint64_t* input, uint8_t* result, int64_t rows,
+                            int last_dim_size, int n_uint64_per_row);
+
+/* csrc/entry.cu:61-76 `blockmask_to_uint64` (kernel csrc/blockmask_to_uint64.cuh:10-74). */
+int infllmv2_blockmask_to_uint64(void* stream, const uint8_t* blockmask, uint64_t* result,
+                                 int64_t rows, int last_dim_size, int n_uint64_per_row);
+
+/* Replaces the uint64_to_bool -> transpose -> synchronize -> blockmask_to_uint64 sequence of
+ * infllm_v2/infllmv2_sparse_attention.py:344-350 with one launch.
+ * fwd_mask (heads, total_q, n64_fwd) -> bwd_mask (heads, k_blocks, n64_bwd = ceil(total_q/64)):
+ * bwd[h, kb, w] bit u = fwd[h, 64 w + u, kb / 64] bit (kb % 64). */
+int infllmv2_transpose_blockmask(void* stream, const uint64_t* fwd_mask, uint64_t* bwd_mask, int heads,
+                                 int64_t total_q, int n64_fwd, int k_blocks, int n64_bwd);
+
+/* ---- pooling and selection ------------------------------------------------------------------ */
+
+/* csrc/entry.cu:116-154 `max_pooling_1d` (kernel csrc/max_pooling_1d.cuh:107-160, 203-227).
+ * dtype: 0 = fp16, 1 = bf16.  input (num_heads, q_len, k_len), output (num_heads, q_len, out_len). */
+int infllmv2_max_pooling_1d(void* stream, const void* input, void* output, int dtype, int num_heads,
+                            int q_len, int k_len, int out_len, int cache_len, int kernel_size,
+                            int stride, int padding, int block_size, int local_blocks, int init_blocks);
+
+/* Same operator for an input whose rows are not densely packed (strides in elements), so the
+ * padded score buffer of Stage 1 is pooled in place instead of being copied first
+ * (the reference forces `.contiguous()`, infllm_v2/max_pooling_1d.py:13). */
+int infllmv2_max_pooling_1d_strided(void* stream, const void* input, void* output, int dtype,
+                                    int num_heads, int q_len, int k_len, int64_t in_head_stride,
+                                    int64_t in_row_stride, int out_len, int cache_len, int kernel_size,
+                                    int stride, int padding, int block_size, int local_blocks,
+                                    int init_blocks);
+
+/* csrc/entry.cu:156-195 `max_pooling_1d_varlen` (kernel csrc/max_pooling_1d.cuh:12-103, 165-199).
+ * Like the reference this variant reads cu_seqlens_q[batch_size] back to the host (one stream
+ * synchronisation) to learn the number of packed rows. */
+int infllmv2_max_pooling_1d_varlen(void* stream, const void* input, void* output,
+                                   const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                                   const int32_t* cache_lens, int dtype, int batch_size, int num_heads,
+                                   int max_seqlen_q, int max_seqlen_k, int out_len, int kernel_size,
+                                   int stride, int padding, int block_size, int local_blocks,
+                                   int init_blocks);
+
+/* The same with the packed row count and input strides given by the caller: no host sync. */
+int infllmv2_max_pooling_1d_varlen_strided(void* stream, const void* input, void* output,
+                                           const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                                           const int32_t* cache_lens, int dtype, int batch_size,
+                                           int num_heads, int total_q, int max_seqlen_q,
+                                           int max_seqlen_k, int64_t in_head_stride,
+                                           int64_t in_row_stride, int out_len, int kernel_size,
+                                           int stride, int padding, int block_size, int local_blocks,
+                                           int init_blocks);
+
+/* csrc/entry.cu:31-45 `topk` (kernel csrc/topk.cuh:99-181): per row of `dim` values the `top`
+ * largest (value descending, equal values by ascending position); output rows have stride
+ * top_size = next power of two >= top (csrc/topk.cuh:108,119-141).  Unlike the reference
+ * (dim <= 1024, top <= 32) rows up to 8192 and top up to 2048 are accepted. */
+int infllmv2_topk(void* stream, int num_tokens, int dim, int top, int dtype, const void* x,
+                  void* topk_val, int32_t* topk_pos);
+
+/* Block selection between pooling and packing.  The reference leaves this step to the caller
+ * (README.md:42,125-126: torch.topk); its stated order is csrc/topk.cuh:17,26,37.
+ * pooled: rows of n 16-bit scores (fp16 or bf16 bits; row stride in elements);
+ * topk_idx (rows, k) int32 = first k columns of a stable descending sort, -1 padded. */
+int infllmv2_topk_blocks(void* stream, const void* pooled, int64_t row_stride, int32_t* topk_idx,
+                         int64_t rows, int n, int k);
+
+/* ---- Stage 2: block-sparse attention -------------------------------------------------------- */
+
+/* Scratch needed by infllmv2_varlen_fwd / _bwd for the fragment-major K/V block images. */
+size_t infllmv2_kv_image_bytes(int64_t total_k, int batch, int num_heads_k);
+
+/* csrc/entry.cu:14,210 `varlen_fwd` = mha_varlen_fwd (csrc/flash_attn/flash_api.cpp:519-782) on
+ * the sparse path (blockmask given) and on the dense path (blockmask null).
+ * bf16, head_dim 128, num_heads == 16 * num_heads_k.
+ * q/out: element strides {token, head-in-group, kv-head}; the caller's (T, Hq, d) tensor is
+ *   {Hq*d, d, 16*d}; the reference's re-laid-out (T*16, Hk, d) tensor is {16*Hk*d, Hk*d, d}.
+ * k/v: (total_k, Hk, d), strides {row, head}.  softmax_lse strides {token, head-in-group, kv-head};
+ *   the reference's (Hk, T*16) layout (flash_api.cpp:665) is {16, 1, T*16}.
+ * blockmask (Hk, total_q, n_uint64_per_row): block indices local to each sequence, rows by packed
+ *   token index (flash_blockmask.h:20-31). */
+int infllmv2_varlen_fwd(void* stream, const void* q, const void* k, const void* v, void* out,
+                        float* softmax_lse, const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                        const uint64_t* blockmask, void* workspace, size_t workspace_bytes, int batch,
+                        int64_t total_q, int64_t total_k, int num_heads, int num_heads_k, int head_dim,
+                        int max_seqlen_q, int max_seqlen_k, const int64_t* q_strides,
+                        const int64_t* k_strides, const int64_t* v_strides, const int64_t* o_strides,
+                        const int64_t* lse_strides, int n_uint64_per_row, float softmax_scale,
+                        int is_causal);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* INFLLMV2_HIP_H */

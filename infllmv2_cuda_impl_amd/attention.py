@@ -1,0 +1,249 @@
+"""Stage-1 scoring, Stage-2 block-sparse attention (forward/backward) and decode.
+
+Host-side counterpart of infllm_v2/infllmv2_sparse_attention.py of the reference: same function
+names, arguments and results.  The reference re-lays-out q / out / dout into a
+``(T*16, Hk, d)`` tensor before every kernel call (lines 71-95, 174-191, 551-559 there); here the
+kernels address the caller's ``(T, Hq, d)`` tensors through strides, so no copy is made.
+"""
+from __future__ import annotations
+
+from typing import Optional, Union
+
+import torch
+
+from . import _lib
+from ._util import ptr, require_gpu, stream_ptr
+from .masks import topk_to_uint64, transpose_blockmask
+
+GROUP = 16          # query heads per KV head the kernels are built for (flash_api.cpp:941)
+BLOCK_N = 64        # key-block size of the sparse mask (infllmv2_sparse_attention.py:93)
+
+
+def _dense_last_dim(x):
+    return x.contiguous() if x is not None and x.stride(-1) != 1 else x
+
+
+def _reject_unsupported(dropout_p, window_size, softcap, alibi_slopes, causal):
+    """Options the reference build compiles out (setup.py:235-239) fail with its messages
+    (flash_api.cpp:107-109, 131-133, 144-147, 330-332)."""
+    if softcap > 0.0:
+        raise RuntimeError("This flash attention build does not support softcap.")
+    if not dropout_p < 1.0:
+        raise RuntimeError("Expected p_dropout < 1.f to be true, but got false.")
+    if dropout_p != 0.0:
+        raise RuntimeError("This flash attention build does not support dropout.")
+    wl, wr = window_size
+    if causal:
+        wr = 0
+    is_causal = wl < 0 and wr == 0
+    if not (is_causal or (wl < 0 and wr < 0)):
+        raise RuntimeError("This flash attention build does not support local attention.")
+    if alibi_slopes is not None:
+        raise RuntimeError("This flash attention build does not support alibi.")
+
+
+def _check_qkv(q, k, v, cu_seqlens_q, cu_seqlens_k):
+    """Input checks of mha_varlen_fwd (flash_api.cpp:552-616) that apply to this build."""
+    if q.dtype not in (torch.float16, torch.bfloat16):
+        raise RuntimeError("FlashAttention only support fp16 and bf16 data type")
+    if k.dtype != q.dtype:
+        raise RuntimeError("query and key must have the same dtype")
+    if v.dtype != q.dtype:
+        raise RuntimeError("query and value must have the same dtype")
+    if q.dtype != torch.bfloat16:
+        # the reference build instantiates bf16 kernels only (static_switch.h:79-83)
+        raise RuntimeError("this build only has bf16 kernels")
+    if cu_seqlens_q.dtype != torch.int32:
+        raise RuntimeError("cu_seqlens_q must have dtype int32")
+    if cu_seqlens_k.dtype != torch.int32:
+        raise RuntimeError("cu_seqlens_k must have dtype int32")
+    for name, t in (("q", q), ("k", k), ("v", v), ("cu_seqlens_q", cu_seqlens_q), ("cu_seqlens_k", cu_seqlens_k)):
+        require_gpu(t, name)
+    for t in (q, k, v):
+        if t.stride(-1) != 1:
+            raise RuntimeError("Input tensor must have contiguous last dimension")
+    if not cu_seqlens_q.is_contiguous():
+        raise RuntimeError("cu_seqlens_q must be contiguous")
+    if not cu_seqlens_k.is_contiguous():
+        raise RuntimeError("cu_seqlens_k must be contiguous")
+    batch = cu_seqlens_q.numel() - 1
+    if batch <= 0:
+        raise RuntimeError("batch size must be positive")
+    if q.dim() != 3 or k.dim() != 3 or v.dim() != 3:
+        raise RuntimeError("q, k, v must have shape (total, nheads, headdim)")
+    head_size = q.shape[2]
+    if head_size > 256:
+        raise RuntimeError("FlashAttention forward only supports head dimension at most 256")
+    if head_size % 8 != 0:
+        raise RuntimeError("query, key, value, and out_ must have a head_size that is a multiple of 8")
+    if q.shape[1] % k.shape[1] != 0:
+        raise RuntimeError("Number of heads in key/value must divide number of heads in query")
+    if tuple(k.shape) != (k.shape[0], k.shape[1], head_size) or tuple(v.shape) != tuple(k.shape):
+        raise RuntimeError("k and v must have shape (total_k, num_heads_k, head_size)")
+    if cu_seqlens_k.numel() != batch + 1:
+        raise RuntimeError("cu_seqlens_k must have shape (batch_size + 1)")
+    if head_size != 128:
+        raise RuntimeError("this build only supports head dimension 128")
+    if q.shape[1] != GROUP * k.shape[1]:
+        raise RuntimeError("this build requires 16 query heads per key/value head")
+    return batch
+
+
+def _natural_strides(t: torch.Tensor):
+    """{token, head-in-group, kv-head} element strides of a (T, Hq, d) tensor."""
+    return _lib.i64_array([t.stride(0), t.stride(1), GROUP * t.stride(1)])
+
+
+def _sparse_forward(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, softmax_scale, causal,
+                    fwd_mask, lse_expanded: bool):
+    """Runs the Stage-2 forward kernel.  Returns (out (T,Hq,d), lse)."""
+    batch = cu_seqlens_q.numel() - 1
+    total_q, Hq, d = q.shape
+    total_k, Hk = k.shape[0], k.shape[1]
+    out = torch.empty_like(q)
+    if lse_expanded:
+        lse = torch.empty((Hk, total_q * GROUP), dtype=torch.float32, device=q.device)       # flash_api.cpp:665
+        lse_strides = _lib.i64_array([GROUP, 1, total_q * GROUP])
+    else:
+        lse = torch.empty((Hq, total_q), dtype=torch.float32, device=q.device)
+        lse_strides = _lib.i64_array([1, total_q, GROUP * total_q])
+    ws_bytes = _lib.lib.infllmv2_kv_image_bytes(total_k, batch, Hk)
+    workspace = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=q.device)
+    n64 = 0 if fwd_mask is None else fwd_mask.shape[-1]
+    with torch.cuda.device(q.device):
+        _lib.call("infllmv2_varlen_fwd", stream_ptr(q.device), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                  out.data_ptr(), lse.data_ptr(), cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), ptr(fwd_mask),
+                  workspace.data_ptr(), workspace.numel(), batch, total_q, total_k, Hq, Hk, d, max_seqlen_q,
+                  max_seqlen_k, _natural_strides(q), _lib.i64_array([k.stride(0), k.stride(1)]),
+                  _lib.i64_array([v.stride(0), v.stride(1)]), _natural_strides(out), lse_strides, n64,
+                  float(softmax_scale), int(bool(causal)))
+    return out, lse
+
+
+class Infllmv2AttnVarlenFunc(torch.autograd.Function):
+    """Autograd wrapper (infllmv2_sparse_attention.py:275-385 of the reference)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p, softmax_scale,
+                causal, window_size, softcap, alibi_slopes, deterministic, return_softmax, block_table, topk_idx):
+        if softmax_scale is None:
+            softmax_scale = q.shape[-1] ** (-0.5)
+        _reject_unsupported(dropout_p, window_size, softcap, alibi_slopes, causal)
+        if block_table is not None:
+            raise RuntimeError("paged KV (block_table) is not supported by this build")
+        q, k, v = [_dense_last_dim(x) for x in (q, k, v)]
+        _check_qkv(q, k, v, cu_seqlens_q, cu_seqlens_k)
+        fwd_mask = None
+        if topk_idx is not None:
+            assert topk_idx.dtype == torch.int32
+            fwd_mask, _ = topk_to_uint64(topk_idx, max_seqlen_k, BLOCK_N)
+            if fwd_mask.dim() != 3 or fwd_mask.shape[0] != k.shape[1] or fwd_mask.shape[1] != q.shape[0]:
+                raise RuntimeError("topk_idx must have shape (num_heads_k, total_q, k)")
+        out, lse = _sparse_forward(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
+                                   softmax_scale, causal, fwd_mask, lse_expanded=topk_idx is not None)
+        ctx.save_for_backward(q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, fwd_mask)
+        ctx.max_seqlen_q = max_seqlen_q
+        ctx.max_seqlen_k = max_seqlen_k
+        ctx.softmax_scale = softmax_scale
+        ctx.causal = causal
+        ctx.deterministic = deterministic
+        ctx.sparse = topk_idx is not None
+        if not return_softmax:
+            return out
+        # S_dmask is only materialised with dropout, which this build rejects
+        # (infllmv2_sparse_attention.py:319, flash_api.cpp:672-674): an empty tensor is returned.
+        s_dmask = torch.empty((0,), dtype=q.dtype, device=q.device)
+        ctx.mark_non_differentiable(lse, s_dmask)
+        return out, lse, s_dmask
+
+    @staticmethod
+    def backward(ctx, dout, *args):
+        from .backward import sparse_backward
+        q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, fwd_mask = ctx.saved_tensors
+        dq, dk, dv = sparse_backward(dout, q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, ctx.max_seqlen_q,
+                                     ctx.max_seqlen_k, ctx.softmax_scale, ctx.causal, fwd_mask, ctx.sparse)
+        return (dq, dk, dv) + (None,) * 14
+
+
+def infllmv2_attn_varlen_func(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p=0.0,
+                              softmax_scale=None, causal=False, window_size=(-1, -1), softcap=0.0,
+                              alibi_slopes=None, deterministic=False, return_attn_probs=False, block_table=None,
+                              topk_idx=None):
+    """Block-sparse (or, with ``topk_idx=None``, dense) attention over packed variable-length sequences.
+
+    q ``(total_q, nheads, 128)``, k/v ``(total_k, nheads_k, 128)`` bf16 with ``nheads == 16*nheads_k``;
+    ``cu_seqlens_q/k`` int32 ``(batch+1,)``.  ``topk_idx`` int32 ``(nheads_k, total_q, k)`` lists, per KV head
+    and packed query token, the 64-key blocks (indices local to the token's sequence, ``-1`` = unused) the
+    token attends to; all 16 query heads of a group share the row.  ``causal=True`` aligns the causal mask to
+    the bottom-right corner; a query with no visible key yields zeros.  Differentiable w.r.t. q, k, v.
+
+    Returns ``out (total_q, nheads, 128)``; with ``return_attn_probs`` the tuple ``(out, softmax_lse, S_dmask)``
+    where ``softmax_lse`` is fp32 ``(nheads_k, total_q*16)`` with column ``t*16 + g`` on the sparse path
+    (``(nheads, total_q)`` on the dense path) and ``S_dmask`` is empty.  dropout, softcap, ALiBi, sliding
+    windows and paged KV are rejected exactly as the reference build rejects them.
+    """
+    return Infllmv2AttnVarlenFunc.apply(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p,
+                                        softmax_scale, causal, window_size, softcap, alibi_slopes, deterministic,
+                                        return_attn_probs, block_table, topk_idx)
+
+
+def infllmv2_attn_stage1(q, k, v, cu_seqlens_q, cu_seqlens_k, cu_seqlens_v, max_seqlen_q, max_seqlen_k,
+                         dropout_p=0.0, softmax_scale=None, causal=False, window_size=(-1, -1), softcap=0.0,
+                         alibi_slopes=None, deterministic=False, return_attn_probs=True, block_table=None):
+    """Stage-1 group scores over compressed keys.
+
+    q ``(total_q, nheads, 128)``; k ``(sum Lk, nheads_k, 128)`` the stride-16 compressed keys; v
+    ``(sum Lc, nheads_k, 128)`` the key set the log-sum-exp is taken over (the stride-64 compressed keys, or
+    ``k`` itself for an exact softmax); ``cu_seqlens_{q,k,v}`` int32.  Returns bf16
+    ``(nheads_k, total_q, max_seqlen_k)``: for every token and KV head the sum over the 16 grouped heads of
+    ``exp(scale*q.k_j - lse)`` on the keys the token may see, 0 elsewhere.
+    """
+    from .stage1 import stage1_scores
+    if softmax_scale is None:
+        softmax_scale = q.shape[-1] ** (-0.5)
+    _reject_unsupported(dropout_p, window_size, softcap, alibi_slopes, causal)
+    if block_table is not None:
+        raise RuntimeError("paged KV (block_table) is not supported by this build")
+    q, k, v = [_dense_last_dim(x) for x in (q, k, v)]
+    _check_qkv(q, k, v, cu_seqlens_q, cu_seqlens_k)
+    if cu_seqlens_v.dtype != torch.int32:
+        raise RuntimeError("cu_seqlens_v must have dtype int32")
+    return stage1_scores(q, k, v, cu_seqlens_q, cu_seqlens_k, cu_seqlens_v, max_seqlen_q, max_seqlen_k,
+                         softmax_scale, causal)
+
+
+def infllmv2_attn_with_kvcache(q, k_cache, v_cache, k=None, v=None, rotary_cos=None, rotary_sin=None,
+                               cache_seqlens: Optional[Union[int, torch.Tensor]] = None,
+                               cache_batch_idx: Optional[torch.Tensor] = None,
+                               cache_leftpad: Optional[torch.Tensor] = None,
+                               block_table: Optional[torch.Tensor] = None, softmax_scale=None, causal=False,
+                               window_size=(-1, -1), softcap=0.0, rotary_interleaved=True, alibi_slopes=None,
+                               num_splits=0, return_softmax_lse=False, topk_idx=None):
+    """Decode step against a KV cache, restricted to the blocks in ``topk_idx``.
+
+    q ``(batch, 1, nheads, 128)``; caches ``(batch, capacity, nheads_k, 128)``; ``cache_seqlens`` int or int32
+    ``(batch,)``.  If ``k``/``v`` ``(batch, s_new, nheads_k, 128)`` are given they are written into the caches
+    at ``cache_seqlens`` first (in place) and take part in the attention.  ``topk_idx`` int32
+    ``(batch, nheads_k, 1, k)`` selects 64-key blocks of the cache (mask width from the cache capacity).
+    Returns ``out (batch, 1, nheads, 128)`` or ``(out, softmax_lse (batch, nheads, 1))``.  No backward.
+    Rotary embedding, paged KV, ``cache_batch_idx`` and ``cache_leftpad`` are not supported.
+    """
+    from .decode import decode_with_kvcache
+    assert k_cache.stride(-1) == 1, "k_cache must have contiguous last dimension"
+    assert v_cache.stride(-1) == 1, "v_cache must have contiguous last dimension"
+    if softmax_scale is None:
+        softmax_scale = q.shape[-1] ** (-0.5)
+    _reject_unsupported(0.0, window_size, softcap, alibi_slopes, causal)
+    for name, val in (("rotary_cos", rotary_cos), ("rotary_sin", rotary_sin), ("cache_batch_idx", cache_batch_idx),
+                      ("cache_leftpad", cache_leftpad), ("block_table", block_table)):
+        if val is not None:
+            raise RuntimeError(f"{name} is not supported by this build")
+    q, k, v = [_dense_last_dim(x) for x in (q, k, v)]
+    if cache_seqlens is not None and isinstance(cache_seqlens, int):
+        cache_seqlens = torch.full((k_cache.shape[0],), cache_seqlens, dtype=torch.int32, device=k_cache.device)
+    mask = None
+    if topk_idx is not None:
+        assert topk_idx.dtype == torch.int32
+        mask, _ = topk_to_uint64(topk_idx, k_cache.shape[1], BLOCK_N)
+    out, lse = decode_with_kvcache(q, k_cache, v_cache, k, v, cache_seqlens, softmax_scale, causal, num_splits, mask)
+    return (out, lse) if return_softmax_lse else out

@@ -1,0 +1,358 @@
+// Stage-2 block-sparse flash-attention forward for gfx950 (bf16, head_dim 128, 16 query heads
+// per KV head).
+//
+// Semantics follow compute_attn_1rowblock (csrc/flash_attn/src/flash_fwd_kernel.h:137-602) with
+// the bitmask walk of flash_blockmask.h:5-100: token i of a sequence attends key t iff
+// t <= i + Sk - Sq (causal, bottom-right aligned), t < Sk, and bit t/64 of its mask row is set;
+// O = softmax(scale * q.K^T) V with fp32 softmax and P rounded to bf16 before P.V; rows with no
+// allowed key give O = 0 and LSE = +inf (softmax.h:240-256).
+//
+// Design (not the reference's): the 16 grouped heads of one token form the 16-column N side of
+// v_mfma_f32_16x16x32_bf16.  S^T = K.Q^T puts keys on the M side, so one lane owns one head's
+// scores for 16 keys and the same registers, converted to bf16, are the B operand of
+// O^T = V^T.P^T.  K and V come from fragment-major block images (kv_image.h) built by
+// pack_kv_kernel, so every operand fetch is one contiguous 1 KiB wavefront load.  Q, O and the
+// LSE are addressed through strides: the caller's (T, Hq, d) tensors are used in place.
+#include "common.h"
+#include "kv_image.h"
+#include "../../include/infllmv2_hip.h"
+#include <math.h>
+
+namespace infllmv2 {
+
+// ---------------------------------------------------------------------------------------------
+// K/V -> block images
+// ---------------------------------------------------------------------------------------------
+struct PackParams {
+    const bf16_bits* k;
+    const bf16_bits* v;
+    bf16_bits* kimg;
+    bf16_bits* vimg;
+    const int* cu_seqlens_k;        // cumulative (batch + 1) or, for a cache, null
+    const int* seqlens_k;           // per-sequence lengths when cu_seqlens_k is null
+    int64_t k_batch_stride, k_row_stride, k_head_stride;
+    int64_t v_batch_stride, v_row_stride, v_head_stride;
+    int64_t n_slots;
+    int slots_per_batch;            // used when cu_seqlens_k is null
+};
+
+constexpr int kVPad = 8;            // LDS row padding (elements) for the V transposition
+
+__global__ __launch_bounds__(256)
+void pack_kv_kernel(const PackParams p) {
+    __shared__ __attribute__((aligned(16))) bf16_bits vt[kBlockN][kHeadDim + kVPad];
+    const int j = blockIdx.x, b = blockIdx.y, h = blockIdx.z;
+    int64_t row0, slot;
+    int Sk;
+    if (p.cu_seqlens_k != nullptr) {
+        const int k0 = p.cu_seqlens_k[b];
+        Sk = p.cu_seqlens_k[b + 1] - k0;
+        row0 = k0;
+        slot = image_slot0(p.cu_seqlens_k, b) + j;
+    } else {
+        Sk = p.seqlens_k[b];
+        row0 = 0;
+        slot = static_cast<int64_t>(b) * p.slots_per_batch + j;
+    }
+    if (static_cast<int64_t>(j) * kBlockN >= Sk) return;
+    const int tid = threadIdx.x;
+    const bf16_bits* kb = p.k + b * p.k_batch_stride + (row0 + static_cast<int64_t>(j) * kBlockN) * p.k_row_stride + h * p.k_head_stride;
+    const bf16_bits* vb = p.v + b * p.v_batch_stride + (row0 + static_cast<int64_t>(j) * kBlockN) * p.v_row_stride + h * p.v_head_stride;
+    bf16_bits* kdst = p.kimg + (static_cast<int64_t>(h) * p.n_slots + slot) * kImageElems;
+    bf16_bits* vdst = p.vimg + (static_cast<int64_t>(h) * p.n_slots + slot) * kImageElems;
+    const int valid = Sk - j * kBlockN;                       // keys of this block inside the sequence
+    const uint4 zero = make_uint4(0, 0, 0, 0);
+
+    for (int u = tid; u < 1024; u += 256) {
+        const int kt = u >> 8, c = (u >> 6) & 3, lane = u & 63;
+        const int r = lane & 15, g = lane >> 4;
+        const int key = 16 * kt + r;
+        uint4 val = zero;
+        if (key < valid) val = *reinterpret_cast<const uint4*>(kb + key * p.k_row_stride + 32 * c + 8 * g);
+        *reinterpret_cast<uint4*>(kdst + u * 8) = val;
+    }
+    for (int u = tid; u < 1024; u += 256) {
+        const int key = u >> 4, d0 = (u & 15) * 8;
+        uint4 val = zero;
+        if (key < valid) val = *reinterpret_cast<const uint4*>(vb + key * p.v_row_stride + d0);
+        *reinterpret_cast<uint4*>(&vt[key][d0]) = val;
+    }
+    __syncthreads();
+    for (int u = tid; u < 1024; u += 256) {
+        const int dt = u >> 7, cc = (u >> 6) & 1, lane = u & 63;
+        const int r = lane & 15, g = lane >> 4;
+        const int d = 16 * dt + r;
+        uint32_t w[4];
+#pragma unroll
+        for (int jj = 0; jj < 8; jj += 2) {
+            const int key_a = 32 * cc + (jj < 4 ? 4 * g + jj : 16 + 4 * g + jj - 4);
+            w[jj >> 1] = static_cast<uint32_t>(vt[key_a][d]) | (static_cast<uint32_t>(vt[key_a + 1][d]) << 16);
+        }
+        *reinterpret_cast<uint4*>(vdst + u * 8) = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// forward
+// ---------------------------------------------------------------------------------------------
+struct FwdParams {
+    const bf16_bits* q;
+    bf16_bits* out;
+    float* lse;
+    const bf16_bits* kimg;
+    const bf16_bits* vimg;
+    const int* cu_seqlens_q;
+    const int* cu_seqlens_k;
+    const uint64_t* mask;           // (Hk, total_q, n64) or null for dense
+    int64_t q_tok_stride, q_grp_stride, q_kvh_stride;
+    int64_t o_tok_stride, o_grp_stride, o_kvh_stride;
+    int64_t lse_tok_stride, lse_grp_stride, lse_kvh_stride;
+    int64_t n_slots;
+    int64_t total_q;
+    int n64;
+    float scale_log2;               // softmax_scale * log2(e)
+};
+
+// Walks the set bits of one mask row in ascending block order, clipped to [0, last_blk].
+struct BlockWalker {
+    const uint64_t* row;
+    int n_words;                    // words that can hold an allowed block
+    int last_blk;
+    int w;
+    uint64_t bits;
+
+    __device__ __forceinline__ uint64_t load_word(int word) const {
+        uint64_t v = row ? row[word] : ~0ull;
+        if (word == (last_blk >> 6)) {
+            const int t = last_blk & 63;
+            v &= (t == 63) ? ~0ull : ((1ull << (t + 1)) - 1ull);
+        }
+        // the row is shared by the whole wavefront: keep the loop control in scalar registers
+        const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
+        const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
+        return (static_cast<uint64_t>(hi) << 32) | lo;
+    }
+    __device__ __forceinline__ void init(const uint64_t* r, int words_in_row, int last) {
+        row = r;
+        last_blk = last;
+        n_words = last < 0 ? 0 : (last >> 6) + 1;
+        if (row && n_words > words_in_row) n_words = words_in_row;
+        w = 0;
+        bits = n_words > 0 ? load_word(0) : 0ull;
+    }
+    __device__ __forceinline__ int next() {
+        while (bits == 0ull) {
+            if (++w >= n_words) return -1;
+            bits = load_word(w);
+        }
+        const int bit = __builtin_ctzll(bits);
+        bits &= bits - 1ull;
+        return w * 64 + bit;
+    }
+};
+
+__device__ __forceinline__ float wave_max_over_g(float x) {
+    x = fmaxf(x, __shfl_xor(x, 16));
+    return fmaxf(x, __shfl_xor(x, 32));
+}
+__device__ __forceinline__ float wave_sum_over_g(float x) {
+    x += __shfl_xor(x, 16);
+    return x + __shfl_xor(x, 32);
+}
+
+template <bool kCausal>
+__global__ __launch_bounds__(256)
+void stage2_fwd_kernel(const FwdParams p) {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int b = blockIdx.y, h = blockIdx.z;
+    const int i = blockIdx.x * 4 + wave;                        // token inside the sequence
+    const int q0 = p.cu_seqlens_q[b];
+    const int Sq = p.cu_seqlens_q[b + 1] - q0;
+    if (i >= Sq) return;                                        // uniform per wavefront; no barriers in this kernel
+    const int k0 = p.cu_seqlens_k[b];
+    const int Sk = p.cu_seqlens_k[b + 1] - k0;
+    const int64_t tok = static_cast<int64_t>(q0) + i;
+    const int n = lane & 15, g = lane >> 4;
+
+    const bf16_bits* qp = p.q + tok * p.q_tok_stride + h * p.q_kvh_stride + n * p.q_grp_stride + 8 * g;
+    bf16x8 qf[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) qf[c] = *reinterpret_cast<const bf16x8*>(qp + 32 * c);
+
+    int last_key = kCausal ? (i + Sk - Sq) : (Sk - 1);          // largest allowed key index
+    if (last_key > Sk - 1) last_key = Sk - 1;
+    const int last_blk = last_key < 0 ? -1 : (last_key >> 6);
+
+    BlockWalker walk;
+    walk.init(p.mask ? p.mask + (static_cast<int64_t>(h) * p.total_q + tok) * p.n64 : nullptr, p.n64, last_blk);
+
+    const int64_t img0 = (static_cast<int64_t>(h) * p.n_slots + image_slot0(p.cu_seqlens_k, b)) * kImageElems;
+    const bf16_bits* kimg = p.kimg + img0 + lane * 8;
+    const bf16_bits* vimg = p.vimg + img0 + lane * 8;
+
+    float m = -INFINITY, l = 0.f;
+    floatx4 o[8];
+#pragma unroll
+    for (int dt = 0; dt < 8; ++dt) o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    bf16x8 kreg[16], vreg[16];
+    int j = walk.next();
+    if (j >= 0) {
+        const bf16_bits* src = kimg + static_cast<int64_t>(j) * kImageElems;
+#pragma unroll
+        for (int f = 0; f < 16; ++f) kreg[f] = *reinterpret_cast<const bf16x8*>(src + f * 512);
+    }
+    while (j >= 0) {
+        {
+            const bf16_bits* src = vimg + static_cast<int64_t>(j) * kImageElems;
+#pragma unroll
+            for (int f = 0; f < 16; ++f) vreg[f] = *reinterpret_cast<const bf16x8*>(src + f * 512);
+        }
+        floatx4 s[4];
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt) {
+            s[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+                s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[kt * 4 + c], qf[c], s[kt], 0, 0, 0);
+        }
+        const int jn = walk.next();
+        if (jn >= 0) {
+            const bf16_bits* src = kimg + static_cast<int64_t>(jn) * kImageElems;
+#pragma unroll
+            for (int f = 0; f < 16; ++f) kreg[f] = *reinterpret_cast<const bf16x8*>(src + f * 512);
+        }
+        if (j == last_blk) {                                    // only the last allowed block needs element masking
+            const int lim = last_key - j * kBlockN;              // keys with in-block index > lim are masked
+#pragma unroll
+            for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (16 * kt + 4 * g + e > lim) s[kt][e] = -INFINITY;
+        }
+        float mx = -INFINITY;
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) mx = fmaxf(mx, s[kt][e]);
+        mx = wave_max_over_g(mx);
+        const float m_new = fmaxf(m, mx * p.scale_log2);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f(m - m_use);
+        float rs = 0.f;
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float pv = __builtin_amdgcn_exp2f(s[kt][e] * p.scale_log2 - m_use);
+                s[kt][e] = pv;
+                rs += pv;
+            }
+        l = l * alpha + rs;
+        m = m_new;
+#pragma unroll
+        for (int dt = 0; dt < 8; ++dt) o[dt] *= alpha;
+        bf16x8 pf[2];
+#pragma unroll
+        for (int cc = 0; cc < 2; ++cc)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                pf[cc][e] = static_cast<__bf16>(s[2 * cc][e]);
+                pf[cc][4 + e] = static_cast<__bf16>(s[2 * cc + 1][e]);
+            }
+#pragma unroll
+        for (int dt = 0; dt < 8; ++dt)
+#pragma unroll
+            for (int cc = 0; cc < 2; ++cc)
+                o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg[dt * 2 + cc], pf[cc], o[dt], 0, 0, 0);
+        j = jn;
+    }
+
+    const float l_tot = wave_sum_over_g(l);
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    bf16_bits* op = p.out + tok * p.o_tok_stride + h * p.o_kvh_stride + n * p.o_grp_stride + 4 * g;
+#pragma unroll
+    for (int dt = 0; dt < 8; ++dt) {
+        uint2 w;
+        w.x = pack_bf16x2(o[dt][0] * inv, o[dt][1] * inv);
+        w.y = pack_bf16x2(o[dt][2] * inv, o[dt][3] * inv);
+        *reinterpret_cast<uint2*>(op + 16 * dt) = w;
+    }
+    if (g == 0) {
+        const float lse = l_tot > 0.f ? m * 0.69314718055994530942f + logf(l_tot) : INFINITY;
+        p.lse[h * p.lse_kvh_stride + tok * p.lse_tok_stride + n * p.lse_grp_stride] = lse;
+    }
+}
+
+}  // namespace infllmv2
+
+using namespace infllmv2;
+
+extern "C" size_t infllmv2_kv_image_bytes(int64_t total_k, int batch, int num_heads_k) {
+    return static_cast<size_t>(image_slots(total_k, batch)) * num_heads_k * kImageElems * sizeof(bf16_bits) * 2;
+}
+
+extern "C" int infllmv2_varlen_fwd(void* stream, const void* q, const void* k, const void* v, void* out,
+                                   float* softmax_lse, const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                                   const uint64_t* blockmask, void* workspace, size_t workspace_bytes,
+                                   int batch, int64_t total_q, int64_t total_k, int num_heads, int num_heads_k,
+                                   int head_dim, int max_seqlen_q, int max_seqlen_k,
+                                   const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                                   const int64_t* o_strides, const int64_t* lse_strides,
+                                   int n_uint64_per_row, float softmax_scale, int is_causal) {
+    IV2_CHECK(head_dim == kHeadDim, "varlen_fwd: this build only supports head_dim 128 (got %d)", head_dim);
+    IV2_CHECK(num_heads_k > 0 && num_heads == num_heads_k * kGroup,
+              "varlen_fwd: requires num_heads == 16 * num_heads_k (got %d and %d)", num_heads, num_heads_k);
+    IV2_CHECK(batch > 0 && total_q >= 0 && total_k >= 0 && max_seqlen_q >= 0 && max_seqlen_k >= 0, "varlen_fwd: bad sizes");
+    IV2_CHECK(q && k && v && out && softmax_lse && cu_seqlens_q && cu_seqlens_k, "varlen_fwd: null pointer");
+    IV2_CHECK(num_heads_k <= 65535 && batch <= 65535, "varlen_fwd: batch and num_heads_k must not exceed 65535");
+    IV2_CHECK(workspace_bytes >= infllmv2_kv_image_bytes(total_k, batch, num_heads_k), "varlen_fwd: workspace too small");
+    IV2_CHECK(reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(k) % 16 == 0 &&
+              reinterpret_cast<uintptr_t>(v) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 8 == 0 &&
+              reinterpret_cast<uintptr_t>(workspace) % 16 == 0, "varlen_fwd: q, k, v and workspace must be 16-byte aligned");
+    for (int s = 0; s < 3; ++s) {
+        IV2_CHECK(q_strides[s] % 8 == 0 && o_strides[s] % 4 == 0, "varlen_fwd: q strides must be multiples of 8 and out strides of 4 elements");
+    }
+    IV2_CHECK(k_strides[0] % 8 == 0 && k_strides[1] % 8 == 0 && v_strides[0] % 8 == 0 && v_strides[1] % 8 == 0,
+              "varlen_fwd: k/v row and head strides must be multiples of 8 elements");
+    IV2_CHECK(blockmask == nullptr || n_uint64_per_row > 0, "varlen_fwd: mask given without words per row");
+    if (total_q == 0 || max_seqlen_q == 0) return 0;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+
+    const int64_t n_slots = image_slots(total_k, batch);
+    bf16_bits* kimg = static_cast<bf16_bits*>(workspace);
+    bf16_bits* vimg = kimg + n_slots * num_heads_k * kImageElems;
+    const int max_blocks = (max_seqlen_k + kBlockN - 1) / kBlockN;
+    if (max_blocks > 0 && total_k > 0) {
+        PackParams pp{};
+        pp.k = static_cast<const bf16_bits*>(k);
+        pp.v = static_cast<const bf16_bits*>(v);
+        pp.kimg = kimg; pp.vimg = vimg;
+        pp.cu_seqlens_k = cu_seqlens_k;
+        pp.k_row_stride = k_strides[0]; pp.k_head_stride = k_strides[1];
+        pp.v_row_stride = v_strides[0]; pp.v_head_stride = v_strides[1];
+        pp.n_slots = n_slots;
+        hipLaunchKernelGGL(pack_kv_kernel, dim3(max_blocks, batch, num_heads_k), dim3(256), 0, st, pp);
+        IV2_LAUNCH_CHECK();
+    }
+    FwdParams fp{};
+    fp.q = static_cast<const bf16_bits*>(q);
+    fp.out = static_cast<bf16_bits*>(out);
+    fp.lse = softmax_lse;
+    fp.kimg = kimg; fp.vimg = vimg;
+    fp.cu_seqlens_q = cu_seqlens_q; fp.cu_seqlens_k = cu_seqlens_k;
+    fp.mask = blockmask;
+    fp.q_tok_stride = q_strides[0]; fp.q_grp_stride = q_strides[1]; fp.q_kvh_stride = q_strides[2];
+    fp.o_tok_stride = o_strides[0]; fp.o_grp_stride = o_strides[1]; fp.o_kvh_stride = o_strides[2];
+    fp.lse_tok_stride = lse_strides[0]; fp.lse_grp_stride = lse_strides[1]; fp.lse_kvh_stride = lse_strides[2];
+    fp.n_slots = n_slots;
+    fp.total_q = total_q;
+    fp.n64 = n_uint64_per_row;
+    fp.scale_log2 = softmax_scale * 1.44269504088896340736f;
+    const dim3 grid((max_seqlen_q + 3) / 4, batch, num_heads_k);
+    if (is_causal) hipLaunchKernelGGL(stage2_fwd_kernel<true>, grid, dim3(256), 0, st, fp);
+    else hipLaunchKernelGGL(stage2_fwd_kernel<false>, grid, dim3(256), 0, st, fp);
+    IV2_LAUNCH_CHECK();
+    return 0;
+}
