@@ -107,6 +107,23 @@ int infllmv2_topk(void* stream, int num_tokens, int dim, int top, int dtype, con
 int infllmv2_topk_blocks(void* stream, const void* pooled, int64_t row_stride, int32_t* topk_idx,
                          int64_t rows, int n, int k);
 
+/* ---- Stage 1: scoring over compressed keys --------------------------------------------------- */
+
+/* csrc/entry.cu:15,211 `varlen_fwd_stage1` = mha_varlen_fwd_stage1
+ * (csrc/flash_attn/flash_api.cpp:784-1049; kernel flash_fwd_kernel.h:1203-1744).
+ * q (total_q, Hq, 128) with strides {token, head-in-group, kv-head}; k = fine compressed keys
+ * (sum Lk, Hk, 128), v = the key set of the log-sum-exp (sum Lc, Hk, 128), strides {row, head};
+ * cu_seqlens_{q,k,v} are cumulative token / Lk / Lc counts.  score (Hk, total_q, row) bf16 with the
+ * given head/row strides (row stride >= max_seqlen_k): every column < max_seqlen_k of every row is
+ * written (0 where the reference leaves its zero fill or produces NaN that its wrapper zeroes). */
+int infllmv2_varlen_fwd_stage1(void* stream, const void* q, const void* k, const void* v, void* score,
+                               const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                               const int32_t* cu_seqlens_v, int batch, int64_t total_q, int num_heads,
+                               int num_heads_k, int head_dim, int max_seqlen_q, int max_seqlen_k,
+                               const int64_t* q_strides, const int64_t* k_strides,
+                               const int64_t* v_strides, int64_t score_head_stride,
+                               int64_t score_row_stride, float softmax_scale, int is_causal);
+
 /* ---- Stage 2: block-sparse attention -------------------------------------------------------- */
 
 /* Scratch needed by infllmv2_varlen_fwd / _bwd for the fragment-major K/V block images. */

@@ -28,6 +28,7 @@ SIGNATURES = {
     "infllmv2_max_pooling_1d_varlen_strided": [_p, _p, _p, _p, _p, _p] + [_i] * 6 + [_i64, _i64] + [_i] * 7,
     "infllmv2_topk": [_p, _i, _i, _i, _i, _p, _p, _p],
     "infllmv2_topk_blocks": [_p, _p, _i64, _p, _i64, _i, _i],
+    "infllmv2_varlen_fwd_stage1": [_p, _p, _p, _p, _p, _p, _p, _p, _i, _i64, _i, _i, _i, _i, _i, _p, _p, _p, _i64, _i64, _f, _i],
     "infllmv2_varlen_fwd": [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _sz, _i, _i64, _i64, _i, _i, _i, _i, _i,
                             _p, _p, _p, _p, _p, _i, _f, _i],
 }
@@ -45,7 +46,7 @@ def exported_names():
 def _load():
     if not os.path.exists(LIB_PATH):
         raise ImportError(
-            f"{LIB_PATH} is missing: build it with `python -m infllmv2_cuda_impl_amd.build` "
+            f"{LIB_PATH} is missing: build it with `python infllmv2_cuda_impl_amd/csrc/build.py` "
             "(hipcc, --offload-arch=gfx950). There is no fallback path.")
     lib = C.CDLL(LIB_PATH)
     for name, argtypes in SIGNATURES.items():

@@ -1,6 +1,7 @@
 """Builds libinfllmv2_hip.so (gfx950 code objects + C ABI) in-tree with hipcc.
 
-Run as ``python -m infllmv2_cuda_impl_amd.build``.  There is exactly one target architecture.
+Run as ``python infllmv2_cuda_impl_amd/csrc/build.py`` (a plain script: it must work when no
+library exists yet, so it does not import the package).  There is exactly one target architecture.
 """
 from __future__ import annotations
 
@@ -9,10 +10,10 @@ import subprocess
 import sys
 from concurrent.futures import ThreadPoolExecutor
 
-HERE = os.path.dirname(os.path.abspath(__file__))
-CSRC = os.path.join(HERE, "csrc")
-LIB_PATH = os.path.join(HERE, "libinfllmv2_hip.so")
-OBJ_DIR = os.path.join(HERE, "build")
+CSRC = os.path.dirname(os.path.abspath(__file__))
+PKG = os.path.dirname(CSRC)
+LIB_PATH = os.path.join(PKG, "libinfllmv2_hip.so")
+OBJ_DIR = os.path.join(PKG, "build")
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffast-math", "-fno-finite-math-only",

@@ -1,0 +1,304 @@
+// Stage-1 scoring for gfx950: softmax-like scores of the 16 grouped query heads against the
+// compressed keys, normalised by a log-sum-exp taken over a (usually coarser) second key set,
+// summed over the 16 heads.
+//
+// Semantics follow compute_attn_1rowblock_splitkv_stage1
+// (csrc/flash_attn/src/flash_fwd_kernel.h:1203-1744), Mask::apply_mask_stage1
+// (csrc/flash_attn/src/mask.h:225-319), softmax_rescale_simple / softmax_rescale_gt
+// (csrc/flash_attn/src/softmax.h:94-121,198-237) and hdim16_reduce (flash_fwd_kernel.h:53-112):
+//   vis_s(i) = min(L, max(0, (i+1)/s - 1 + L - (Sq - s + 1)/s))     (C++ truncating divisions)
+//   lse_g(i) = log sum_{c < vis_c(i)} exp(scale * q_g . kc_c),  s = 64, or 16 when Lc == Lk
+//   score[h, i, j] = bf16( sum_g exp(scale * q_g . kf_j - lse_g(i)) )   for j < vis_16(i), else 0
+//   rows with vis_c(i) == 0 are all zero (the reference's early exit leaves its zero fill).
+//
+// Design: S = Q.K^T with the 16 heads of one token as the 16 MFMA rows and 16 compressed keys as
+// the columns, so a lane owns four heads of one key column; the per-head running max/sum of
+// pass 1 stay lane-local until one 16-lane butterfly at the end, and the sum over the 16 heads
+// in pass 2 is an in-lane add of four values plus two cross-lane adds.  A workgroup is 4
+// wavefronts x 4 consecutive tokens; each 64-key tile of compressed keys is staged once in LDS
+// in MFMA-operand order (conflict-free ds_read_b128) and reused by all 16 tokens, and inside a
+// wavefront one operand read feeds four MFMAs.
+#include "common.h"
+#include "../../include/infllmv2_hip.h"
+#include <math.h>
+
+namespace infllmv2 {
+
+struct Stage1Params {
+    const bf16_bits* q;
+    const bf16_bits* k;              // fine compressed keys   (sum Lk, Hk, d)
+    const bf16_bits* c;              // coarse compressed keys (sum Lc, Hk, d)
+    bf16_bits* score;                // (Hk, total_q, row_stride)
+    const int* cu_seqlens_q;
+    const int* cu_seqlens_k;
+    const int* cu_seqlens_c;
+    int64_t q_tok_stride, q_grp_stride, q_kvh_stride;
+    int64_t k_row_stride, k_head_stride, c_row_stride, c_head_stride;
+    int64_t score_head_stride, score_row_stride;
+    int score_cols;                  // columns to define in every row (max_seqlen_k)
+    float scale_log2;
+    int causal;
+};
+
+constexpr int kTokPerWave = 4;
+constexpr int kWavesS1 = 4;
+constexpr int kTokPerBlock = kTokPerWave * kWavesS1;   // 16
+
+__device__ __forceinline__ int trunc_div(int a, int b) { return a / b; }   // C++ semantics on purpose
+
+__device__ __forceinline__ int stage1_visible(int i, int s, int L, int Sq, bool causal) {
+    if (!causal) return L;
+    const int cq = trunc_div(Sq - s + 1, s);
+    int v = (i + 1) / s - 1 + L - cq;
+    v = v < 0 ? 0 : v;
+    return v < L ? v : L;
+}
+
+// global (64 keys x 128 d) tile -> registers; thread t of 256 owns 16-byte units t, t+256, ...
+__device__ __forceinline__ void load_tile_regs(uint4 (&r)[4], const bf16_bits* base, int64_t row_stride,
+                                               int key0, int L, int tid) {
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+        const int u = tid + it * 256;
+        const int key = u >> 4, chunk = u & 15;
+        r[it] = make_uint4(0, 0, 0, 0);
+        if (key0 + key < L) r[it] = *reinterpret_cast<const uint4*>(base + (key0 + key) * row_stride + chunk * 8);
+    }
+}
+
+// registers -> LDS in operand order: unit ((kt*4 + c)*64 + 16*g + n) holds K[16*kt + n][32*c + 8*g ..]
+__device__ __forceinline__ void store_tile_lds(const uint4 (&r)[4], uint4* lds, int tid) {
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+        const int u = tid + it * 256;
+        const int key = u >> 4, chunk = u & 15;
+        const int kt = key >> 4, n = key & 15, c = chunk >> 2, g = chunk & 3;
+        lds[(kt * 4 + c) * 64 + 16 * g + n] = r[it];
+    }
+}
+
+template <bool kCausal>
+__global__ __launch_bounds__(256)
+void stage1_kernel(const Stage1Params p) {
+    __shared__ uint4 tile[2][1024];                            // two 16 KiB operand-ordered key tiles
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int n = lane & 15, g = lane >> 4;
+    const int b = blockIdx.y, h = blockIdx.z;
+    const int q0 = p.cu_seqlens_q[b];
+    const int Sq = p.cu_seqlens_q[b + 1] - q0;
+    const int tok_block0 = blockIdx.x * kTokPerBlock;
+    if (tok_block0 >= Sq) return;                              // uniform per workgroup
+    const int k0 = p.cu_seqlens_k[b], Lk = p.cu_seqlens_k[b + 1] - k0;
+    const int c0 = p.cu_seqlens_c[b], Lc = p.cu_seqlens_c[b + 1] - c0;
+    const int s1 = (Lk == Lc) ? 16 : 64;                       // flash_fwd_kernel.h:1236-1240
+
+    const int tok0 = tok_block0 + wave * kTokPerWave;          // first token of this wavefront
+    int vis_f[kTokPerWave], vis_c[kTokPerWave];
+    bool live[kTokPerWave];
+#pragma unroll
+    for (int t = 0; t < kTokPerWave; ++t) {
+        const int i = tok0 + t;
+        live[t] = i < Sq;
+        vis_f[t] = live[t] ? stage1_visible(i, 16, Lk, Sq, kCausal) : 0;
+        vis_c[t] = live[t] ? stage1_visible(i, s1, Lc, Sq, kCausal) : 0;
+        if (vis_c[t] == 0) vis_f[t] = 0;                       // early exit of flash_fwd_kernel.h:1271-1276
+    }
+    // tile counts are taken over the whole workgroup (its last live token sees the most keys)
+    const int i_last = (tok_block0 + kTokPerBlock - 1 < Sq ? tok_block0 + kTokPerBlock - 1 : Sq - 1);
+    const int wg_vis_c = stage1_visible(i_last, s1, Lc, Sq, kCausal);
+    const int wg_vis_f = wg_vis_c == 0 ? 0 : stage1_visible(i_last, 16, Lk, Sq, kCausal);
+    const int tiles_c = (wg_vis_c + 63) >> 6;
+    const int tiles_f = (wg_vis_f + 63) >> 6;
+
+    // Q as the A operand: lane (row = head n... here r = lane % 16 is the head, g the k-group)
+    bf16x8 qf[kTokPerWave][4];
+#pragma unroll
+    for (int t = 0; t < kTokPerWave; ++t) {
+        const int i = live[t] ? tok0 + t : Sq - 1;
+        const bf16_bits* qp = p.q + (static_cast<int64_t>(q0) + i) * p.q_tok_stride + h * p.q_kvh_stride + n * p.q_grp_stride + 8 * g;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) qf[t][c] = *reinterpret_cast<const bf16x8*>(qp + 32 * c);
+    }
+
+    // ---------------- pass 1: per-head log-sum-exp over the coarse keys ----------------
+    float m[kTokPerWave][4], l[kTokPerWave][4];                // lane-local over keys == n (mod 16); head 4g+e
+#pragma unroll
+    for (int t = 0; t < kTokPerWave; ++t)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { m[t][e] = -INFINITY; l[t][e] = 0.f; }
+
+    const bf16_bits* cbase = p.c + static_cast<int64_t>(c0) * p.c_row_stride + h * p.c_head_stride;
+    const bf16_bits* kbase = p.k + static_cast<int64_t>(k0) * p.k_row_stride + h * p.k_head_stride;
+    uint4 stage[4];
+    if (tiles_c > 0) {
+        load_tile_regs(stage, cbase, p.c_row_stride, 0, Lc, tid);
+        store_tile_lds(stage, tile[0], tid);
+    }
+    __syncthreads();
+    for (int ti = 0; ti < tiles_c; ++ti) {
+        const bool more = ti + 1 < tiles_c;
+        if (more) load_tile_regs(stage, cbase, p.c_row_stride, (ti + 1) * 64, Lc, tid);
+        const uint4* cur = tile[ti & 1];
+        floatx4 s[kTokPerWave][4];
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt) {
+#pragma unroll
+            for (int t = 0; t < kTokPerWave; ++t) s[t][kt] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const uint4 raw = cur[(kt * 4 + c) * 64 + lane];
+                bf16x8 kf;
+                __builtin_memcpy(&kf, &raw, 16);
+#pragma unroll
+                for (int t = 0; t < kTokPerWave; ++t)
+                    s[t][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[t][c], kf, s[t][kt], 0, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < kTokPerWave; ++t) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float v[4];
+                float mx = -INFINITY;
+#pragma unroll
+                for (int kt = 0; kt < 4; ++kt) {
+                    const int j = ti * 64 + kt * 16 + n;
+                    v[kt] = (j < vis_c[t]) ? s[t][kt][e] * p.scale_log2 : -INFINITY;
+                    mx = fmaxf(mx, v[kt]);
+                }
+                const float m_new = fmaxf(m[t][e], mx);
+                const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+                float acc = l[t][e] * __builtin_amdgcn_exp2f(m[t][e] - m_use);
+#pragma unroll
+                for (int kt = 0; kt < 4; ++kt) acc += __builtin_amdgcn_exp2f(v[kt] - m_use);
+                l[t][e] = acc;
+                m[t][e] = m_new;
+            }
+        }
+        if (more) store_tile_lds(stage, tile[(ti + 1) & 1], tid);
+        __syncthreads();
+    }
+    // merge the 16 key-column lanes of each head: lse2 = m + log2(l) in log2 units
+    float lse2[kTokPerWave][4];
+#pragma unroll
+    for (int t = 0; t < kTokPerWave; ++t)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            float mm = m[t][e], ll = l[t][e];
+#pragma unroll
+            for (int off = 1; off < 16; off <<= 1) {
+                const float mo = __shfl_xor(mm, off);
+                const float lo = __shfl_xor(ll, off);
+                const float mn = fmaxf(mm, mo);
+                const float mu = (mn == -INFINITY) ? 0.f : mn;
+                ll = ll * __builtin_amdgcn_exp2f(mm - mu) + lo * __builtin_amdgcn_exp2f(mo - mu);
+                mm = mn;
+            }
+            lse2[t][e] = mm + __builtin_amdgcn_logf(ll);        // v_log_f32 is log2
+        }
+
+    // ---------------- pass 2: scores over the fine keys ----------------
+    if (tiles_f > 0) {
+        load_tile_regs(stage, kbase, p.k_row_stride, 0, Lk, tid);
+        store_tile_lds(stage, tile[0], tid);
+    }
+    __syncthreads();
+    bf16_bits* out_rows[kTokPerWave];
+#pragma unroll
+    for (int t = 0; t < kTokPerWave; ++t)
+        out_rows[t] = p.score + h * p.score_head_stride + (static_cast<int64_t>(q0) + tok0 + t) * p.score_row_stride;
+
+    for (int ti = 0; ti < tiles_f; ++ti) {
+        const bool more = ti + 1 < tiles_f;
+        if (more) load_tile_regs(stage, kbase, p.k_row_stride, (ti + 1) * 64, Lk, tid);
+        const uint4* cur = tile[ti & 1];
+        float mine[kTokPerWave];                               // the score this lane will store: key 16*g + n
+#pragma unroll
+        for (int t = 0; t < kTokPerWave; ++t) mine[t] = 0.f;
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt) {
+            floatx4 s[kTokPerWave];
+#pragma unroll
+            for (int t = 0; t < kTokPerWave; ++t) s[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const uint4 raw = cur[(kt * 4 + c) * 64 + lane];
+                bf16x8 kf;
+                __builtin_memcpy(&kf, &raw, 16);
+#pragma unroll
+                for (int t = 0; t < kTokPerWave; ++t)
+                    s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[t][c], kf, s[t], 0, 0, 0);
+            }
+            const int j = ti * 64 + kt * 16 + n;
+#pragma unroll
+            for (int t = 0; t < kTokPerWave; ++t) {
+                float sum = 0.f;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) sum += __builtin_amdgcn_exp2f(s[t][e] * p.scale_log2 - lse2[t][e]);
+                sum = (j < vis_f[t]) ? sum : 0.f;
+                sum += __shfl_xor(sum, 16);
+                sum += __shfl_xor(sum, 32);                    // all four g-groups now hold the 16-head sum
+                if (g == kt) mine[t] = sum;
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < kTokPerWave; ++t) {
+            const int col = ti * 64 + lane;                    // lane = 16*g + n  <->  key 16*g + n of this tile
+            if (live[t] && col < p.score_cols) out_rows[t][col] = f32_to_bf16(mine[t]);
+        }
+        if (more) store_tile_lds(stage, tile[(ti + 1) & 1], tid);
+        __syncthreads();
+    }
+    // columns no tile covered are zero
+#pragma unroll
+    for (int t = 0; t < kTokPerWave; ++t) {
+        if (!live[t]) continue;
+        for (int col = tiles_f * 64 + lane; col < p.score_cols; col += 64) out_rows[t][col] = 0;
+    }
+}
+
+}  // namespace infllmv2
+
+using namespace infllmv2;
+
+extern "C" int infllmv2_varlen_fwd_stage1(void* stream, const void* q, const void* k, const void* v, void* score,
+                                          const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                                          const int32_t* cu_seqlens_v, int batch, int64_t total_q, int num_heads,
+                                          int num_heads_k, int head_dim, int max_seqlen_q, int max_seqlen_k,
+                                          const int64_t* q_strides, const int64_t* k_strides,
+                                          const int64_t* v_strides, int64_t score_head_stride,
+                                          int64_t score_row_stride, float softmax_scale, int is_causal) {
+    IV2_CHECK(head_dim == kHeadDim, "varlen_fwd_stage1: this build only supports head_dim 128 (got %d)", head_dim);
+    IV2_CHECK(num_heads_k > 0 && num_heads == num_heads_k * kGroup,
+              "varlen_fwd_stage1: requires num_heads == 16 * num_heads_k (got %d and %d)", num_heads, num_heads_k);
+    IV2_CHECK(batch > 0 && total_q >= 0 && max_seqlen_q >= 0 && max_seqlen_k >= 0, "varlen_fwd_stage1: bad sizes");
+    IV2_CHECK(q && k && v && score && cu_seqlens_q && cu_seqlens_k && cu_seqlens_v, "varlen_fwd_stage1: null pointer");
+    IV2_CHECK(num_heads_k <= 65535 && batch <= 65535, "varlen_fwd_stage1: batch and num_heads_k must not exceed 65535");
+    IV2_CHECK(reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(k) % 16 == 0 &&
+              reinterpret_cast<uintptr_t>(v) % 16 == 0, "varlen_fwd_stage1: q, k, v must be 16-byte aligned");
+    for (int s = 0; s < 3; ++s) IV2_CHECK(q_strides[s] % 8 == 0, "varlen_fwd_stage1: q strides must be multiples of 8 elements");
+    IV2_CHECK(k_strides[0] % 8 == 0 && k_strides[1] % 8 == 0 && v_strides[0] % 8 == 0 && v_strides[1] % 8 == 0,
+              "varlen_fwd_stage1: k/v strides must be multiples of 8 elements");
+    IV2_CHECK(score_row_stride >= max_seqlen_k, "varlen_fwd_stage1: score row stride shorter than max_seqlen_k");
+    if (total_q == 0 || max_seqlen_q == 0) return 0;
+    Stage1Params p{};
+    p.q = static_cast<const bf16_bits*>(q);
+    p.k = static_cast<const bf16_bits*>(k);
+    p.c = static_cast<const bf16_bits*>(v);
+    p.score = static_cast<bf16_bits*>(score);
+    p.cu_seqlens_q = cu_seqlens_q; p.cu_seqlens_k = cu_seqlens_k; p.cu_seqlens_c = cu_seqlens_v;
+    p.q_tok_stride = q_strides[0]; p.q_grp_stride = q_strides[1]; p.q_kvh_stride = q_strides[2];
+    p.k_row_stride = k_strides[0]; p.k_head_stride = k_strides[1];
+    p.c_row_stride = v_strides[0]; p.c_head_stride = v_strides[1];
+    p.score_head_stride = score_head_stride; p.score_row_stride = score_row_stride;
+    p.score_cols = max_seqlen_k;
+    p.scale_log2 = softmax_scale * 1.44269504088896340736f;
+    p.causal = is_causal;
+    const dim3 grid((max_seqlen_q + kTokPerBlock - 1) / kTokPerBlock, batch, num_heads_k);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (is_causal) hipLaunchKernelGGL(stage1_kernel<true>, grid, dim3(256), 0, st, p);
+    else hipLaunchKernelGGL(stage1_kernel<false>, grid, dim3(256), 0, st, p);
+    IV2_LAUNCH_CHECK();
+    return 0;
+}
