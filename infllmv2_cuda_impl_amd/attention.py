@@ -42,7 +42,7 @@ def _reject_unsupported(dropout_p, window_size, softcap, alibi_slopes, causal):
         raise RuntimeError("This flash attention build does not support alibi.")
 
 
-def _check_qkv(q, k, v, cu_seqlens_q, cu_seqlens_k):
+def _check_qkv(q, k, v, cu_seqlens_q, cu_seqlens_k, same_kv_len=True):
     """Input checks of mha_varlen_fwd (flash_api.cpp:552-616) that apply to this build."""
     if q.dtype not in (torch.float16, torch.bfloat16):
         raise RuntimeError("FlashAttention only support fp16 and bf16 data type")
@@ -78,7 +78,7 @@ def _check_qkv(q, k, v, cu_seqlens_q, cu_seqlens_k):
         raise RuntimeError("query, key, value, and out_ must have a head_size that is a multiple of 8")
     if q.shape[1] % k.shape[1] != 0:
         raise RuntimeError("Number of heads in key/value must divide number of heads in query")
-    if tuple(k.shape) != (k.shape[0], k.shape[1], head_size) or tuple(v.shape) != tuple(k.shape):
+    if k.shape[2] != head_size or tuple(v.shape[1:]) != tuple(k.shape[1:]) or (same_kv_len and v.shape[0] != k.shape[0]):
         raise RuntimeError("k and v must have shape (total_k, num_heads_k, head_size)")
     if cu_seqlens_k.numel() != batch + 1:
         raise RuntimeError("cu_seqlens_k must have shape (batch_size + 1)")
@@ -205,7 +205,7 @@ def infllmv2_attn_stage1(q, k, v, cu_seqlens_q, cu_seqlens_k, cu_seqlens_v, max_
     if block_table is not None:
         raise RuntimeError("paged KV (block_table) is not supported by this build")
     q, k, v = [_dense_last_dim(x) for x in (q, k, v)]
-    _check_qkv(q, k, v, cu_seqlens_q, cu_seqlens_k)
+    _check_qkv(q, k, v, cu_seqlens_q, cu_seqlens_k, same_kv_len=False)
     if cu_seqlens_v.dtype != torch.int32:
         raise RuntimeError("cu_seqlens_v must have dtype int32")
     return stage1_scores(q, k, v, cu_seqlens_q, cu_seqlens_k, cu_seqlens_v, max_seqlen_q, max_seqlen_k,
