@@ -1,0 +1,224 @@
+#!/usr/bin/env python3
+"""Benchmark of the InfLLM-V2 sparse-attention hot path on one MI355X.
+
+A step is one end-to-end prefill forward of BASELINE config 2: one sequence of 32768 tokens, bf16,
+GQA 32 query / 2 KV heads, d = 128, compressed keys kernel 32 / stride 16 (LSE over kernel 128 /
+stride 64), block 64, topk = 64 (1 init + 32 local blocks forced), causal:
+Stage-1 scores -> max-pool -> top-k -> mask packing -> Stage-2 block-sparse forward.
+Inputs (q, k, v and the caller-side compressed keys) are resident in HBM before the timed region.
+
+`value` = Stage-2 algorithmic sparse FLOPs (4*16*64*128 per selected causal block per token and KV head)
+divided by the time of the WHOLE step, in TFLOP/s.  The JSON line also carries the per-stage times, the
+Stage-2 forward kernel's own roofline figures (HIP events around the kernel alone, K/V images
+prepacked) and the CPU oracle timed on BASELINE config 1.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0      # MI355X dense bf16 MFMA peak (vendor figure, no sparsity)
+PEAK_HBM_GBS = 8000.0          # MI355X HBM3E peak
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--seqlen", type=int, default=32768)
+    ap.add_argument("--topk", type=int, default=64)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-stages", action="store_true", help="skip the per-stage and kernel-only timings")
+    return ap.parse_args()
+
+
+def make_inputs(torch, S, dev, seed=0):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    q = torch.randn(S, 32, 128, generator=g).to(torch.bfloat16).to(dev)
+    k = torch.randn(S, 2, 128, generator=g).to(torch.bfloat16).to(dev)
+    v = torch.randn(S, 2, 128, generator=g).to(torch.bfloat16).to(dev)
+    # caller-side compression (mean over [16j, 16j+32) and [64j, 64j+128)), outside the step
+    kf = k.unfold(0, 32, 16).float().mean(-1).to(torch.bfloat16).contiguous()
+    kc = k.unfold(0, 128, 64).float().mean(-1).to(torch.bfloat16).contiguous()
+    mk = lambda n: torch.tensor([0, n], dtype=torch.int32, device=dev)
+    return q, k, v, kf, kc, mk(S), mk(kf.shape[0]), mk(kc.shape[0])
+
+
+def event_ms(torch, fn, iters, warmup=2):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / iters
+
+
+def cpu_baseline():
+    """The CPU oracle on BASELINE config 1 (2048 tokens, topk 16, block 0 + 2 local blocks forced)."""
+    import numpy as np
+    from oracle import infllmv2_oracle as O
+    try:
+        from threadpoolctl import threadpool_info
+        threads = max([p.get("num_threads", 1) for p in threadpool_info()] or [1])
+    except Exception:
+        threads = 1
+    S, topk = 2048, 16
+    r = np.random.default_rng(0)
+    q = O.bf16_round(r.standard_normal((S, 32, 128)).astype(np.float32))
+    k = O.bf16_round(r.standard_normal((S, 2, 128)).astype(np.float32))
+    v = O.bf16_round(r.standard_normal((S, 2, 128)).astype(np.float32))
+    cu = np.array([0, S], np.int32)
+    kf, cu_f = O.compress_keys(k, cu, 32, 16)
+    kc, cu_c = O.compress_keys(k, cu, 128, 64)
+    times = []
+    flops = 0
+    for _ in range(3):
+        t0 = time.perf_counter()
+        score = O.stage1_scores(q, kf, kc, cu, cu_f, cu_c, int(cu_f[-1]), 128 ** -0.5, True)
+        pooled = O.max_pooling_1d_fast(score, 0, 1, 1)
+        idx = O.topk_blocks(pooled, topk)
+        words, kb = O.topk_to_uint64(idx, S, 64)
+        O.stage2_forward(q, k, v, cu, cu, words, 128 ** -0.5, True, dtype=np.float32)
+        times.append(time.perf_counter() - t0)
+        bits = O.uint64_to_bool(words, kb)
+        causal = np.arange(kb)[None, :] <= (np.arange(S) // 64)[:, None]
+        flops = 4 * 16 * 64 * 128 * int((bits & causal[None]).sum())
+    t = sorted(times)[1]
+    return {"value": flops / t / 1e12, "unit": "TFLOP/s", "cores": int(threads), "kind": "port",
+            "sample": f"BASELINE config 1 (2048 tokens, 32q/2kv, d=128, topk=16, init 1 + 2 local blocks), whole "
+                      f"pipeline in the numpy oracle, median of 3 runs = {t:.2f} s",
+            "seconds": t}
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU; --gpus must be 1 "
+              "(the path shards by KV head or query range with no collective in the kernels; no multi-GPU figure is produced)",
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+    import infllmv2_cuda_impl_amd as ops
+    from infllmv2_cuda_impl_amd import _lib
+
+    dev = torch.device("cuda:0")
+    S, topk = args.seqlen, args.topk
+    nblk = (S + 63) // 64
+    local_blocks, init_blocks = 31, 1
+    q, k, v, kf, kc, cu_q, cu_f, cu_c = make_inputs(torch, S, dev)
+    Lk = kf.shape[0]
+
+    def step():
+        score = ops.infllmv2_attn_stage1(q, kf, kc, cu_q, cu_f, cu_c, S, Lk, causal=True)
+        pooled = ops.max_pooling_1d(score, 0, local_blocks, init_blocks)
+        idx = ops.topk_blocks(pooled, topk)
+        return ops.infllmv2_attn_varlen_func(q, k, v, cu_q, cu_q, S, S, causal=True, topk_idx=idx), idx
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        out, idx = step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # algorithmic FLOPs from the mask actually selected
+    words, _ = ops.topk_to_uint64(idx, S, 64)
+    bits = ops.uint64_to_bool(words, nblk)
+    causal_blk = torch.arange(nblk, device=dev)[None, :] <= (torch.arange(S, device=dev) // 64)[:, None]
+    nsel = int((bits & causal_blk[None]).sum())
+    fwd_flops = 4 * 16 * 64 * 128 * nsel
+    s1_flops = 2 * 16 * 128 * 2 * sum(max(0, (t + 1) // 16 - 1) + max(0, (t + 1) // 64 - 1) for t in range(S))
+
+    result = {
+        "metric": "sparse_attn_fwd_tflops_32k", "value": fwd_flops / ms_per_step / 1e9, "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"BASELINE config 2: prefill forward, 1 x {S} tokens, GQA 32q/2kv, d=128, "
+                               f"kernel 32/stride 16 compressed keys, block 64, topk={topk} "
+                               f"(1 init + 32 local forced), causal; Stage-1 + pool + top-k + pack + Stage-2 fwd",
+                   "seqlen": S, "topk": topk, "selected_causal_blocks_per_token_head": nsel / (2 * S)},
+        "stage2_fwd_algorithmic_flops": fwd_flops, "stage1_algorithmic_flops": s1_flops,
+        "frac_bf16_mfma_peak_whole_step": fwd_flops / ms_per_step / 1e9 / PEAK_BF16_TFLOPS,
+        "peaks": {"bf16_mfma_tflops": PEAK_BF16_TFLOPS, "hbm_gbs": PEAK_HBM_GBS},
+    }
+
+    if not args.no_stages:
+        score = ops.infllmv2_attn_stage1(q, kf, kc, cu_q, cu_f, cu_c, S, Lk, causal=True)
+        pooled = ops.max_pooling_1d(score, 0, local_blocks, init_blocks)
+        stages = {
+            "stage1": event_ms(torch, lambda: ops.infllmv2_attn_stage1(q, kf, kc, cu_q, cu_f, cu_c, S, Lk, causal=True), 10),
+            "pool": event_ms(torch, lambda: ops.max_pooling_1d(score, 0, local_blocks, init_blocks), 10),
+            "topk": event_ms(torch, lambda: ops.topk_blocks(pooled, topk), 10),
+            "pack_mask": event_ms(torch, lambda: ops.topk_to_uint64(idx, S, 64), 10),
+            "stage2_fwd_op": event_ms(torch, lambda: ops.infllmv2_attn_varlen_func(q, k, v, cu_q, cu_q, S, S, causal=True, topk_idx=idx), 10),
+            "transpose_mask": event_ms(torch, lambda: ops.transpose_blockmask(words, nblk), 10),
+        }
+        n64 = words.shape[-1]
+        stages_gbs = {
+            "pool": (2 * S * Lk * 2 + 2 * S * nblk * 2) / stages["pool"] / 1e6,
+            "topk": (2 * S * nblk * 2 + 2 * S * topk * 4) / stages["topk"] / 1e6,
+            "pack_mask": (2 * S * topk * 4 + 2 * S * n64 * 8) / stages["pack_mask"] / 1e6,
+            "transpose_mask": (2 * 2 * S * n64 * 8) / stages["transpose_mask"] / 1e6,
+        }
+        result["stages_ms"] = stages
+        result["stages_hbm_gbs"] = stages_gbs
+        result["stage1_tflops"] = s1_flops / stages["stage1"] / 1e9
+        sel_ms = stages["stage1"] + stages["pool"] + stages["topk"]
+        result["stage1_pool_topk_share_of_fwd"] = sel_ms / (sel_ms + stages["pack_mask"] + stages["stage2_fwd_op"])
+
+        # the dominant kernel alone: K/V images prepacked, mask packed, HIP events on the launch stream
+        out_k = torch.empty_like(q)
+        lse = torch.empty((2, S * 16), dtype=torch.float32, device=dev)
+        ws = torch.empty(_lib.lib.infllmv2_kv_image_bytes(S, 1, 2), dtype=torch.uint8, device=dev)
+        qs = _lib.i64_array([q.stride(0), q.stride(1), 16 * q.stride(1)])
+        ks = _lib.i64_array([k.stride(0), k.stride(1)])
+        ls = _lib.i64_array([16, 1, S * 16])
+        stream = torch.cuda.current_stream(dev).cuda_stream
+
+        def kernel_only(prepacked=1):
+            _lib.call("infllmv2_varlen_fwd", stream, q.data_ptr(), k.data_ptr(), v.data_ptr(), out_k.data_ptr(),
+                      lse.data_ptr(), cu_q.data_ptr(), cu_q.data_ptr(), words.data_ptr(), ws.data_ptr(), ws.numel(),
+                      prepacked, 1, S, S, 32, 2, 128, S, S, qs, ks, ks, qs, ls, n64, 128 ** -0.5, 1)
+        kernel_only(0)
+        k_ms = event_ms(torch, kernel_only, max(10, args.steps))
+        achieved = fwd_flops / k_ms / 1e9
+        result["roofline"] = {"bound": "mfma", "kernel": "stage2_fwd_kernel<causal>", "achieved": achieved,
+                              "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS,
+                              "traffic": None, "kernel_ms": k_ms}
+        try:
+            from infllmv2_cuda_impl_amd.backward import HAVE_BACKWARD  # noqa: F401
+            qg, kg, vg = [t.clone().requires_grad_(True) for t in (q, k, v)]
+            dout = torch.randn_like(q)
+
+            def fwd_bwd():
+                o = ops.infllmv2_attn_varlen_func(qg, kg, vg, cu_q, cu_q, S, S, causal=True, topk_idx=idx)
+                o.backward(dout)
+                qg.grad = kg.grad = vg.grad = None
+            fb_ms = event_ms(torch, fwd_bwd, 5)
+            result["stage2_fwd_bwd_ms"] = fb_ms
+            result["stage2_fwd_bwd_tflops"] = 3.5 * fwd_flops / fb_ms / 1e9
+            result["stage2_fwd_bwd_frac_peak"] = 3.5 * fwd_flops / fb_ms / 1e9 / PEAK_BF16_TFLOPS
+        except ImportError:
+            pass
+
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -137,15 +137,25 @@ size_t infllmv2_kv_image_bytes(int64_t total_k, int batch, int num_heads_k);
  * k/v: (total_k, Hk, d), strides {row, head}.  softmax_lse strides {token, head-in-group, kv-head};
  *   the reference's (Hk, T*16) layout (flash_api.cpp:665) is {16, 1, T*16}.
  * blockmask (Hk, total_q, n_uint64_per_row): block indices local to each sequence, rows by packed
- *   token index (flash_blockmask.h:20-31). */
+ *   token index (flash_blockmask.h:20-31).
+ * workspace: infllmv2_kv_image_bytes() bytes, 16-byte aligned; filled here unless kv_prepacked. */
 int infllmv2_varlen_fwd(void* stream, const void* q, const void* k, const void* v, void* out,
                         float* softmax_lse, const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
-                        const uint64_t* blockmask, void* workspace, size_t workspace_bytes, int batch,
-                        int64_t total_q, int64_t total_k, int num_heads, int num_heads_k, int head_dim,
-                        int max_seqlen_q, int max_seqlen_k, const int64_t* q_strides,
-                        const int64_t* k_strides, const int64_t* v_strides, const int64_t* o_strides,
-                        const int64_t* lse_strides, int n_uint64_per_row, float softmax_scale,
-                        int is_causal);
+                        const uint64_t* blockmask, void* workspace, size_t workspace_bytes,
+                        int kv_prepacked, int batch, int64_t total_q, int64_t total_k, int num_heads,
+                        int num_heads_k, int head_dim, int max_seqlen_q, int max_seqlen_k,
+                        const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                        const int64_t* o_strides, const int64_t* lse_strides, int n_uint64_per_row,
+                        float softmax_scale, int is_causal);
+
+/* First half of infllmv2_varlen_fwd on its own: rewrites k, v (total_k, Hk, 128; strides {row, head})
+ * into the block images in `workspace`.  A later infllmv2_varlen_fwd / _bwd call on the same k, v
+ * may then pass kv_prepacked = 1 (k and v are not read).  No counterpart in the reference, whose
+ * kernels read K/V in the caller's layout. */
+int infllmv2_pack_kv(void* stream, const void* k, const void* v, const int32_t* cu_seqlens_k,
+                     void* workspace, size_t workspace_bytes, int batch, int64_t total_k,
+                     int num_heads_k, int head_dim, int max_seqlen_k, const int64_t* k_strides,
+                     const int64_t* v_strides);
 
 #ifdef __cplusplus
 }

@@ -29,8 +29,9 @@ SIGNATURES = {
     "infllmv2_topk": [_p, _i, _i, _i, _i, _p, _p, _p],
     "infllmv2_topk_blocks": [_p, _p, _i64, _p, _i64, _i, _i],
     "infllmv2_varlen_fwd_stage1": [_p, _p, _p, _p, _p, _p, _p, _p, _i, _i64, _i, _i, _i, _i, _i, _p, _p, _p, _i64, _i64, _f, _i],
-    "infllmv2_varlen_fwd": [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _sz, _i, _i64, _i64, _i, _i, _i, _i, _i,
+    "infllmv2_varlen_fwd": [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _sz, _i, _i, _i64, _i64, _i, _i, _i, _i, _i,
                             _p, _p, _p, _p, _p, _i, _f, _i],
+    "infllmv2_pack_kv": [_p, _p, _p, _p, _p, _sz, _i, _i64, _i, _i, _i, _p, _p],
 }
 OTHER = {
     "infllmv2_last_error": (C.c_char_p, []),

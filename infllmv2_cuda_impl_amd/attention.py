@@ -113,7 +113,7 @@ def _sparse_forward(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqle
     with torch.cuda.device(q.device):
         _lib.call("infllmv2_varlen_fwd", stream_ptr(q.device), q.data_ptr(), k.data_ptr(), v.data_ptr(),
                   out.data_ptr(), lse.data_ptr(), cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), ptr(fwd_mask),
-                  workspace.data_ptr(), workspace.numel(), batch, total_q, total_k, Hq, Hk, d, max_seqlen_q,
+                  workspace.data_ptr(), workspace.numel(), 0, batch, total_q, total_k, Hq, Hk, d, max_seqlen_q,
                   max_seqlen_k, _natural_strides(q), _lib.i64_array([k.stride(0), k.stride(1)]),
                   _lib.i64_array([v.stride(0), v.stride(1)]), _natural_strides(out), lse_strides, n64,
                   float(softmax_scale), int(bool(causal)))

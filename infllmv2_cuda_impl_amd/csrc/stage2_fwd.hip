@@ -293,11 +293,48 @@ extern "C" size_t infllmv2_kv_image_bytes(int64_t total_k, int batch, int num_he
     return static_cast<size_t>(image_slots(total_k, batch)) * num_heads_k * kImageElems * sizeof(bf16_bits) * 2;
 }
 
+static int launch_pack(hipStream_t st, const void* k, const void* v, const int32_t* cu_seqlens_k, void* workspace,
+                       size_t workspace_bytes, int batch, int64_t total_k, int num_heads_k, int max_seqlen_k,
+                       const int64_t* k_strides, const int64_t* v_strides) {
+    IV2_CHECK(k && v && cu_seqlens_k && workspace, "pack_kv: null pointer");
+    IV2_CHECK(batch > 0 && num_heads_k > 0 && total_k >= 0 && max_seqlen_k >= 0, "pack_kv: bad sizes");
+    IV2_CHECK(num_heads_k <= 65535 && batch <= 65535, "pack_kv: batch and num_heads_k must not exceed 65535");
+    IV2_CHECK(workspace_bytes >= infllmv2_kv_image_bytes(total_k, batch, num_heads_k), "pack_kv: workspace too small");
+    IV2_CHECK(reinterpret_cast<uintptr_t>(k) % 16 == 0 && reinterpret_cast<uintptr_t>(v) % 16 == 0 &&
+              reinterpret_cast<uintptr_t>(workspace) % 16 == 0, "pack_kv: k, v and workspace must be 16-byte aligned");
+    IV2_CHECK(k_strides[0] % 8 == 0 && k_strides[1] % 8 == 0 && v_strides[0] % 8 == 0 && v_strides[1] % 8 == 0,
+              "pack_kv: k/v row and head strides must be multiples of 8 elements");
+    const int64_t n_slots = image_slots(total_k, batch);
+    const int max_blocks = (max_seqlen_k + kBlockN - 1) / kBlockN;
+    if (max_blocks == 0 || total_k == 0) return 0;
+    PackParams pp{};
+    pp.k = static_cast<const bf16_bits*>(k);
+    pp.v = static_cast<const bf16_bits*>(v);
+    pp.kimg = static_cast<bf16_bits*>(workspace);
+    pp.vimg = pp.kimg + n_slots * num_heads_k * kImageElems;
+    pp.cu_seqlens_k = cu_seqlens_k;
+    pp.k_row_stride = k_strides[0]; pp.k_head_stride = k_strides[1];
+    pp.v_row_stride = v_strides[0]; pp.v_head_stride = v_strides[1];
+    pp.n_slots = n_slots;
+    hipLaunchKernelGGL(pack_kv_kernel, dim3(max_blocks, batch, num_heads_k), dim3(256), 0, st, pp);
+    IV2_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int infllmv2_pack_kv(void* stream, const void* k, const void* v, const int32_t* cu_seqlens_k,
+                                void* workspace, size_t workspace_bytes, int batch, int64_t total_k,
+                                int num_heads_k, int head_dim, int max_seqlen_k, const int64_t* k_strides,
+                                const int64_t* v_strides) {
+    IV2_CHECK(head_dim == kHeadDim, "pack_kv: this build only supports head_dim 128 (got %d)", head_dim);
+    return launch_pack(static_cast<hipStream_t>(stream), k, v, cu_seqlens_k, workspace, workspace_bytes, batch,
+                       total_k, num_heads_k, max_seqlen_k, k_strides, v_strides);
+}
+
 extern "C" int infllmv2_varlen_fwd(void* stream, const void* q, const void* k, const void* v, void* out,
                                    float* softmax_lse, const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
                                    const uint64_t* blockmask, void* workspace, size_t workspace_bytes,
-                                   int batch, int64_t total_q, int64_t total_k, int num_heads, int num_heads_k,
-                                   int head_dim, int max_seqlen_q, int max_seqlen_k,
+                                   int kv_prepacked, int batch, int64_t total_q, int64_t total_k, int num_heads,
+                                   int num_heads_k, int head_dim, int max_seqlen_q, int max_seqlen_k,
                                    const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
                                    const int64_t* o_strides, const int64_t* lse_strides,
                                    int n_uint64_per_row, float softmax_scale, int is_causal) {
@@ -305,42 +342,30 @@ extern "C" int infllmv2_varlen_fwd(void* stream, const void* q, const void* k, c
     IV2_CHECK(num_heads_k > 0 && num_heads == num_heads_k * kGroup,
               "varlen_fwd: requires num_heads == 16 * num_heads_k (got %d and %d)", num_heads, num_heads_k);
     IV2_CHECK(batch > 0 && total_q >= 0 && total_k >= 0 && max_seqlen_q >= 0 && max_seqlen_k >= 0, "varlen_fwd: bad sizes");
-    IV2_CHECK(q && k && v && out && softmax_lse && cu_seqlens_q && cu_seqlens_k, "varlen_fwd: null pointer");
+    IV2_CHECK(q && out && softmax_lse && cu_seqlens_q && cu_seqlens_k && workspace, "varlen_fwd: null pointer");
     IV2_CHECK(num_heads_k <= 65535 && batch <= 65535, "varlen_fwd: batch and num_heads_k must not exceed 65535");
     IV2_CHECK(workspace_bytes >= infllmv2_kv_image_bytes(total_k, batch, num_heads_k), "varlen_fwd: workspace too small");
-    IV2_CHECK(reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(k) % 16 == 0 &&
-              reinterpret_cast<uintptr_t>(v) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 8 == 0 &&
-              reinterpret_cast<uintptr_t>(workspace) % 16 == 0, "varlen_fwd: q, k, v and workspace must be 16-byte aligned");
+    IV2_CHECK(reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 8 == 0 &&
+              reinterpret_cast<uintptr_t>(workspace) % 16 == 0, "varlen_fwd: q and workspace must be 16-byte aligned, out 8-byte");
     for (int s = 0; s < 3; ++s) {
         IV2_CHECK(q_strides[s] % 8 == 0 && o_strides[s] % 4 == 0, "varlen_fwd: q strides must be multiples of 8 and out strides of 4 elements");
     }
-    IV2_CHECK(k_strides[0] % 8 == 0 && k_strides[1] % 8 == 0 && v_strides[0] % 8 == 0 && v_strides[1] % 8 == 0,
-              "varlen_fwd: k/v row and head strides must be multiples of 8 elements");
     IV2_CHECK(blockmask == nullptr || n_uint64_per_row > 0, "varlen_fwd: mask given without words per row");
+    IV2_CHECK(softmax_scale > 0.f, "varlen_fwd: softmax_scale must be positive");
     if (total_q == 0 || max_seqlen_q == 0) return 0;
     hipStream_t st = static_cast<hipStream_t>(stream);
-
-    const int64_t n_slots = image_slots(total_k, batch);
-    bf16_bits* kimg = static_cast<bf16_bits*>(workspace);
-    bf16_bits* vimg = kimg + n_slots * num_heads_k * kImageElems;
-    const int max_blocks = (max_seqlen_k + kBlockN - 1) / kBlockN;
-    if (max_blocks > 0 && total_k > 0) {
-        PackParams pp{};
-        pp.k = static_cast<const bf16_bits*>(k);
-        pp.v = static_cast<const bf16_bits*>(v);
-        pp.kimg = kimg; pp.vimg = vimg;
-        pp.cu_seqlens_k = cu_seqlens_k;
-        pp.k_row_stride = k_strides[0]; pp.k_head_stride = k_strides[1];
-        pp.v_row_stride = v_strides[0]; pp.v_head_stride = v_strides[1];
-        pp.n_slots = n_slots;
-        hipLaunchKernelGGL(pack_kv_kernel, dim3(max_blocks, batch, num_heads_k), dim3(256), 0, st, pp);
-        IV2_LAUNCH_CHECK();
+    if (!kv_prepacked) {
+        int rc = launch_pack(st, k, v, cu_seqlens_k, workspace, workspace_bytes, batch, total_k, num_heads_k,
+                             max_seqlen_k, k_strides, v_strides);
+        if (rc != 0) return rc;
     }
+    const int64_t n_slots = image_slots(total_k, batch);
     FwdParams fp{};
     fp.q = static_cast<const bf16_bits*>(q);
     fp.out = static_cast<bf16_bits*>(out);
     fp.lse = softmax_lse;
-    fp.kimg = kimg; fp.vimg = vimg;
+    fp.kimg = static_cast<const bf16_bits*>(workspace);
+    fp.vimg = fp.kimg + n_slots * num_heads_k * kImageElems;
     fp.cu_seqlens_q = cu_seqlens_q; fp.cu_seqlens_k = cu_seqlens_k;
     fp.mask = blockmask;
     fp.q_tok_stride = q_strides[0]; fp.q_grp_stride = q_strides[1]; fp.q_kvh_stride = q_strides[2];
