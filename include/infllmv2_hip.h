@@ -157,6 +157,31 @@ int infllmv2_pack_kv(void* stream, const void* k, const void* v, const int32_t* 
                      int num_heads_k, int head_dim, int max_seqlen_k, const int64_t* k_strides,
                      const int64_t* v_strides);
 
+/* Scratch for infllmv2_varlen_bwd: four K/V block images, the transposed mask, D = rowsum(dO*O),
+ * transposed per-token images of q and dout, fp32 dK/dV accumulators. */
+size_t infllmv2_varlen_bwd_workspace_bytes(int batch, int64_t total_q, int64_t total_k, int num_heads_k,
+                                           int max_seqlen_k);
+
+/* csrc/entry.cu:17,213 `varlen_bwd` = mha_varlen_bwd (csrc/flash_attn/flash_api.cpp:1278-1547; kernels
+ * flash_bwd_kernel.h:80-856, flash_bwd_preprocess_kernel.h:56-137,181-263) together with the mask
+ * transposition the reference does in Python (infllmv2_sparse_attention.py:344-350): it takes the
+ * FORWARD mask (Hk, total_q, n_uint64_per_row), or null for dense attention.
+ * dout, q, out, dq: strides {token, head-in-group, kv-head} as in infllmv2_varlen_fwd; k, v, dk, dv:
+ * {row, head}; softmax_lse: the forward's output with its strides.  dq, dk, dv are fully written
+ * (bf16).  workspace: infllmv2_varlen_bwd_workspace_bytes() bytes, 256-byte aligned.  dK/dV are
+ * accumulated with fp32 atomics (one flush per 64-key block and 2048-token slice), so their last bits
+ * can differ between runs, as the reference's dQ does; dQ is bit-reproducible. */
+int infllmv2_varlen_bwd(void* stream, const void* dout, const void* q, const void* k, const void* v,
+                        const void* out, const float* softmax_lse, void* dq, void* dk, void* dv,
+                        const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                        const uint64_t* fwd_blockmask, void* workspace, size_t workspace_bytes, int batch,
+                        int64_t total_q, int64_t total_k, int num_heads, int num_heads_k, int head_dim,
+                        int max_seqlen_q, int max_seqlen_k, const int64_t* q_strides,
+                        const int64_t* k_strides, const int64_t* v_strides, const int64_t* o_strides,
+                        const int64_t* do_strides, const int64_t* dq_strides, const int64_t* dk_strides,
+                        const int64_t* dv_strides, const int64_t* lse_strides, int n_uint64_per_row,
+                        float softmax_scale, int is_causal);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,54 @@
+// Mask-row iteration and small cross-lane helpers shared by the Stage-2 kernels.
+#pragma once
+#include "common.h"
+
+namespace infllmv2 {
+
+// Walks the set bits of one mask row in ascending block order, clipped to [0, last_blk].
+struct BlockWalker {
+    const uint64_t* row;
+    int n_words;                    // words that can hold an allowed block
+    int last_blk;
+    int w;
+    uint64_t bits;
+
+    __device__ __forceinline__ uint64_t load_word(int word) const {
+        uint64_t v = row ? row[word] : ~0ull;
+        if (word == (last_blk >> 6)) {
+            const int t = last_blk & 63;
+            v &= (t == 63) ? ~0ull : ((1ull << (t + 1)) - 1ull);
+        }
+        // the row is shared by the whole wavefront: keep the loop control in scalar registers
+        const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
+        const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
+        return (static_cast<uint64_t>(hi) << 32) | lo;
+    }
+    __device__ __forceinline__ void init(const uint64_t* r, int words_in_row, int last) {
+        row = r;
+        last_blk = last;
+        n_words = last < 0 ? 0 : (last >> 6) + 1;
+        if (row && n_words > words_in_row) n_words = words_in_row;
+        w = 0;
+        bits = n_words > 0 ? load_word(0) : 0ull;
+    }
+    __device__ __forceinline__ int next() {
+        while (bits == 0ull) {
+            if (++w >= n_words) return -1;
+            bits = load_word(w);
+        }
+        const int bit = __builtin_ctzll(bits);
+        bits &= bits - 1ull;
+        return w * 64 + bit;
+    }
+};
+
+__device__ __forceinline__ float wave_max_over_g(float x) {
+    x = fmaxf(x, __shfl_xor(x, 16));
+    return fmaxf(x, __shfl_xor(x, 32));
+}
+__device__ __forceinline__ float wave_sum_over_g(float x) {
+    x += __shfl_xor(x, 16);
+    return x + __shfl_xor(x, 32);
+}
+
+}  // namespace infllmv2

@@ -15,6 +15,7 @@
 // LSE are addressed through strides: the caller's (T, Hq, d) tensors are used in place.
 #include "common.h"
 #include "kv_image.h"
+#include "block_walker.h"
 #include "../../include/infllmv2_hip.h"
 #include <math.h>
 
@@ -26,8 +27,10 @@ namespace infllmv2 {
 struct PackParams {
     const bf16_bits* k;
     const bf16_bits* v;
-    bf16_bits* kimg;
-    bf16_bits* vimg;
+    bf16_bits* kimg;                // K in K-image order (A/B operand of a GEMM contracting over d)
+    bf16_bits* vimg;                // V in V-image order (A operand of a GEMM contracting over keys)
+    bf16_bits* kimg_t;              // optional: K in V-image order (backward: dQ^T = K^T dS^T)
+    bf16_bits* vimg_r;              // optional: V in K-image order (backward: dP = dO V^T)
     const int* cu_seqlens_k;        // cumulative (batch + 1) or, for a cache, null
     const int* seqlens_k;           // per-sequence lengths when cu_seqlens_k is null
     int64_t k_batch_stride, k_row_stride, k_head_stride;
@@ -58,8 +61,9 @@ void pack_kv_kernel(const PackParams p) {
     const int tid = threadIdx.x;
     const bf16_bits* kb = p.k + b * p.k_batch_stride + (row0 + static_cast<int64_t>(j) * kBlockN) * p.k_row_stride + h * p.k_head_stride;
     const bf16_bits* vb = p.v + b * p.v_batch_stride + (row0 + static_cast<int64_t>(j) * kBlockN) * p.v_row_stride + h * p.v_head_stride;
-    bf16_bits* kdst = p.kimg + (static_cast<int64_t>(h) * p.n_slots + slot) * kImageElems;
-    bf16_bits* vdst = p.vimg + (static_cast<int64_t>(h) * p.n_slots + slot) * kImageElems;
+    const int64_t img_off = (static_cast<int64_t>(h) * p.n_slots + slot) * kImageElems;
+    bf16_bits* kdst = p.kimg + img_off;
+    bf16_bits* vdst = p.vimg + img_off;
     const int valid = Sk - j * kBlockN;                       // keys of this block inside the sequence
     const uint4 zero = make_uint4(0, 0, 0, 0);
 
@@ -70,6 +74,11 @@ void pack_kv_kernel(const PackParams p) {
         uint4 val = zero;
         if (key < valid) val = *reinterpret_cast<const uint4*>(kb + key * p.k_row_stride + 32 * c + 8 * g);
         *reinterpret_cast<uint4*>(kdst + u * 8) = val;
+        if (p.vimg_r != nullptr) {
+            uint4 vv = zero;
+            if (key < valid) vv = *reinterpret_cast<const uint4*>(vb + key * p.v_row_stride + 32 * c + 8 * g);
+            *reinterpret_cast<uint4*>(p.vimg_r + img_off + u * 8) = vv;
+        }
     }
     for (int u = tid; u < 1024; u += 256) {
         const int key = u >> 4, d0 = (u & 15) * 8;
@@ -89,6 +98,27 @@ void pack_kv_kernel(const PackParams p) {
             w[jj >> 1] = static_cast<uint32_t>(vt[key_a][d]) | (static_cast<uint32_t>(vt[key_a + 1][d]) << 16);
         }
         *reinterpret_cast<uint4*>(vdst + u * 8) = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+    if (p.kimg_t == nullptr) return;                          // uniform per workgroup
+    __syncthreads();
+    for (int u = tid; u < 1024; u += 256) {
+        const int key = u >> 4, d0 = (u & 15) * 8;
+        uint4 val = zero;
+        if (key < valid) val = *reinterpret_cast<const uint4*>(kb + key * p.k_row_stride + d0);
+        *reinterpret_cast<uint4*>(&vt[key][d0]) = val;
+    }
+    __syncthreads();
+    for (int u = tid; u < 1024; u += 256) {
+        const int dt = u >> 7, cc = (u >> 6) & 1, lane = u & 63;
+        const int r = lane & 15, g = lane >> 4;
+        const int d = 16 * dt + r;
+        uint32_t w[4];
+#pragma unroll
+        for (int jj = 0; jj < 8; jj += 2) {
+            const int key_a = 32 * cc + (jj < 4 ? 4 * g + jj : 16 + 4 * g + jj - 4);
+            w[jj >> 1] = static_cast<uint32_t>(vt[key_a][d]) | (static_cast<uint32_t>(vt[key_a + 1][d]) << 16);
+        }
+        *reinterpret_cast<uint4*>(p.kimg_t + img_off + u * 8) = make_uint4(w[0], w[1], w[2], w[3]);
     }
 }
 
@@ -112,53 +142,6 @@ struct FwdParams {
     int n64;
     float scale_log2;               // softmax_scale * log2(e)
 };
-
-// Walks the set bits of one mask row in ascending block order, clipped to [0, last_blk].
-struct BlockWalker {
-    const uint64_t* row;
-    int n_words;                    // words that can hold an allowed block
-    int last_blk;
-    int w;
-    uint64_t bits;
-
-    __device__ __forceinline__ uint64_t load_word(int word) const {
-        uint64_t v = row ? row[word] : ~0ull;
-        if (word == (last_blk >> 6)) {
-            const int t = last_blk & 63;
-            v &= (t == 63) ? ~0ull : ((1ull << (t + 1)) - 1ull);
-        }
-        // the row is shared by the whole wavefront: keep the loop control in scalar registers
-        const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
-        const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
-        return (static_cast<uint64_t>(hi) << 32) | lo;
-    }
-    __device__ __forceinline__ void init(const uint64_t* r, int words_in_row, int last) {
-        row = r;
-        last_blk = last;
-        n_words = last < 0 ? 0 : (last >> 6) + 1;
-        if (row && n_words > words_in_row) n_words = words_in_row;
-        w = 0;
-        bits = n_words > 0 ? load_word(0) : 0ull;
-    }
-    __device__ __forceinline__ int next() {
-        while (bits == 0ull) {
-            if (++w >= n_words) return -1;
-            bits = load_word(w);
-        }
-        const int bit = __builtin_ctzll(bits);
-        bits &= bits - 1ull;
-        return w * 64 + bit;
-    }
-};
-
-__device__ __forceinline__ float wave_max_over_g(float x) {
-    x = fmaxf(x, __shfl_xor(x, 16));
-    return fmaxf(x, __shfl_xor(x, 32));
-}
-__device__ __forceinline__ float wave_sum_over_g(float x) {
-    x += __shfl_xor(x, 16);
-    return x + __shfl_xor(x, 32);
-}
 
 template <bool kCausal>
 __global__ __launch_bounds__(256)
@@ -293,13 +276,15 @@ extern "C" size_t infllmv2_kv_image_bytes(int64_t total_k, int batch, int num_he
     return static_cast<size_t>(image_slots(total_k, batch)) * num_heads_k * kImageElems * sizeof(bf16_bits) * 2;
 }
 
-static int launch_pack(hipStream_t st, const void* k, const void* v, const int32_t* cu_seqlens_k, void* workspace,
-                       size_t workspace_bytes, int batch, int64_t total_k, int num_heads_k, int max_seqlen_k,
-                       const int64_t* k_strides, const int64_t* v_strides) {
+namespace infllmv2 {
+int launch_pack(hipStream_t st, const void* k, const void* v, const int32_t* cu_seqlens_k, void* workspace,
+                size_t workspace_bytes, int batch, int64_t total_k, int num_heads_k, int max_seqlen_k,
+                const int64_t* k_strides, const int64_t* v_strides, bool backward_images) {
     IV2_CHECK(k && v && cu_seqlens_k && workspace, "pack_kv: null pointer");
     IV2_CHECK(batch > 0 && num_heads_k > 0 && total_k >= 0 && max_seqlen_k >= 0, "pack_kv: bad sizes");
     IV2_CHECK(num_heads_k <= 65535 && batch <= 65535, "pack_kv: batch and num_heads_k must not exceed 65535");
-    IV2_CHECK(workspace_bytes >= infllmv2_kv_image_bytes(total_k, batch, num_heads_k), "pack_kv: workspace too small");
+    IV2_CHECK(workspace_bytes >= infllmv2_kv_image_bytes(total_k, batch, num_heads_k) * (backward_images ? 2 : 1),
+              "pack_kv: workspace too small");
     IV2_CHECK(reinterpret_cast<uintptr_t>(k) % 16 == 0 && reinterpret_cast<uintptr_t>(v) % 16 == 0 &&
               reinterpret_cast<uintptr_t>(workspace) % 16 == 0, "pack_kv: k, v and workspace must be 16-byte aligned");
     IV2_CHECK(k_strides[0] % 8 == 0 && k_strides[1] % 8 == 0 && v_strides[0] % 8 == 0 && v_strides[1] % 8 == 0,
@@ -312,6 +297,10 @@ static int launch_pack(hipStream_t st, const void* k, const void* v, const int32
     pp.v = static_cast<const bf16_bits*>(v);
     pp.kimg = static_cast<bf16_bits*>(workspace);
     pp.vimg = pp.kimg + n_slots * num_heads_k * kImageElems;
+    if (backward_images) {
+        pp.kimg_t = pp.vimg + n_slots * num_heads_k * kImageElems;
+        pp.vimg_r = pp.kimg_t + n_slots * num_heads_k * kImageElems;
+    }
     pp.cu_seqlens_k = cu_seqlens_k;
     pp.k_row_stride = k_strides[0]; pp.k_head_stride = k_strides[1];
     pp.v_row_stride = v_strides[0]; pp.v_head_stride = v_strides[1];
@@ -320,6 +309,7 @@ static int launch_pack(hipStream_t st, const void* k, const void* v, const int32
     IV2_LAUNCH_CHECK();
     return 0;
 }
+}  // namespace infllmv2
 
 extern "C" int infllmv2_pack_kv(void* stream, const void* k, const void* v, const int32_t* cu_seqlens_k,
                                 void* workspace, size_t workspace_bytes, int batch, int64_t total_k,
@@ -327,7 +317,7 @@ extern "C" int infllmv2_pack_kv(void* stream, const void* k, const void* v, cons
                                 const int64_t* v_strides) {
     IV2_CHECK(head_dim == kHeadDim, "pack_kv: this build only supports head_dim 128 (got %d)", head_dim);
     return launch_pack(static_cast<hipStream_t>(stream), k, v, cu_seqlens_k, workspace, workspace_bytes, batch,
-                       total_k, num_heads_k, max_seqlen_k, k_strides, v_strides);
+                       total_k, num_heads_k, max_seqlen_k, k_strides, v_strides, false);
 }
 
 extern "C" int infllmv2_varlen_fwd(void* stream, const void* q, const void* k, const void* v, void* out,
@@ -356,7 +346,7 @@ extern "C" int infllmv2_varlen_fwd(void* stream, const void* q, const void* k, c
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (!kv_prepacked) {
         int rc = launch_pack(st, k, v, cu_seqlens_k, workspace, workspace_bytes, batch, total_k, num_heads_k,
-                             max_seqlen_k, k_strides, v_strides);
+                             max_seqlen_k, k_strides, v_strides, false);
         if (rc != 0) return rc;
     }
     const int64_t n_slots = image_slots(total_k, batch);
