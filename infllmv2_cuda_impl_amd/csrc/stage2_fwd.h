@@ -1,0 +1,30 @@
+// Parameters of the Stage-2 forward kernels.
+#pragma once
+#include "common.h"
+
+namespace infllmv2 {
+
+struct FwdParams {
+    const bf16_bits* q;
+    bf16_bits* out;
+    float* lse;
+    const bf16_bits* kimg;
+    const bf16_bits* vimg;
+    const int* cu_seqlens_q;
+    const int* cu_seqlens_k;
+    const uint64_t* mask;           // (Hk, total_q, n64) or null for dense
+    int64_t q_tok_stride, q_grp_stride, q_kvh_stride;
+    int64_t o_tok_stride, o_grp_stride, o_kvh_stride;
+    int64_t lse_tok_stride, lse_grp_stride, lse_kvh_stride;
+    int64_t n_slots;
+    int64_t total_q;
+    int n64;
+    float scale_log2;               // softmax_scale * log2(e)
+};
+
+// Workgroup-shared forward: 16 consecutive tokens per workgroup walk the union of their mask rows
+// and stage every K/V block image once in LDS.
+int launch_stage2_fwd_shared(hipStream_t st, const FwdParams& p, int batch, int num_heads_k, int max_seqlen_q,
+                             int max_seqlen_k, bool causal);
+
+}  // namespace infllmv2

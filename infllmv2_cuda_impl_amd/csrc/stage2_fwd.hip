@@ -16,8 +16,10 @@
 #include "common.h"
 #include "kv_image.h"
 #include "block_walker.h"
+#include "stage2_fwd.h"
 #include "../../include/infllmv2_hip.h"
 #include <math.h>
+#include <stdlib.h>
 
 namespace infllmv2 {
 
@@ -125,24 +127,6 @@ void pack_kv_kernel(const PackParams p) {
 // ---------------------------------------------------------------------------------------------
 // forward
 // ---------------------------------------------------------------------------------------------
-struct FwdParams {
-    const bf16_bits* q;
-    bf16_bits* out;
-    float* lse;
-    const bf16_bits* kimg;
-    const bf16_bits* vimg;
-    const int* cu_seqlens_q;
-    const int* cu_seqlens_k;
-    const uint64_t* mask;           // (Hk, total_q, n64) or null for dense
-    int64_t q_tok_stride, q_grp_stride, q_kvh_stride;
-    int64_t o_tok_stride, o_grp_stride, o_kvh_stride;
-    int64_t lse_tok_stride, lse_grp_stride, lse_kvh_stride;
-    int64_t n_slots;
-    int64_t total_q;
-    int n64;
-    float scale_log2;               // softmax_scale * log2(e)
-};
-
 template <bool kCausal>
 __global__ __launch_bounds__(256)
 void stage2_fwd_kernel(const FwdParams p) {
@@ -365,6 +349,11 @@ extern "C" int infllmv2_varlen_fwd(void* stream, const void* q, const void* k, c
     fp.total_q = total_q;
     fp.n64 = n_uint64_per_row;
     fp.scale_log2 = softmax_scale * 1.44269504088896340736f;
+    static const bool per_wave = [] {                          // diagnostic switch: one wavefront per token, no LDS
+        const char* e = getenv("INFLLMV2_FWD_PER_WAVE");
+        return e != nullptr && e[0] == '1';
+    }();
+    if (!per_wave) return launch_stage2_fwd_shared(st, fp, batch, num_heads_k, max_seqlen_q, max_seqlen_k, is_causal != 0);
     const dim3 grid((max_seqlen_q + 3) / 4, batch, num_heads_k);
     if (is_causal) hipLaunchKernelGGL(stage2_fwd_kernel<true>, grid, dim3(256), 0, st, fp);
     else hipLaunchKernelGGL(stage2_fwd_kernel<false>, grid, dim3(256), 0, st, fp);
