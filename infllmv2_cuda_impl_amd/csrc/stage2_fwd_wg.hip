@@ -18,16 +18,15 @@
 #include "block_walker.h"
 #include "stage2_fwd.h"
 #include <math.h>
+#include <stdlib.h>
 
 namespace infllmv2 {
 
-constexpr int kTokWG = 16;
-constexpr int kWavesWG = 8;
 constexpr int kChunkGroups = 32;                               // token groups per XCD chunk
 constexpr int kImgUnits = 2048;                                // 16-byte units of one K + V image pair
 
 struct SharedFwdExtra {
-    int groups_per_seq;                                        // ceil(max_seqlen_q / 16)
+    int groups_per_seq;                                        // ceil(max_seqlen_q / tokens per workgroup)
     int batch;
     int num_heads_k;
     int nw_alloc;                                              // mask words reserved per row in LDS
@@ -77,8 +76,9 @@ __device__ __forceinline__ void softmax_tile(floatx4 (&s)[4], float& m, float& l
 
 template <bool kDoA, bool kDoB>
 __device__ __forceinline__ void process_block(const uint4* kb, const uint4* vb, int lane, int g,
-                                              const bf16x8 (&qf)[2][4], floatx4 (&o)[2][8], float (&m)[2],
-                                              float (&l)[2], int limA, int limB, float scale_log2) {
+                                              const bf16x8 (&qA)[4], const bf16x8 (&qB)[4], floatx4 (&oA)[8],
+                                              floatx4 (&oB)[8], float& mA, float& mB, float& lA, float& lB,
+                                              int limA, int limB, float scale_log2) {
     floatx4 sA[4], sB[4];
 #pragma unroll
     for (int kt = 0; kt < 4; ++kt) {
@@ -89,13 +89,13 @@ __device__ __forceinline__ void process_block(const uint4* kb, const uint4* vb, 
             const uint4 raw = kb[(kt * 4 + c) * 64 + lane];
             bf16x8 kf;
             __builtin_memcpy(&kf, &raw, 16);
-            if (kDoA) sA[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[0][c], sA[kt], 0, 0, 0);
-            if (kDoB) sB[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[1][c], sB[kt], 0, 0, 0);
+            if (kDoA) sA[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qA[c], sA[kt], 0, 0, 0);
+            if (kDoB) sB[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qB[c], sB[kt], 0, 0, 0);
         }
     }
     bf16x8 pA[2], pB[2];
-    if (kDoA) softmax_tile(sA, m[0], l[0], o[0], pA, limA, g, scale_log2);
-    if (kDoB) softmax_tile(sB, m[1], l[1], o[1], pB, limB, g, scale_log2);
+    if (kDoA) softmax_tile(sA, mA, lA, oA, pA, limA, g, scale_log2);
+    if (kDoB) softmax_tile(sB, mB, lB, oB, pB, limB, g, scale_log2);
 #pragma unroll
     for (int dt = 0; dt < 8; ++dt)
 #pragma unroll
@@ -103,8 +103,8 @@ __device__ __forceinline__ void process_block(const uint4* kb, const uint4* vb, 
             const uint4 raw = vb[(dt * 2 + cc) * 64 + lane];
             bf16x8 vf;
             __builtin_memcpy(&vf, &raw, 16);
-            if (kDoA) o[0][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pA[cc], o[0][dt], 0, 0, 0);
-            if (kDoB) o[1][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pB[cc], o[1][dt], 0, 0, 0);
+            if (kDoA) oA[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pA[cc], oA[dt], 0, 0, 0);
+            if (kDoB) oB[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pB[cc], oB[dt], 0, 0, 0);
         }
 }
 
@@ -114,13 +114,35 @@ __device__ __forceinline__ uint64_t uniform64(uint64_t v) {
     return (static_cast<uint64_t>(hi) << 32) | lo;
 }
 
-template <bool kCausal>
+__device__ __forceinline__ uint32_t lds_address(const void* ptr) {
+    return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const void*)ptr));
+}
+
+// One wavefront copies 4 KiB from global memory straight into LDS (no registers): lane l moves bytes
+// [16 l, 16 l + 16) of each 1 KiB quarter; the destination base travels in M0.  The compiler does not
+// see these loads, so the callers order them by hand with s_waitcnt vmcnt(n) + barrier.
+__device__ __forceinline__ void dma_copy_4k(const void* src_lane, uint32_t lds_dst) {
+    asm volatile("s_mov_b32 m0, %1\n\t"
+                 "global_load_lds_dwordx4 %0, off\n\t"
+                 "global_load_lds_dwordx4 %0, off offset:1024\n\t"
+                 "global_load_lds_dwordx4 %0, off offset:2048\n\t"
+                 "global_load_lds_dwordx4 %0, off offset:3072\n\t"
+                 :
+                 : "v"(src_lane), "s"(lds_dst)
+                 : "memory", "m0");
+}
+
+constexpr int kWaitVm4 = 0x0F74;                               // s_waitcnt vmcnt(4), other counters untouched
+constexpr int kWaitVm0 = 0x0F70;                               // s_waitcnt vmcnt(0)
+
+template <bool kCausal, int kTW>
 __global__ __launch_bounds__(512)
 void stage2_fwd_shared_kernel(const FwdParams p, const SharedFwdExtra x) {
+    constexpr int kTokWG = 8 * kTW;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-    uint4* img = reinterpret_cast<uint4*>(smem_raw);                               // [2][2048]
-    unsigned long long* uni = reinterpret_cast<unsigned long long*>(smem_raw + 2 * kImgUnits * 16);
-    unsigned long long* rows = uni + x.nw_alloc;                                   // [16][nw_alloc]
+    uint4* img = reinterpret_cast<uint4*>(smem_raw);                               // [3][2048]: K units 0..1023, V units 1024..2047
+    unsigned long long* uni = reinterpret_cast<unsigned long long*>(smem_raw + 3 * kImgUnits * 16);
+    unsigned long long* rows = uni + x.nw_alloc;                                   // [kTokWG][nw_alloc]
 
     // ---- which tokens: XCD-chunked, heaviest first ----
     const int bid = blockIdx.x;
@@ -141,11 +163,11 @@ void stage2_fwd_shared_kernel(const FwdParams p, const SharedFwdExtra x) {
     if (i0 >= Sq) return;                                                          // uniform per workgroup
     const int Sk = p.cu_seqlens_k[b + 1] - p.cu_seqlens_k[b];
 
-    int tok_i[2], last_key[2], last_blk[2];
-    bool live[2];
+    int tok_i[kTW], last_key[kTW], last_blk[kTW];
+    bool live[kTW];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-        tok_i[t] = i0 + 2 * wave + t;
+    for (int t = 0; t < kTW; ++t) {
+        tok_i[t] = i0 + kTW * wave + t;
         live[t] = tok_i[t] < Sq;
         int lk = kCausal ? (tok_i[t] + Sk - Sq) : (Sk - 1);
         if (lk > Sk - 1) lk = Sk - 1;
@@ -166,7 +188,7 @@ void stage2_fwd_shared_kernel(const FwdParams p, const SharedFwdExtra x) {
     for (int w = tid; w < nw; w += 512) uni[w] = 0ull;
     __syncthreads();
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
+    for (int t = 0; t < kTW; ++t) {
         const int64_t tok = static_cast<int64_t>(q0) + (live[t] ? tok_i[t] : 0);
         const uint64_t* mrow = p.mask ? p.mask + (static_cast<int64_t>(h) * p.total_q + tok) * p.n64 : nullptr;
         for (int w = lane; w < nw; w += 64) {
@@ -178,34 +200,43 @@ void stage2_fwd_shared_kernel(const FwdParams p, const SharedFwdExtra x) {
                     v &= (tb == 63) ? ~0ull : ((1ull << (tb + 1)) - 1ull);
                 }
             }
-            rows[(2 * wave + t) * x.nw_alloc + w] = v;
+            rows[(kTW * wave + t) * x.nw_alloc + w] = v;
             if (v != 0ull) atomicOr(&uni[w], static_cast<unsigned long long>(v));
         }
     }
     __syncthreads();
 
     // ---- Q operands (dead tokens read a live row and never compute) ----
-    bf16x8 qf[2][4];
+    bf16x8 qf[kTW][4];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
+    for (int t = 0; t < kTW; ++t) {
         const int64_t tok = static_cast<int64_t>(q0) + (live[t] ? tok_i[t] : i0);
         const bf16_bits* qp = p.q + tok * p.q_tok_stride + h * p.q_kvh_stride + n * p.q_grp_stride + 8 * g;
 #pragma unroll
         for (int c = 0; c < 4; ++c) qf[t][c] = *reinterpret_cast<const bf16x8*>(qp + 32 * c);
     }
-    float m[2] = {-INFINITY, -INFINITY}, l[2] = {0.f, 0.f};
-    floatx4 o[2][8];
+    float m[kTW], l[kTW];
+    floatx4 o[kTW][8];
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+    for (int t = 0; t < kTW; ++t) {
+        m[t] = -INFINITY;
+        l[t] = 0.f;
 #pragma unroll
         for (int dt = 0; dt < 8; ++dt) o[t][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
 
-    // ---- walk the union ----
+    // ---- walk the union; tiles are filled two blocks ahead by LDS DMA ----
     const int64_t slot0 = static_cast<int64_t>(h) * p.n_slots + image_slot0(p.cu_seqlens_k, b);
-    const uint4* kimg = reinterpret_cast<const uint4*>(p.kimg) + slot0 * 1024;
-    const uint4* vimg = reinterpret_cast<const uint4*>(p.vimg) + slot0 * 1024;
-    int cw = -1;                                                                   // word index being walked
-    uint64_t ubits = 0ull, wordA = 0ull, wordB = 0ull;
+    const uint4* src_lane = (wave < 4 ? reinterpret_cast<const uint4*>(p.kimg) + slot0 * 1024 + wave * 256
+                                      : reinterpret_cast<const uint4*>(p.vimg) + slot0 * 1024 + (wave - 4) * 256) + lane;
+    const uint32_t ring_base = __builtin_amdgcn_readfirstlane(lds_address(img) + wave * 4096);
+    auto issue = [&](int jj, int tile) { dma_copy_4k(src_lane + static_cast<int64_t>(jj) * 1024, ring_base + tile * (kImgUnits * 16)); };
+
+    int cw = -1, row_w = -1;
+    uint64_t ubits = 0ull;
+    uint64_t word[kTW];
+#pragma unroll
+    for (int t = 0; t < kTW; ++t) word[t] = 0ull;
     auto next_block = [&]() -> int {
         while (ubits == 0ull) {
             if (++cw >= nw) return -1;
@@ -215,54 +246,46 @@ void stage2_fwd_shared_kernel(const FwdParams p, const SharedFwdExtra x) {
         ubits &= ubits - 1ull;
         return cw * 64 + bit;
     };
-    uint4 stage[4];
-    auto fetch = [&](int j) {
-#pragma unroll
-        for (int it = 0; it < 4; ++it) {
-            const int u = tid + it * 512;
-            stage[it] = (u < 1024) ? kimg[static_cast<int64_t>(j) * 1024 + u] : vimg[static_cast<int64_t>(j) * 1024 + (u - 1024)];
-        }
-    };
-    auto deposit = [&](int buf) {
-#pragma unroll
-        for (int it = 0; it < 4; ++it) img[buf * kImgUnits + tid + it * 512] = stage[it];
-    };
 
-    int j = next_block();
-    int row_w = -1;
-    if (j >= 0) {
-        fetch(j);
-        deposit(0);
-    }
-    __syncthreads();
-    int cur = 0;
-    while (j >= 0) {
-        if ((j >> 6) != row_w) {
-            row_w = j >> 6;
-            wordA = uniform64(rows[(2 * wave) * x.nw_alloc + row_w]);
-            wordB = uniform64(rows[(2 * wave + 1) * x.nw_alloc + row_w]);
+    int j0 = next_block();
+    int j1 = j0 >= 0 ? next_block() : -1;
+    if (j0 >= 0) issue(j0, 0);
+    if (j1 >= 0) issue(j1, 1);
+    int tile = 0;
+    while (j0 >= 0) {
+        if (j1 >= 0) __builtin_amdgcn_s_waitcnt(kWaitVm4); else __builtin_amdgcn_s_waitcnt(kWaitVm0);
+        __syncthreads();                                       // block j0 is in LDS for everyone; tile (tile+2)%3 is free
+        const int j2 = j1 >= 0 ? next_block() : -1;
+        if (j2 >= 0) issue(j2, tile >= 1 ? tile - 1 : 2);
+        if ((j0 >> 6) != row_w) {
+            row_w = j0 >> 6;
+#pragma unroll
+            for (int t = 0; t < kTW; ++t) word[t] = uniform64(rows[(kTW * wave + t) * x.nw_alloc + row_w]);
         }
-        const bool doA = (wordA >> (j & 63)) & 1ull;
-        const bool doB = (wordB >> (j & 63)) & 1ull;
-        // the union walker may already have advanced cw past row_w; remember j before asking for the next
-        const int jn = next_block();
-        if (jn >= 0) fetch(jn);
-        const uint4* kb = img + cur * kImgUnits;
+        const uint4* kb = img + tile * kImgUnits;
         const uint4* vb = kb + 1024;
-        const int limA = (j == last_blk[0]) ? last_key[0] - j * kBlockN : kBlockN;
-        const int limB = (j == last_blk[1]) ? last_key[1] - j * kBlockN : kBlockN;
-        if (doA && doB) process_block<true, true>(kb, vb, lane, g, qf, o, m, l, limA, limB, p.scale_log2);
-        else if (doA) process_block<true, false>(kb, vb, lane, g, qf, o, m, l, limA, limB, p.scale_log2);
-        else if (doB) process_block<false, true>(kb, vb, lane, g, qf, o, m, l, limA, limB, p.scale_log2);
-        if (jn >= 0) deposit(cur ^ 1);
-        __syncthreads();
-        j = jn;
-        cur ^= 1;
+#pragma unroll
+        for (int pr = 0; pr < kTW / 2; ++pr) {
+            const int tA = 2 * pr, tB = 2 * pr + 1;
+            const bool doA = (word[tA] >> (j0 & 63)) & 1ull;
+            const bool doB = (word[tB] >> (j0 & 63)) & 1ull;
+            const int limA = (j0 == last_blk[tA]) ? last_key[tA] - j0 * kBlockN : kBlockN;
+            const int limB = (j0 == last_blk[tB]) ? last_key[tB] - j0 * kBlockN : kBlockN;
+            if (doA && doB)
+                process_block<true, true>(kb, vb, lane, g, qf[tA], qf[tB], o[tA], o[tB], m[tA], m[tB], l[tA], l[tB], limA, limB, p.scale_log2);
+            else if (doA)
+                process_block<true, false>(kb, vb, lane, g, qf[tA], qf[tB], o[tA], o[tB], m[tA], m[tB], l[tA], l[tB], limA, limB, p.scale_log2);
+            else if (doB)
+                process_block<false, true>(kb, vb, lane, g, qf[tA], qf[tB], o[tA], o[tB], m[tA], m[tB], l[tA], l[tB], limA, limB, p.scale_log2);
+        }
+        j0 = j1;
+        j1 = j2;
+        tile = tile == 2 ? 0 : tile + 1;
     }
 
     // ---- epilogue ----
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
+    for (int t = 0; t < kTW; ++t) {
         if (!live[t]) continue;
         const int64_t tok = static_cast<int64_t>(q0) + tok_i[t];
         const float l_tot = wave_sum_over_g(l[t]);
@@ -282,36 +305,40 @@ void stage2_fwd_shared_kernel(const FwdParams p, const SharedFwdExtra x) {
     }
 }
 
+template <bool kCausal, int kTW>
+static int launch_variant(hipStream_t st, const FwdParams& p, SharedFwdExtra x, int max_seqlen_q) {
+    constexpr int kTokWG = 8 * kTW;
+    x.groups_per_seq = (max_seqlen_q + kTokWG - 1) / kTokWG;
+    const int64_t total = static_cast<int64_t>(x.num_heads_k) * x.batch * x.groups_per_seq;
+    IV2_CHECK(total <= 0x3fffffff, "varlen_fwd: too many token groups");
+    x.total_groups = static_cast<int>(total);
+    const int64_t per_round = 8 * kChunkGroups;
+    const int64_t grid = (total + per_round - 1) / per_round * per_round;
+    const size_t lds = 3 * kImgUnits * 16 + static_cast<size_t>(1 + kTokWG) * x.nw_alloc * 8;
+    IV2_CHECK(lds <= 160 * 1024, "varlen_fwd: mask rows too wide for LDS (%d words)", x.nw_alloc);
+    const void* fn = reinterpret_cast<const void*>(&stage2_fwd_shared_kernel<kCausal, kTW>);
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+    IV2_CHECK(e == hipSuccess, "varlen_fwd: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+    hipLaunchKernelGGL((stage2_fwd_shared_kernel<kCausal, kTW>), dim3(static_cast<unsigned>(grid)), dim3(512), lds, st, p, x);
+    IV2_LAUNCH_CHECK();
+    return 0;
+}
+
 int launch_stage2_fwd_shared(hipStream_t st, const FwdParams& p, int batch, int num_heads_k, int max_seqlen_q,
                              int max_seqlen_k, bool causal) {
     SharedFwdExtra x{};
-    x.groups_per_seq = (max_seqlen_q + kTokWG - 1) / kTokWG;
     x.batch = batch;
     x.num_heads_k = num_heads_k;
     const int k_blocks = (max_seqlen_k + kBlockN - 1) / kBlockN;
     x.nw_alloc = p.mask ? p.n64 : (k_blocks + 63) / 64;
     if (x.nw_alloc < 1) x.nw_alloc = 1;
-    const int64_t total = static_cast<int64_t>(num_heads_k) * batch * x.groups_per_seq;
-    IV2_CHECK(total <= 0x3fffffff, "varlen_fwd: too many token groups");
-    x.total_groups = static_cast<int>(total);
-    const int64_t per_round = 8 * kChunkGroups;
-    const int64_t grid = (total + per_round - 1) / per_round * per_round;
-    const size_t lds = 2 * kImgUnits * 16 + static_cast<size_t>(1 + kTokWG) * x.nw_alloc * 8;
-    IV2_CHECK(lds <= 160 * 1024, "varlen_fwd: mask rows too wide for LDS (%d words)", x.nw_alloc);
-    hipError_t e;
-    if (causal) {
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(&stage2_fwd_shared_kernel<true>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
-        IV2_CHECK(e == hipSuccess, "varlen_fwd: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
-        hipLaunchKernelGGL(stage2_fwd_shared_kernel<true>, dim3(static_cast<unsigned>(grid)), dim3(512), lds, st, p, x);
-    } else {
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(&stage2_fwd_shared_kernel<false>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
-        IV2_CHECK(e == hipSuccess, "varlen_fwd: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
-        hipLaunchKernelGGL(stage2_fwd_shared_kernel<false>, dim3(static_cast<unsigned>(grid)), dim3(512), lds, st, p, x);
-    }
-    IV2_LAUNCH_CHECK();
-    return 0;
+    static const int tokens_per_wave = [] {                    // diagnostic switch: 2 or 4 tokens per wavefront
+        const char* e = getenv("INFLLMV2_FWD_TOKENS_PER_WAVE");
+        return (e != nullptr && e[0] == '4') ? 4 : 2;
+    }();
+    if (tokens_per_wave == 4)
+        return causal ? launch_variant<true, 4>(st, p, x, max_seqlen_q) : launch_variant<false, 4>(st, p, x, max_seqlen_q);
+    return causal ? launch_variant<true, 2>(st, p, x, max_seqlen_q) : launch_variant<false, 2>(st, p, x, max_seqlen_q);
 }
 
 }  // namespace infllmv2
