@@ -182,6 +182,31 @@ int infllmv2_varlen_bwd(void* stream, const void* dout, const void* q, const voi
                         const int64_t* dv_strides, const int64_t* lse_strides, int n_uint64_per_row,
                         float softmax_scale, int is_causal);
 
+/* ---- Stage 2: decode against a KV cache -------------------------------------------------------- */
+
+/* The split count infllmv2_fwd_kvcache will use: `requested` if > 0 (capped at 64), else a heuristic
+ * (replaces num_splits_heuristic, csrc/flash_attn/flash_api.cpp:261-295). */
+int infllmv2_fwd_kvcache_num_splits(int batch, int num_heads_k, int requested);
+/* fp32 partial outputs and LSEs of the splits (0 bytes for one split). */
+size_t infllmv2_fwd_kvcache_workspace_bytes(int batch, int num_heads_k, int num_splits);
+
+/* csrc/entry.cu:18,214 `fwd_kvcache` = mha_fwd_kvcache (csrc/flash_attn/flash_api.cpp:1549-1843; kernels
+ * flash_fwd_kernel.h:606-1199 and 1794-1975) for seqlen_q == 1 without rotary / paged KV / cache_batch_idx /
+ * leftpad.  q, out (batch, 1, Hq, 128): strides {batch, head}.  kcache, vcache (batch, capacity, Hk, 128),
+ * k_new, v_new (batch, seqlen_new, Hk, 128) or null: strides {batch, row, head}.  cache_seqlens (batch) int32
+ * or null (= capacity).  New rows are written at cache_seqlens[b] + t first, then attention runs over
+ * [0, cache_seqlens[b] + seqlen_new) restricted to the blocks set in blockmask (batch, Hk, n_uint64_per_row),
+ * or all blocks when it is null.  softmax_lse (batch, Hq) fp32.  num_splits >= 1 as returned by
+ * infllmv2_fwd_kvcache_num_splits. */
+int infllmv2_fwd_kvcache(void* stream, const void* q, void* kcache, void* vcache, const void* k_new,
+                         const void* v_new, const int32_t* cache_seqlens, void* out, float* softmax_lse,
+                         const uint64_t* blockmask, void* workspace, size_t workspace_bytes, int batch,
+                         int seqlen_q, int num_heads, int num_heads_k, int head_dim, int cache_capacity,
+                         int seqlen_new, const int64_t* q_strides, const int64_t* kcache_strides,
+                         const int64_t* vcache_strides, const int64_t* knew_strides,
+                         const int64_t* vnew_strides, const int64_t* o_strides, int n_uint64_per_row,
+                         int num_splits, float softmax_scale);
+
 #ifdef __cplusplus
 }
 #endif

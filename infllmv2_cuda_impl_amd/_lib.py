@@ -32,12 +32,15 @@ SIGNATURES = {
     "infllmv2_varlen_fwd": [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _sz, _i, _i, _i64, _i64, _i, _i, _i, _i, _i,
                             _p, _p, _p, _p, _p, _i, _f, _i],
     "infllmv2_varlen_bwd": [_p] * 14 + [_sz, _i, _i64, _i64, _i, _i, _i, _i, _i] + [_p] * 9 + [_i, _f, _i],
+    "infllmv2_fwd_kvcache": [_p] * 11 + [_sz] + [_i] * 7 + [_p] * 6 + [_i, _i, _f],
     "infllmv2_pack_kv": [_p, _p, _p, _p, _p, _sz, _i, _i64, _i, _i, _i, _p, _p],
 }
 OTHER = {
     "infllmv2_last_error": (C.c_char_p, []),
     "infllmv2_abi_version": (_i, []),
     "infllmv2_kv_image_bytes": (_sz, [_i64, _i, _i]),
+    "infllmv2_fwd_kvcache_workspace_bytes": (_sz, [_i, _i, _i]),
+    "infllmv2_fwd_kvcache_num_splits": (_i, [_i, _i, _i]),
     "infllmv2_varlen_bwd_workspace_bytes": (_sz, [_i, _i64, _i64, _i, _i]),
 }
 

@@ -1,0 +1,362 @@
+// Stage-2 decode against a KV cache for gfx950: one query token per sequence, attention restricted
+// to the 64-key blocks set in the sequence's mask row, optional in-place append of new keys/values.
+//
+// Semantics follow mha_fwd_kvcache (csrc/flash_attn/flash_api.cpp:1549-1843) on the path the
+// Python wrapper takes (infllm_v2/infllmv2_sparse_attention.py:730-757): seqlen_q == 1, so the
+// causal flag is dropped (flash_api.cpp:1628); the 16 grouped heads of a KV head form the row tile
+// (flash_api.cpp:1633-1639); keys [0, cache_seqlens[b] + seqlen_new) are visible; new k/v are
+// written at cache_seqlens[b] first (flash_fwd_kernel.h:792-891); the result must not depend on
+// the number of KV splits (combine by LSE, flash_fwd_kernel.h:1866-1946).
+//
+// Design: decode is HBM-bound (each selected block is 32 KiB of K+V read exactly once, ~2 MiB per
+// sequence and KV head), so the kernel reads the cache in the caller's layout, with no repacking
+// pass.  One single-wavefront workgroup handles one (sequence, KV head, split); a split is a
+// contiguous run of the row's selected blocks (by ordinal, so splits are balanced whatever the
+// mask looks like).  K rows are the MFMA A operand as they lie in memory (contraction over d);
+// V is contracted over keys, so its tile takes one trip through a wavefront-private LDS buffer and
+// is read back transposed.  Partial results are merged by a small combine kernel.
+#include "common.h"
+#include "block_walker.h"
+#include "../../include/infllmv2_hip.h"
+#include <math.h>
+
+namespace infllmv2 {
+
+struct DecodeParams {
+    const bf16_bits* q;
+    bf16_bits* kcache;
+    bf16_bits* vcache;
+    const bf16_bits* knew;
+    const bf16_bits* vnew;
+    bf16_bits* out;
+    float* lse;                     // (batch, Hq)
+    float* o_part;                  // (batch, Hk, splits, 16, 128) fp32, normalised per split
+    float* lse_part;                // (batch, Hk, splits, 16)
+    const int* cache_seqlens;       // null: every sequence fills the whole cache
+    const uint64_t* mask;           // (batch, Hk, n64) or null
+    int64_t q_batch, q_head;        // element strides of q (batch, head); head dim dense
+    int64_t o_batch, o_head;
+    int64_t kc_batch, kc_row, kc_head, vc_batch, vc_row, vc_head;
+    int64_t kn_batch, kn_row, kn_head, vn_batch, vn_row, vn_head;
+    int batch, num_heads_k, capacity, seqlen_new, n64, splits;
+    float scale_log2;
+};
+
+constexpr int kVtPitch = kHeadDim + 8;                         // LDS row pitch (elements) of the V tile
+
+__global__ __launch_bounds__(256)
+void decode_append_kernel(const DecodeParams p) {
+    // one thread moves 16 bytes of one new row of K and of V
+    const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    const int64_t total = static_cast<int64_t>(p.batch) * p.seqlen_new * p.num_heads_k * 16;
+    if (idx >= total) return;
+    const int chunk = static_cast<int>(idx & 15);
+    int64_t r = idx >> 4;
+    const int h = static_cast<int>(r % p.num_heads_k); r /= p.num_heads_k;
+    const int t = static_cast<int>(r % p.seqlen_new);
+    const int b = static_cast<int>(r / p.seqlen_new);
+    const int pos = (p.cache_seqlens ? p.cache_seqlens[b] : 0) + t;
+    if (pos >= p.capacity) return;
+    const uint4 kv = *reinterpret_cast<const uint4*>(p.knew + b * p.kn_batch + t * p.kn_row + h * p.kn_head + chunk * 8);
+    const uint4 vv = *reinterpret_cast<const uint4*>(p.vnew + b * p.vn_batch + t * p.vn_row + h * p.vn_head + chunk * 8);
+    *reinterpret_cast<uint4*>(p.kcache + b * p.kc_batch + static_cast<int64_t>(pos) * p.kc_row + h * p.kc_head + chunk * 8) = kv;
+    *reinterpret_cast<uint4*>(p.vcache + b * p.vc_batch + static_cast<int64_t>(pos) * p.vc_row + h * p.vc_head + chunk * 8) = vv;
+}
+
+template <bool kDirect>
+__global__ __launch_bounds__(64)
+void decode_split_kernel(const DecodeParams p) {
+    __shared__ __attribute__((aligned(16))) bf16_bits vt[kBlockN * kVtPitch];
+    const int lane = threadIdx.x;
+    const int n = lane & 15, g = lane >> 4;
+    const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    int L = (p.cache_seqlens ? p.cache_seqlens[b] : p.capacity - p.seqlen_new) + p.seqlen_new;
+    if (L > p.capacity) L = p.capacity;
+    const int last_blk = L <= 0 ? -1 : ((L - 1) >> 6);
+    const uint64_t* row = p.mask ? p.mask + (static_cast<int64_t>(b) * p.num_heads_k + h) * p.n64 : nullptr;
+    BlockWalker walk;
+    walk.init(row, p.n64, last_blk);
+
+    // how many blocks does the row select, and which run of them is this split's
+    int total = 0;
+    for (int w = lane; w < walk.n_words; w += 64) {
+        uint64_t v = row ? row[w] : ~0ull;
+        if (w == (last_blk >> 6)) {
+            const int t = last_blk & 63;
+            v &= (t == 63) ? ~0ull : ((1ull << (t + 1)) - 1ull);
+        }
+        total += __builtin_popcountll(v);
+    }
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) total += __shfl_xor(total, off);
+    total = __builtin_amdgcn_readfirstlane(total);
+    const int per = (total + p.splits - 1) / p.splits;
+    const int begin = split * per;
+    int count = total - begin;
+    if (count > per) count = per;
+
+    bf16x8 qf[4];
+    {
+        const bf16_bits* qp = p.q + b * p.q_batch + (16 * h + n) * p.q_head + 8 * g;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) qf[c] = *reinterpret_cast<const bf16x8*>(qp + 32 * c);
+    }
+    float m = -INFINITY, l = 0.f;
+    floatx4 o[8];
+#pragma unroll
+    for (int dt = 0; dt < 8; ++dt) o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    const bf16_bits* kbase = p.kcache + b * p.kc_batch + h * p.kc_head;
+    const bf16_bits* vbase = p.vcache + b * p.vc_batch + h * p.vc_head;
+    int j = -1;
+    for (int skip = 0; skip <= begin && count > 0; ++skip) j = walk.next();   // ordinal `begin` of the row
+    for (int it = 0; it < count && j >= 0; ++it) {
+        const int key0 = j * kBlockN;
+        // K rows as A operands; rows past the end are clamped to a valid row and masked below
+        bf16x8 kreg[16];
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt) {
+            int key = key0 + 16 * kt + n;
+            key = key < L ? key : L - 1;
+            const bf16_bits* src = kbase + static_cast<int64_t>(key) * p.kc_row + 8 * g;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) kreg[kt * 4 + c] = *reinterpret_cast<const bf16x8*>(src + 32 * c);
+        }
+        // V tile -> LDS, row-major
+        uint4 vreg[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+            const int unit = lane + 64 * u;
+            int key = key0 + (unit >> 4);
+            key = key < L ? key : L - 1;
+            vreg[u] = *reinterpret_cast<const uint4*>(vbase + static_cast<int64_t>(key) * p.vc_row + (unit & 15) * 8);
+        }
+        floatx4 s[4];
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt) {
+            s[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+                s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[kt * 4 + c], qf[c], s[kt], 0, 0, 0);
+        }
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+            const int unit = lane + 64 * u;
+            *reinterpret_cast<uint4*>(&vt[(unit >> 4) * kVtPitch + (unit & 15) * 8]) = vreg[u];
+        }
+        const int lim = L - 1 - key0;                           // in-block index of the last valid key
+        if (lim < kBlockN - 1) {
+#pragma unroll
+            for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (16 * kt + 4 * g + e > lim) s[kt][e] = -INFINITY;
+        }
+        float mx = -INFINITY;
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) mx = fmaxf(mx, s[kt][e]);
+        mx = wave_max_over_g(mx);
+        const float m_new = fmaxf(m, mx * p.scale_log2);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f(m - m_use);
+        float rs = 0.f;
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float pv = __builtin_amdgcn_exp2f(s[kt][e] * p.scale_log2 - m_use);
+                s[kt][e] = pv;
+                rs += pv;
+            }
+        l = l * alpha + rs;
+        m = m_new;
+#pragma unroll
+        for (int dt = 0; dt < 8; ++dt) o[dt] *= alpha;
+        bf16x8 pf[2];
+#pragma unroll
+        for (int cc = 0; cc < 2; ++cc)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                pf[cc][e] = static_cast<__bf16>(s[2 * cc][e]);
+                pf[cc][4 + e] = static_cast<__bf16>(s[2 * cc + 1][e]);
+            }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_s_barrier();                          // single-wavefront workgroup: orders the LDS tile
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+#pragma unroll
+        for (int dt = 0; dt < 8; ++dt)
+#pragma unroll
+            for (int cc = 0; cc < 2; ++cc) {
+                const int d = 16 * dt + n;
+                uint32_t w[4];
+#pragma unroll
+                for (int jj = 0; jj < 8; jj += 2) {
+                    const int key = 32 * cc + (jj < 4 ? 4 * g + jj : 16 + 4 * g + jj - 4);
+                    w[jj >> 1] = static_cast<uint32_t>(vt[key * kVtPitch + d]) |
+                                 (static_cast<uint32_t>(vt[(key + 1) * kVtPitch + d]) << 16);
+                }
+                const uint4 raw = make_uint4(w[0], w[1], w[2], w[3]);
+                bf16x8 vf;
+                __builtin_memcpy(&vf, &raw, 16);
+                o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[cc], o[dt], 0, 0, 0);
+            }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_s_barrier();                          // tile consumed before the next block overwrites it
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        j = walk.next();
+    }
+
+    const float l_tot = wave_sum_over_g(l);
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    const float lse = l_tot > 0.f ? m * 0.69314718055994530942f + logf(l_tot) : (kDirect ? INFINITY : -INFINITY);
+    if (kDirect) {
+        bf16_bits* op = p.out + b * p.o_batch + (16 * h + n) * p.o_head + 4 * g;
+#pragma unroll
+        for (int dt = 0; dt < 8; ++dt) {
+            uint2 w;
+            w.x = pack_bf16x2(o[dt][0] * inv, o[dt][1] * inv);
+            w.y = pack_bf16x2(o[dt][2] * inv, o[dt][3] * inv);
+            *reinterpret_cast<uint2*>(op + 16 * dt) = w;
+        }
+        if (g == 0) p.lse[static_cast<int64_t>(b) * p.num_heads_k * 16 + 16 * h + n] = lse;
+    } else {
+        const int64_t slot = (static_cast<int64_t>(b) * p.num_heads_k + h) * p.splits + split;
+        float* op = p.o_part + (slot * 16 + n) * kHeadDim + 4 * g;
+#pragma unroll
+        for (int dt = 0; dt < 8; ++dt)
+            *reinterpret_cast<float4*>(op + 16 * dt) = make_float4(o[dt][0] * inv, o[dt][1] * inv, o[dt][2] * inv, o[dt][3] * inv);
+        if (g == 0) p.lse_part[slot * 16 + n] = lse;
+    }
+}
+
+// merge the per-split partials: one workgroup per (sequence, KV head); thread t -> head t / 16, 8 columns
+__global__ __launch_bounds__(256)
+void decode_combine_kernel(const DecodeParams p) {
+    const int h = blockIdx.x, b = blockIdx.y;
+    const int tid = threadIdx.x;
+    const int head = tid >> 4, d0 = (tid & 15) * 8;
+    const int64_t slot0 = (static_cast<int64_t>(b) * p.num_heads_k + h) * p.splits;
+    float mx = -INFINITY;
+    for (int s = 0; s < p.splits; ++s) mx = fmaxf(mx, p.lse_part[(slot0 + s) * 16 + head]);
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    float wsum = 0.f;
+    if (mx != -INFINITY) {
+        for (int s = 0; s < p.splits; ++s) {
+            const float ls = p.lse_part[(slot0 + s) * 16 + head];
+            if (ls == -INFINITY) continue;
+            const float w = expf(ls - mx);
+            wsum += w;
+            const float* src = p.o_part + ((slot0 + s) * 16 + head) * kHeadDim + d0;
+            const float4 a = *reinterpret_cast<const float4*>(src);
+            const float4 c = *reinterpret_cast<const float4*>(src + 4);
+            acc[0] += w * a.x; acc[1] += w * a.y; acc[2] += w * a.z; acc[3] += w * a.w;
+            acc[4] += w * c.x; acc[5] += w * c.y; acc[6] += w * c.z; acc[7] += w * c.w;
+        }
+    }
+    const float inv = wsum > 0.f ? 1.f / wsum : 0.f;
+    uint4 outv;
+    outv.x = pack_bf16x2(acc[0] * inv, acc[1] * inv);
+    outv.y = pack_bf16x2(acc[2] * inv, acc[3] * inv);
+    outv.z = pack_bf16x2(acc[4] * inv, acc[5] * inv);
+    outv.w = pack_bf16x2(acc[6] * inv, acc[7] * inv);
+    *reinterpret_cast<uint4*>(p.out + b * p.o_batch + (16 * h + head) * p.o_head + d0) = outv;
+    if ((tid & 15) == 0)
+        p.lse[static_cast<int64_t>(b) * p.num_heads_k * 16 + 16 * h + head] = wsum > 0.f ? mx + logf(wsum) : INFINITY;
+}
+
+}  // namespace infllmv2
+
+using namespace infllmv2;
+
+extern "C" int infllmv2_fwd_kvcache_num_splits(int batch, int num_heads_k, int requested) {
+    if (requested > 0) return requested > 64 ? 64 : requested;
+    // aim at ~4 single-wavefront workgroups per CU on a 256-CU device
+    const int pairs = batch * num_heads_k;
+    int s = (1024 + pairs - 1) / (pairs > 0 ? pairs : 1);
+    if (s < 1) s = 1;
+    if (s > 16) s = 16;
+    return s;
+}
+
+extern "C" size_t infllmv2_fwd_kvcache_workspace_bytes(int batch, int num_heads_k, int num_splits) {
+    if (num_splits <= 1) return 0;
+    return static_cast<size_t>(batch) * num_heads_k * num_splits * 16 * (kHeadDim + 1) * sizeof(float);
+}
+
+extern "C" int infllmv2_fwd_kvcache(void* stream, const void* q, void* kcache, void* vcache, const void* k_new,
+                                    const void* v_new, const int32_t* cache_seqlens, void* out, float* softmax_lse,
+                                    const uint64_t* blockmask, void* workspace, size_t workspace_bytes, int batch,
+                                    int seqlen_q, int num_heads, int num_heads_k, int head_dim, int cache_capacity,
+                                    int seqlen_new, const int64_t* q_strides, const int64_t* kcache_strides,
+                                    const int64_t* vcache_strides, const int64_t* knew_strides,
+                                    const int64_t* vnew_strides, const int64_t* o_strides, int n_uint64_per_row,
+                                    int num_splits, float softmax_scale) {
+    IV2_CHECK(head_dim == kHeadDim, "fwd_kvcache: this build only supports head_dim 128 (got %d)", head_dim);
+    IV2_CHECK(seqlen_q == 1, "fwd_kvcache: this build only supports one query token per sequence (got %d)", seqlen_q);
+    IV2_CHECK(num_heads_k > 0 && num_heads == num_heads_k * kGroup,
+              "fwd_kvcache: requires num_heads == 16 * num_heads_k (got %d and %d)", num_heads, num_heads_k);
+    IV2_CHECK(batch > 0 && cache_capacity > 0, "fwd_kvcache: batch size and cache capacity must be positive");
+    IV2_CHECK(batch <= 65535 && num_heads_k <= 65535, "fwd_kvcache: batch and num_heads_k must not exceed 65535");
+    IV2_CHECK(q && kcache && vcache && out && softmax_lse, "fwd_kvcache: null pointer");
+    IV2_CHECK((k_new == nullptr) == (v_new == nullptr), "fwd_kvcache: k and v must be given together");
+    IV2_CHECK(k_new == nullptr || seqlen_new > 0, "fwd_kvcache: new keys given with seqlen_new == 0");
+    IV2_CHECK(blockmask == nullptr || n_uint64_per_row > 0, "fwd_kvcache: mask given without words per row");
+    IV2_CHECK(softmax_scale > 0.f, "fwd_kvcache: softmax_scale must be positive");
+    IV2_CHECK(num_splits >= 1 && num_splits <= 64, "fwd_kvcache: num_splits must be in [1, 64]");
+    IV2_CHECK(workspace_bytes >= infllmv2_fwd_kvcache_workspace_bytes(batch, num_heads_k, num_splits),
+              "fwd_kvcache: workspace too small");
+    IV2_CHECK(num_splits == 1 || workspace != nullptr, "fwd_kvcache: split decode needs a workspace");
+    const void* aligned16[] = {q, kcache, vcache, out};
+    for (const void* a : aligned16) IV2_CHECK(reinterpret_cast<uintptr_t>(a) % 16 == 0, "fwd_kvcache: tensors must be 16-byte aligned");
+    IV2_CHECK(q_strides[0] % 8 == 0 && q_strides[1] % 8 == 0 && o_strides[0] % 8 == 0 && o_strides[1] % 8 == 0,
+              "fwd_kvcache: q/out strides must be multiples of 8 elements");
+    for (int s = 0; s < 3; ++s)
+        IV2_CHECK(kcache_strides[s] % 8 == 0 && vcache_strides[s] % 8 == 0, "fwd_kvcache: cache strides must be multiples of 8 elements");
+
+    DecodeParams p{};
+    p.q = static_cast<const bf16_bits*>(q);
+    p.kcache = static_cast<bf16_bits*>(kcache);
+    p.vcache = static_cast<bf16_bits*>(vcache);
+    p.knew = static_cast<const bf16_bits*>(k_new);
+    p.vnew = static_cast<const bf16_bits*>(v_new);
+    p.out = static_cast<bf16_bits*>(out);
+    p.lse = softmax_lse;
+    p.cache_seqlens = cache_seqlens;
+    p.mask = blockmask;
+    p.q_batch = q_strides[0]; p.q_head = q_strides[1];
+    p.o_batch = o_strides[0]; p.o_head = o_strides[1];
+    p.kc_batch = kcache_strides[0]; p.kc_row = kcache_strides[1]; p.kc_head = kcache_strides[2];
+    p.vc_batch = vcache_strides[0]; p.vc_row = vcache_strides[1]; p.vc_head = vcache_strides[2];
+    p.batch = batch; p.num_heads_k = num_heads_k; p.capacity = cache_capacity;
+    p.seqlen_new = k_new ? seqlen_new : 0;
+    p.n64 = n_uint64_per_row; p.splits = num_splits;
+    p.scale_log2 = softmax_scale * 1.44269504088896340736f;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (k_new != nullptr) {
+        IV2_CHECK(reinterpret_cast<uintptr_t>(k_new) % 16 == 0 && reinterpret_cast<uintptr_t>(v_new) % 16 == 0,
+                  "fwd_kvcache: new k/v must be 16-byte aligned");
+        for (int s = 0; s < 3; ++s)
+            IV2_CHECK(knew_strides[s] % 8 == 0 && vnew_strides[s] % 8 == 0, "fwd_kvcache: new k/v strides must be multiples of 8 elements");
+        p.kn_batch = knew_strides[0]; p.kn_row = knew_strides[1]; p.kn_head = knew_strides[2];
+        p.vn_batch = vnew_strides[0]; p.vn_row = vnew_strides[1]; p.vn_head = vnew_strides[2];
+        const int64_t total = static_cast<int64_t>(batch) * seqlen_new * num_heads_k * 16;
+        hipLaunchKernelGGL(decode_append_kernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, st, p);
+        IV2_LAUNCH_CHECK();
+    }
+    const dim3 grid(num_splits, num_heads_k, batch);
+    if (num_splits == 1) {
+        hipLaunchKernelGGL(decode_split_kernel<true>, grid, dim3(64), 0, st, p);
+        IV2_LAUNCH_CHECK();
+    } else {
+        float* ws = static_cast<float*>(workspace);
+        p.o_part = ws;
+        p.lse_part = ws + static_cast<size_t>(batch) * num_heads_k * num_splits * 16 * kHeadDim;
+        hipLaunchKernelGGL(decode_split_kernel<false>, grid, dim3(64), 0, st, p);
+        IV2_LAUNCH_CHECK();
+        hipLaunchKernelGGL(decode_combine_kernel, dim3(num_heads_k, batch), dim3(256), 0, st, p);
+        IV2_LAUNCH_CHECK();
+    }
+    return 0;
+}
