@@ -1,0 +1,95 @@
+"""The mirror of the reference's native module (`infllm_v2.C`) called the way the reference's own Python
+wrappers call it (infllm_v2/infllmv2_sparse_attention.py:71-130, 174-263, 551-589, max_pooling_1d.py:25-41,
+topk_to_uint64.py:60-68): re-laid-out (T*16, Hk, d) queries, cu_seqlens * 16, transposed column mask for
+the backward.  Results must equal those of the package operators, which run the same kernels in place."""
+import numpy as np
+import pytest
+import torch
+
+from test_gpu_stage2_fwd import make_case
+
+pytestmark = pytest.mark.gpu
+
+
+def expand(x, Hk):           # (T, Hq, d) -> (T*16, Hk, d), as infllmv2_sparse_attention.py:88
+    T, Hq, d = x.shape
+    return x.reshape(T, Hk, 16, d).transpose(1, 2).reshape(T * 16, Hk, d).contiguous()
+
+
+def collapse(x, Hk):         # inverse, as infllmv2_sparse_attention.py:130
+    T16, _, d = x.shape
+    return x.reshape(T16 // 16, 16, Hk, d).transpose(1, 2).reshape(T16 // 16, Hk * 16, d).contiguous()
+
+
+def test_reference_style_forward_backward_through_C():
+    import infllm_v2
+    from infllm_v2 import C
+    dev = torch.device("cuda:0")
+    sq = [300, 200]
+    q, k, v, cu_q, cu_k, idx = make_case(21, sq, sq, 2, 3, dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    # topk_to_uint64 through raw pointers (topk_to_uint64.py:56-68)
+    k_blocks, n64 = (max(sq) + 63) // 64, 1
+    words = torch.zeros((2, q.shape[0], n64), dtype=torch.int64, device=dev)
+    C.topk_to_uint64(stream, idx.data_ptr(), words.data_ptr(), 2 * q.shape[0], idx.shape[-1], k_blocks, n64)
+    ref_words, _ = infllm_v2.topk_to_uint64(idx, max(sq), 64)
+    assert torch.equal(words, ref_words)
+    # forward (infllmv2_sparse_attention.py:97-130)
+    qe = expand(q, 2)
+    out_e, lse, p, rng = C.varlen_fwd(qe, k, v, None, cu_q * 16, cu_k, None, None, None, None, max(sq) * 16, max(sq), 0.0,
+                                      128 ** -0.5, False, True, -1, -1, 0.0, False, None, words)
+    out_ref, lse_ref, _ = infllm_v2.infllmv2_attn_varlen_func(q, k, v, cu_q, cu_k, max(sq), max(sq), causal=True,
+                                                            topk_idx=idx, return_attn_probs=True)
+    assert torch.equal(collapse(out_e, 2), out_ref) and torch.equal(lse, lse_ref) and p.numel() == 0
+    # backward with the transposed mask (infllmv2_sparse_attention.py:344-350, 217-243)
+    col_mask = infllm_v2.blockmask_to_uint64(infllm_v2.uint64_to_bool(words, k_blocks).transpose(1, 2).contiguous())[0]
+    dout = torch.randn_like(q)
+    dq_e, dk, dv = torch.empty_like(qe), torch.empty_like(k), torch.empty_like(v)
+    res = C.varlen_bwd(expand(dout, 2), qe, k, v, out_e, lse, dq_e, dk, dv, cu_q * 16, cu_k, None, max(sq) * 16, max(sq),
+                       0.0, 128 ** -0.5, False, True, -1, -1, 0.0, False, col_mask, None, rng)
+    assert len(res) == 4
+    qg, kg, vg = [t.clone().requires_grad_(True) for t in (q, k, v)]
+    infllm_v2.infllmv2_attn_varlen_func(qg, kg, vg, cu_q, cu_k, max(sq), max(sq), causal=True, topk_idx=idx).backward(dout)
+    assert torch.equal(collapse(dq_e, 2), qg.grad)
+    assert (dk.float() - kg.grad.float()).abs().max() <= 0.07 and (dv.float() - vg.grad.float()).abs().max() <= 0.13  # fp32 atomics order
+
+
+def test_reference_style_stage1_and_pooling_through_C():
+    import infllm_v2
+    from infllm_v2 import C
+    dev = torch.device("cuda:0")
+    S = 640
+    g = torch.Generator(device="cpu").manual_seed(5)
+    q = torch.randn(S, 32, 128, generator=g).to(torch.bfloat16).to(dev)
+    kf = torch.randn((S - 32) // 16 + 1, 2, 128, generator=g).to(torch.bfloat16).to(dev)
+    kc = torch.randn((S - 128) // 64 + 1, 2, 128, generator=g).to(torch.bfloat16).to(dev)
+    mk = lambda n: torch.tensor([0, n], dtype=torch.int32, device=dev)
+    Lk = kf.shape[0]
+    res = C.varlen_fwd_stage1(expand(q, 2), kf, kc, None, mk(S) * 16, mk(Lk), mk(kc.shape[0]), None, None, None, None,
+                              S * 16, Lk, 0.0, 128 ** -0.5, True, True, -1, -1, 0.0, True, None)
+    p = res[0]
+    assert tuple(p.shape) == (2, S, 128) and float(p[:, :, Lk:].abs().max()) == 0.0
+    score = infllm_v2.infllmv2_attn_stage1(q, kf, kc, mk(S), mk(Lk), mk(kc.shape[0]), S, Lk, causal=True)
+    assert torch.equal(p[:, :, :Lk], score)
+    # max_pooling_1d through raw pointers (max_pooling_1d.py:25-41)
+    x = score.contiguous()
+    out_len = (S + 63) // 64
+    pooled = torch.zeros(2, S, out_len, dtype=x.dtype, device=dev)
+    C.max_pooling_1d(torch.cuda.current_stream().cuda_stream, x.data_ptr(), pooled.data_ptr(), True, 2, S, Lk, out_len,
+                     0, 5, 4, 1, 64, 1, 1)
+    assert torch.equal(pooled, infllm_v2.max_pooling_1d(score, 0, 1, 1))
+    # varlen variant with its host read-back of total_q
+    pooled_v = torch.zeros_like(pooled)
+    zeros = torch.zeros(1, dtype=torch.int32, device=dev)
+    C.max_pooling_1d_varlen(torch.cuda.current_stream().cuda_stream, x.data_ptr(), pooled_v.data_ptr(), mk(S).data_ptr(),
+                            mk(Lk).data_ptr(), zeros.data_ptr(), True, 1, 2, S, Lk, out_len, 5, 4, 1, 64, 1, 1)
+    assert torch.equal(pooled_v, pooled)
+    # the reference's own top-k binding: values and positions, row stride = next power of two
+    val = torch.zeros(2 * S, 16, dtype=x.dtype, device=dev)
+    pos = torch.zeros(2 * S, 16, dtype=torch.int32, device=dev)
+    C.topk(torch.cuda.current_stream().cuda_stream, 2 * S, out_len, 10, 1, pooled.data_ptr(), val.data_ptr(), pos.data_ptr())
+    ref_idx = infllm_v2.topk_blocks(pooled, 10).reshape(2 * S, 10)
+    assert torch.equal(pos[:, :10], ref_idx)
+    assert torch.equal(val[:, :10], torch.gather(pooled.reshape(2 * S, out_len), 1, ref_idx.long()))
+    with pytest.raises(NotImplementedError):
+        C.fwd()
