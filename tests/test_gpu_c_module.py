@@ -81,8 +81,9 @@ def test_reference_style_stage1_and_pooling_through_C():
     # varlen variant with its host read-back of total_q
     pooled_v = torch.zeros_like(pooled)
     zeros = torch.zeros(1, dtype=torch.int32, device=dev)
-    C.max_pooling_1d_varlen(torch.cuda.current_stream().cuda_stream, x.data_ptr(), pooled_v.data_ptr(), mk(S).data_ptr(),
-                            mk(Lk).data_ptr(), zeros.data_ptr(), True, 1, 2, S, Lk, out_len, 5, 4, 1, 64, 1, 1)
+    cu_q_t, cu_k_t = mk(S), mk(Lk)                          # keep the tensors alive: only raw pointers are passed
+    C.max_pooling_1d_varlen(torch.cuda.current_stream().cuda_stream, x.data_ptr(), pooled_v.data_ptr(), cu_q_t.data_ptr(),
+                            cu_k_t.data_ptr(), zeros.data_ptr(), True, 1, 2, S, Lk, out_len, 5, 4, 1, 64, 1, 1)
     assert torch.equal(pooled_v, pooled)
     # the reference's own top-k binding: values and positions, row stride = next power of two
     val = torch.zeros(2 * S, 16, dtype=x.dtype, device=dev)

@@ -1,0 +1,182 @@
+"""BASELINE-size runs checked through sampled rows and size-independent properties.
+
+Config 2 (prefill, 32768 tokens) end to end; config 3 (four packed sequences, ~64K tokens, forward +
+backward); config 5 (decode, batch 64, cache lengths up to 131072).  Oracle parity on sampled rows; for
+the rest: forced blocks always selected, popcount == k, sum_keys dV = sum_tokens dO and sum_keys dK = 0
+(rows of P sum to one, rows of dS sum to zero)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import infllmv2_oracle as O
+from conftest import bf16_np, words_np
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import infllmv2_cuda_impl_amd as ops
+    return ops
+
+
+def compress(k, kernel, stride):
+    return k.unfold(0, kernel, stride).float().mean(-1).to(torch.bfloat16).contiguous()
+
+
+def token_oracle(q, k, v, words_row, t_local, Sq, Sk, tok_global, dout=None):
+    """Oracle forward (and dQ) of one token: a one-query problem against its visible prefix."""
+    pos = t_local + Sk - Sq
+    kk, vv = bf16_np(k[:pos + 1]), bf16_np(v[:pos + 1])
+    qq = bf16_np(q[tok_global:tok_global + 1])
+    w = words_row[:, None, :]                               # (Hk, 1, n64)
+    o, lse = O.stage2_forward(qq, kk, vv, [0, 1], [0, pos + 1], w, 128 ** -0.5, True)
+    if dout is None:
+        return o[0], None
+    dq, _, _ = O.stage2_backward(qq, kk, vv, bf16_np(dout[tok_global:tok_global + 1]), [0, 1], [0, pos + 1], w,
+                                 128 ** -0.5, True)
+    return o[0], dq[0]
+
+
+def test_config2_prefill_32k(ops):
+    dev = torch.device("cuda:0")
+    S, topk = 32768, 64
+    g = torch.Generator(device="cpu").manual_seed(0)
+    q = torch.randn(S, 32, 128, generator=g).to(torch.bfloat16).to(dev)
+    k = torch.randn(S, 2, 128, generator=g).to(torch.bfloat16).to(dev)
+    v = torch.randn(S, 2, 128, generator=g).to(torch.bfloat16).to(dev)
+    kf, kc = compress(k, 32, 16), compress(k, 128, 64)
+    mk = lambda n: torch.tensor([0, n], dtype=torch.int32, device=dev)
+    Lk = kf.shape[0]
+    score = ops.infllmv2_attn_stage1(q, kf, kc, mk(S), mk(Lk), mk(kc.shape[0]), S, Lk, causal=True)
+    pooled = ops.max_pooling_1d(score, 0, 31, 1)
+    idx = ops.topk_blocks(pooled, topk)
+    words, kb = ops.topk_to_uint64(idx, S, 64)
+    out = ops.infllmv2_attn_varlen_func(q, k, v, mk(S), mk(S), S, S, causal=True, topk_idx=idx)
+    rows = [0, 1, 63, 64, 127, 128, 2047, 2048, 4095, 4096, 10000, 20001, 32767]
+    # Stage 1 on sampled rows (one-row oracle problems: q_len < k_len uses the offset rule, so feed whole prefix lengths)
+    sc = bf16_np(score[:, rows])
+    # pooled / top-k / mask are bit-exact functions of the GPU score rows
+    full_pool = O.max_pooling_1d_fast(sc, (S + 63) // 64, 31, 1, row_cache_lens=np.zeros(len(rows), dtype=np.int64),
+                                      row_qidx=np.array(rows), row_klen=np.full(len(rows), Lk))
+    assert np.array_equal(bf16_np(pooled[:, rows]), full_pool)
+    ref_idx = O.topk_blocks(full_pool, topk)
+    assert np.array_equal(idx[:, rows].cpu().numpy(), ref_idx)
+    assert np.array_equal(words_np(words[:, rows]), O.topk_to_uint64(ref_idx, S, 64)[0])
+    # selection invariants over all rows
+    bits = ops.uint64_to_bool(words, kb)
+    tok = torch.arange(S, device=dev)
+    bq = tok // 64
+    assert bool(bits[:, :, 0].all())
+    assert bool((bits.sum(-1) == topk).all())
+    for d in (0, 1, 15, 31):
+        sel = bits[:, tok, torch.clamp(bq - d, min=0)]
+        assert bool(sel.all())
+    # Stage-1 parity on sampled rows against the oracle (exact prefix semantics: Sq == Sk for the full problem)
+    kf_np, kc_np = bf16_np(kf), bf16_np(kc)
+    for r in rows[::3]:
+        vf = O.stage1_visible(r, 16, Lk, S, True)
+        vc = O.stage1_visible(r, 64, kc.shape[0], S, True)
+        got = bf16_np(score[:, r])
+        if vc == 0:
+            assert np.all(got == 0)
+            continue
+        qq = bf16_np(q[r]).reshape(2, 16, 128).astype(np.float64)
+        for h in range(2):
+            sc_c = qq[h] @ kc_np[:vc, h].astype(np.float64).T * 128 ** -0.5
+            lse = np.log(np.exp(sc_c - sc_c.max(-1, keepdims=True)).sum(-1, keepdims=True)) + sc_c.max(-1, keepdims=True)
+            ref = np.exp(qq[h] @ kf_np[:vf, h].astype(np.float64).T * 128 ** -0.5 - lse).sum(0)
+            assert (np.abs(got[h, :vf] - ref) <= 2.0 ** -7 * np.abs(ref) + 2e-3).all()
+            assert np.all(got[h, vf:] == 0)
+    # Stage-2 forward on sampled tokens
+    wnp = words_np(words)
+    for r in rows:
+        o_ref, _ = token_oracle(q, k, v, wnp[:, r], r, S, S, r)
+        err = np.abs(bf16_np(out[r]) - o_ref)
+        assert err.max() <= 2e-2 and err.mean() <= 1e-3, (r, err.max(), err.mean())
+
+
+def test_config3_varlen_fwd_bwd_64k(ops):
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(1)
+    lens = [int(64 * x) for x in rng.integers(64, 385, size=4)]
+    T = sum(lens)
+    cu = torch.tensor(np.cumsum([0] + lens), dtype=torch.int32, device=dev)
+    g = torch.Generator(device="cpu").manual_seed(0)
+    q = torch.randn(T, 32, 128, generator=g).to(torch.bfloat16).to(dev)
+    k = torch.randn(T, 2, 128, generator=g).to(torch.bfloat16).to(dev)
+    v = torch.randn(T, 2, 128, generator=g).to(torch.bfloat16).to(dev)
+    dout = torch.randn(T, 32, 128, generator=g).to(torch.bfloat16).to(dev)
+    # top-k from random pooled scores with forced blocks (selection itself is covered by config 2)
+    nblk = max(lens) // 64
+    pooled = torch.rand(2, T, nblk, device=dev).to(torch.bfloat16)
+    cu_l = cu.cpu().numpy()
+    for b in range(4):
+        i = torch.arange(lens[b], device=dev)
+        blk = torch.arange(nblk, device=dev)[None, :]
+        bqv = (i // 64)[:, None]
+        forced = (blk < 1) | ((bqv >= blk) & (bqv <= blk + 31))
+        future = blk > bqv
+        seg = pooled[:, cu_l[b]:cu_l[b + 1]]
+        seg[:, forced] = float("inf")
+        seg[:, future & ~forced] = float("-inf")
+    idx = ops.topk_blocks(pooled, 64)
+    idx = torch.where(torch.gather(pooled, 2, idx.long().clamp(min=0)) == float("-inf"), torch.full_like(idx, -1), idx)
+    qg, kg, vg = [t.clone().requires_grad_(True) for t in (q, k, v)]
+    out = ops.infllmv2_attn_varlen_func(qg, kg, vg, cu, cu, max(lens), max(lens), causal=True, topk_idx=idx)
+    out.backward(dout)
+    words = words_np(ops.topk_to_uint64(idx, max(lens), 64)[0])
+    # sampled tokens: forward and dQ against the oracle
+    for b, t_local in [(0, 0), (0, lens[0] - 1), (1, 5000 % lens[1]), (2, 64), (3, lens[3] - 1), (3, 2049 % lens[3])]:
+        t = int(cu_l[b]) + t_local
+        kb_, vb_ = k[cu_l[b]:cu_l[b + 1]], v[cu_l[b]:cu_l[b + 1]]
+        o_ref, dq_ref = token_oracle(q, kb_, vb_, words[:, t], t_local, lens[b], lens[b], t, dout)
+        err = np.abs(bf16_np(out[t]) - o_ref)
+        assert err.max() <= 2e-2 and err.mean() <= 1e-3
+        s = max(1.0, float(np.abs(dq_ref).max()))
+        e2 = np.abs(bf16_np(qg.grad[t]) - dq_ref)
+        assert e2.max() <= 2e-2 * s and e2.mean() <= 1e-3 * s
+    # size-independent identities per sequence and KV head
+    for b in range(4):
+        sl = slice(int(cu_l[b]), int(cu_l[b + 1]))
+        dv_sum = vg.grad[sl].float().sum(0)                                   # (Hk, d)
+        do_sum = dout[sl].float().reshape(-1, 2, 16, 128).sum((0, 2))          # every token attends block 0, so rows of P sum to 1
+        scale = float(dout[sl].float().abs().sum(0).max())
+        assert float((dv_sum - do_sum).abs().max()) <= 2e-3 * scale
+        dk_sum = kg.grad[sl].float().sum(0)
+        dk_scale = float(kg.grad[sl].float().abs().sum(0).max())
+        assert float(dk_sum.abs().max()) <= 2e-2 * dk_scale
+    assert bool(torch.isfinite(qg.grad.float()).all() and torch.isfinite(kg.grad.float()).all())
+
+
+def test_config5_decode_batch64(ops):
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(1)
+    B = 64
+    lens = [int(64 * x) for x in rng.integers(256, 2049, size=B)]
+    cap = max(lens)
+    g = torch.Generator(device="cuda").manual_seed(0)
+    q = torch.randn(B, 1, 32, 128, generator=g, device=dev).to(torch.bfloat16)
+    kc = torch.randn(B, cap, 2, 128, generator=g, device=dev).to(torch.bfloat16)
+    vc = torch.randn(B, cap, 2, 128, generator=g, device=dev).to(torch.bfloat16)
+    idx = torch.full((B, 2, 1, 64), -1, dtype=torch.int32)
+    cg = torch.Generator(device="cpu").manual_seed(2)
+    for b in range(B):
+        nb = lens[b] // 64
+        for h in range(2):
+            forced = torch.cat([torch.tensor([0]), torch.arange(nb - 32, nb)])
+            rest = torch.tensor(sorted(set(range(1, nb - 32))))
+            pick = rest[torch.randperm(len(rest), generator=cg)[:31]]
+            idx[b, h, 0] = torch.cat([forced, pick]).sort().values.to(torch.int32)
+    L = torch.tensor(lens, dtype=torch.int32, device=dev)
+    out, lse = ops.infllmv2_attn_with_kvcache(q, kc, vc, cache_seqlens=L, topk_idx=idx.to(dev), return_softmax_lse=True)
+    for b in (0, 17, 63):
+        words = O.topk_to_uint64(idx[b:b + 1].numpy(), cap, 64)[0]
+        ro, rl = O.decode_forward(bf16_np(q[b:b + 1]), bf16_np(kc[b:b + 1, :lens[b]]), bf16_np(vc[b:b + 1, :lens[b]]),
+                                  [lens[b]], words, 128 ** -0.5)
+        err = np.abs(bf16_np(out[b:b + 1]) - ro)
+        assert err.max() <= 2e-2 and err.mean() <= 1e-3
+        assert np.abs(lse[b:b + 1].cpu().numpy() - rl).max() <= 2e-3
+    # split-count independence at full size
+    out1 = ops.infllmv2_attn_with_kvcache(q, kc, vc, cache_seqlens=L, topk_idx=idx.to(dev), num_splits=1)
+    assert float((out.float() - out1.float()).abs().max()) <= 8e-3
