@@ -37,6 +37,8 @@ def parse_args():
     ap.add_argument("--topk", type=int, default=64)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-stages", action="store_true", help="skip the per-stage and kernel-only timings")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run three plain 1 GiB device copies (a kernel of known traffic for scaling rocprofv3 --pmc counters)")
     return ap.parse_args()
 
 
@@ -63,6 +65,33 @@ def event_ms(torch, fn, iters, warmup=2):
     e1.record()
     torch.cuda.synchronize()
     return e0.elapsed_time(e1) / iters
+
+
+def decode_bench(torch, ops, dev):
+    """BASELINE config 5: batch 64, one query token, cache lengths 64*U[256,2048], topk 64 (1 init + 32 local forced)."""
+    import numpy as np
+    rng = np.random.default_rng(1)
+    B = 64
+    lens = [int(64 * x) for x in rng.integers(256, 2049, size=B)]
+    cap = max(lens)
+    g = torch.Generator(device="cuda").manual_seed(0)
+    q = torch.randn(B, 1, 32, 128, generator=g, device=dev).to(torch.bfloat16)
+    kc = torch.randn(B, cap, 2, 128, generator=g, device=dev).to(torch.bfloat16)
+    vc = torch.randn(B, cap, 2, 128, generator=g, device=dev).to(torch.bfloat16)
+    idx = torch.full((B, 2, 1, 64), -1, dtype=torch.int32)
+    cg = torch.Generator(device="cpu").manual_seed(2)
+    for b in range(B):
+        nb = lens[b] // 64
+        for h in range(2):
+            rest = torch.arange(1, nb - 32)
+            pick = rest[torch.randperm(len(rest), generator=cg)[:31]]
+            idx[b, h, 0] = torch.cat([torch.tensor([0]), torch.arange(nb - 32, nb), pick]).sort().values.to(torch.int32)
+    idx = idx.to(dev)
+    L = torch.tensor(lens, dtype=torch.int32, device=dev)
+    ms = event_ms(torch, lambda: ops.infllmv2_attn_with_kvcache(q, kc, vc, cache_seqlens=L, topk_idx=idx), 20)
+    bytes_ = B * 2 * 64 * 64 * 128 * 2 * 2 + 2 * B * 32 * 128 * 2
+    return {"ms": ms, "algorithmic_bytes": bytes_, "hbm_gbs": bytes_ / ms / 1e6, "frac_hbm_peak": bytes_ / ms / 1e6 / PEAK_HBM_GBS,
+            "workload": "BASELINE config 5: batch 64, seqlen_q 1, cache lengths 64*U[256,2048], topk 64, Stage-2 decode incl. mask packing"}
 
 
 def cpu_baseline():
@@ -214,6 +243,15 @@ def main():
             result["stage2_fwd_bwd_frac_peak"] = 3.5 * fwd_flops / fb_ms / 1e9 / PEAK_BF16_TFLOPS
         except ImportError:
             pass
+
+    if not args.no_stages:
+        result["decode_config5"] = decode_bench(torch, ops, dev)
+    if args.calibrate_copy:
+        src = torch.ones(1 << 30, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
 
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline()
