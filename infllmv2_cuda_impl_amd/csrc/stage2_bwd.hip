@@ -12,9 +12,9 @@
 //     the token's mask row); S and dP are recomputed, dQ stays in registers and is written once
 //     as bf16.  No dq scratch, no zero fill, no conversion pass, bit-reproducible.
 //   * dK/dV: column-parallel.  A workgroup owns one 64-key block and a slice of 2048 query
-//     tokens; it walks the transposed mask, keeps the full 64x128 dK^T and dV^T tiles in
-//     accumulator registers of each wavefront (the four wavefronts take disjoint tokens), reduces
-//     them through LDS and flushes once per slice with fp32 atomics, so atomic traffic is one
+//     tokens; it walks the transposed mask and keeps the 64x128 dK^T and dV^T tiles in accumulator
+//     registers (8 wavefronts = 4 disjoint token streams x 2 key halves), reduces the streams
+//     through LDS and flushes once per slice with fp32 atomics, so atomic traffic is one
 //     64 KiB tile per >= 100 tokens instead of 8 KiB per (token, block).  Slicing bounds the work
 //     of a workgroup: block 0 and the local window are selected by every token.
 //   * S = Q K^T is formed with the 16 heads of a token as MFMA rows; two tokens fill the 32-deep
@@ -201,15 +201,18 @@ void bwd_dq_kernel(const BwdParams p) {
 constexpr int kRedPitch = 65;                                  // floats per d row of the LDS reduction tile
 
 template <bool kCausal>
-__global__ __launch_bounds__(256)
+__global__ __launch_bounds__(512)
 void bwd_dkdv_kernel(const BwdParams p) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     uint4* ldsK = reinterpret_cast<uint4*>(smem_raw);          // 1024 units: K image
     uint4* ldsV = ldsK + 1024;                                 // 1024 units: V in K-image order
     float* red = reinterpret_cast<float*>(smem_raw);           // reused after the main loop: [128][65]
 
+    // 8 wavefronts = 4 token streams x 2 key halves: a wavefront owns 32 of the block's 64 keys, so
+    // its dK^T / dV^T accumulators are 128 registers and two wavefronts fit on a SIMD.
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
+    const int kh = wave & 1, ts = wave >> 1;
     const int n = lane & 15, g = lane >> 4;
     const int j = blockIdx.x / p.n_slices;                     // key block inside the sequence
     const int slice = blockIdx.x - j * p.n_slices;
@@ -233,15 +236,15 @@ void bwd_dkdv_kernel(const BwdParams p) {
         const uint4* ks = reinterpret_cast<const uint4*>(p.kimg + img);
         const uint4* vs = reinterpret_cast<const uint4*>(p.vimg_r + img);
 #pragma unroll
-        for (int u = tid; u < 1024; u += 256) { ldsK[u] = ks[u]; ldsV[u] = vs[u]; }
+        for (int u = tid; u < 1024; u += 512) { ldsK[u] = ks[u]; ldsV[u] = vs[u]; }
     }
     __syncthreads();
 
-    floatx4 dKt[8][4], dVt[8][4];                              // [d tile][key tile]: lane (n, g) holds [16dt+4g+e][16kt+n]
+    floatx4 dKt[8][2], dVt[8][2];                              // [d tile][local key tile]: lane (n, g) holds [16dt+4g+e][16(2kh+kt)+n]
 #pragma unroll
     for (int dt = 0; dt < 8; ++dt)
 #pragma unroll
-        for (int kt = 0; kt < 4; ++kt) {
+        for (int kt = 0; kt < 2; ++kt) {
             dKt[dt][kt] = floatx4{0.f, 0.f, 0.f, 0.f};
             dVt[dt][kt] = floatx4{0.f, 0.f, 0.f, 0.f};
         }
@@ -250,8 +253,10 @@ void bwd_dkdv_kernel(const BwdParams p) {
     const int w_lo = static_cast<int>(t_lo >> 6), w_hi = static_cast<int>((t_hi - 1) >> 6);
     const uint64_t* mrow = p.bwd_mask ? p.bwd_mask + (static_cast<int64_t>(h) * p.k_blocks + j) * p.n64_bwd : nullptr;
     const int64_t head_tok0 = static_cast<int64_t>(h) * p.total_q;
+    const uint4* myK = ldsK + (2 * kh) * 4 * 64 + lane;
+    const uint4* myV = ldsV + (2 * kh) * 4 * 64 + lane;
 
-    for (int w = w_lo + wave; w <= w_hi; w += 4) {
+    for (int w = w_lo + ts; w <= w_hi; w += 4) {
         uint64_t bits = mrow ? mrow[w] : ~0ull;
         const int64_t base = static_cast<int64_t>(w) << 6;
         if (base < t_lo) bits &= ~0ull << (t_lo - base);
@@ -289,8 +294,8 @@ void bwd_dkdv_kernel(const BwdParams p) {
                 }
                 if (!has_b) lim_b = -1;
             }
-            // phase 1: P = exp2(scale*S - lse) for both tokens (fp32, kept for dS)
-            float pa[4][4], pb[4][4];
+            // phase 1: P = exp2(scale*S - lse) for both tokens on this wavefront's 32 keys (fp32, kept for dS)
+            float pa[2][4], pb[2][4];
             {
                 bf16x8 qa[4], qb[4];
                 const bf16_bits* ptr_a = p.q + ta * p.q_tok + h * p.q_kvh + n * p.q_grp + 8 * g;
@@ -301,17 +306,17 @@ void bwd_dkdv_kernel(const BwdParams p) {
                     qb[c] = *reinterpret_cast<const bf16x8*>(ptr_b + 32 * c);
                 }
 #pragma unroll
-                for (int kt = 0; kt < 4; ++kt) {
+                for (int kt = 0; kt < 2; ++kt) {
                     floatx4 sa = floatx4{0.f, 0.f, 0.f, 0.f}, sb = sa;
 #pragma unroll
                     for (int c = 0; c < 4; ++c) {
-                        const uint4 kraw = ldsK[(kt * 4 + c) * 64 + lane];
+                        const uint4 kraw = myK[(kt * 4 + c) * 64];
                         bf16x8 kf;
                         __builtin_memcpy(&kf, &kraw, 16);
                         sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa[c], kf, sa, 0, 0, 0);
                         sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qb[c], kf, sb, 0, 0, 0);
                     }
-                    const int key = 16 * kt + n;
+                    const int key = 16 * (2 * kh + kt) + n;
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         const float xa = __builtin_amdgcn_exp2f(sa[e] * p.scale_log2 - lse_a[e]);
@@ -322,7 +327,7 @@ void bwd_dkdv_kernel(const BwdParams p) {
                 }
             }
             // phase 2: dP = dO V^T, dS = P * (dP - D); both packed to bf16 as B operands
-            bf16x8 pfr[4], dsfr[4];
+            bf16x8 pfr[2], dsfr[2];
             {
                 bf16x8 doa[4], dob[4];
                 const bf16_bits* ptr_a = p.dout + ta * p.do_tok + h * p.do_kvh + n * p.do_grp + 8 * g;
@@ -333,11 +338,11 @@ void bwd_dkdv_kernel(const BwdParams p) {
                     dob[c] = *reinterpret_cast<const bf16x8*>(ptr_b + 32 * c);
                 }
 #pragma unroll
-                for (int kt = 0; kt < 4; ++kt) {
+                for (int kt = 0; kt < 2; ++kt) {
                     floatx4 dpa = floatx4{0.f, 0.f, 0.f, 0.f}, dpb = dpa;
 #pragma unroll
                     for (int c = 0; c < 4; ++c) {
-                        const uint4 vraw = ldsV[(kt * 4 + c) * 64 + lane];
+                        const uint4 vraw = myV[(kt * 4 + c) * 64];
                         bf16x8 vf;
                         __builtin_memcpy(&vf, &vraw, 16);
                         dpa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(doa[c], vf, dpa, 0, 0, 0);
@@ -352,6 +357,7 @@ void bwd_dkdv_kernel(const BwdParams p) {
                     }
                 }
             }
+            __builtin_amdgcn_sched_barrier(0);
             const bf16_bits* qTa = p.qT + (head_tok0 + ta) * kTImageElems + lane * 4;
             const bf16_bits* qTb = p.qT + (head_tok0 + tb) * kTImageElems + lane * 4;
             const bf16_bits* dTa = p.doT + (head_tok0 + ta) * kTImageElems + lane * 4;
@@ -368,7 +374,7 @@ void bwd_dkdv_kernel(const BwdParams p) {
                 __builtin_memcpy(&aq, &aq_raw, 16);
                 __builtin_memcpy(&ad, &ad_raw, 16);
 #pragma unroll
-                for (int kt = 0; kt < 4; ++kt) {
+                for (int kt = 0; kt < 2; ++kt) {
                     dVt[dt][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ad, pfr[kt], dVt[dt][kt], 0, 0, 0);
                     dKt[dt][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aq, dsfr[kt], dKt[dt][kt], 0, 0, 0);
                 }
@@ -376,21 +382,21 @@ void bwd_dkdv_kernel(const BwdParams p) {
         }
     }
 
-    // reduce the four wavefronts' tiles through LDS (dK then dV), one atomic flush per workgroup and tensor
+    // reduce the four token streams through LDS (dK then dV), one atomic flush per workgroup and tensor
     const int valid_keys = (Sk - j * kBlockN) < kBlockN ? (Sk - j * kBlockN) : kBlockN;
     const int64_t row0 = static_cast<int64_t>(k0) + static_cast<int64_t>(j) * kBlockN;
 #pragma unroll
     for (int which = 0; which < 2; ++which) {
         __syncthreads();                                       // LDS free: images consumed / previous flush done
         for (int r = 0; r < 4; ++r) {
-            if (wave == r) {
+            if (ts == r) {
 #pragma unroll
                 for (int dt = 0; dt < 8; ++dt)
 #pragma unroll
-                    for (int kt = 0; kt < 4; ++kt)
+                    for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
-                            const int idx = (16 * dt + 4 * g + e) * kRedPitch + 16 * kt + n;
+                            const int idx = (16 * dt + 4 * g + e) * kRedPitch + 16 * (2 * kh + kt) + n;
                             const float val = which == 0 ? dKt[dt][kt][e] : dVt[dt][kt][e];
                             if (r == 0) red[idx] = val; else red[idx] += val;
                         }
@@ -399,7 +405,7 @@ void bwd_dkdv_kernel(const BwdParams p) {
         }
         float* acc = which == 0 ? p.dk_acc : p.dv_acc;
         const float mul = which == 0 ? p.scale : 1.f;
-        for (int idx = tid; idx < kBlockN * kHeadDim; idx += 256) {
+        for (int idx = tid; idx < kBlockN * kHeadDim; idx += 512) {
             const int key = idx >> 7, d = idx & 127;
             if (key < valid_keys)
                 unsafeAtomicAdd(acc + ((row0 + key) * p.num_heads_k + h) * kHeadDim + d, red[d * kRedPitch + key] * mul);
@@ -559,8 +565,8 @@ extern "C" int infllmv2_varlen_bwd(void* stream, const void* dout, const void* q
         IV2_LAUNCH_CHECK();
         const size_t lds = kHeadDim * kRedPitch * sizeof(float);          // 33280 B >= the 32 KiB of staged images
         const dim3 gk(static_cast<unsigned>(p.k_blocks) * p.n_slices, batch, num_heads_k);
-        if (is_causal) hipLaunchKernelGGL(bwd_dkdv_kernel<true>, gk, dim3(256), lds, st, p);
-        else hipLaunchKernelGGL(bwd_dkdv_kernel<false>, gk, dim3(256), lds, st, p);
+        if (is_causal) hipLaunchKernelGGL(bwd_dkdv_kernel<true>, gk, dim3(512), lds, st, p);
+        else hipLaunchKernelGGL(bwd_dkdv_kernel<false>, gk, dim3(512), lds, st, p);
         IV2_LAUNCH_CHECK();
     } else if (total_q > 0) {
         // no keys at all: dq = 0
