@@ -26,6 +26,7 @@
 #include "block_walker.h"
 #include "../../include/infllmv2_hip.h"
 #include <math.h>
+#include <stdlib.h>
 
 namespace infllmv2 {
 
@@ -42,6 +43,9 @@ struct BwdParams {
     float* dsum;                    // (Hk, total_q * 16): D of head 16h+g of token t at [h][16 t + g]
     bf16_bits* qT;                  // (Hk, total_q, 8, 64, 4): lane (r, g) of d-tile dt holds X[heads 4g..4g+3][16 dt + r]
     bf16_bits* doT;
+    bf16_bits* qF;                  // (Hk, total_q, 4, 64, 8): q and dout as ready-made A-operand fragments, lane (r, g) of
+    bf16_bits* doF;                 //   chunk c holds X[head r][32 c + 8 g ..]
+    float* rowstat;                 // (Hk, total_q, 32): LSE * log2(e) of the 16 heads, then D of the 16 heads
     const bf16_bits* kimg;          // K, K-image order
     const bf16_bits* kimg_t;        // K, V-image order
     const bf16_bits* vimg_r;        // V, K-image order
@@ -80,6 +84,12 @@ void bwd_prep_kernel(const BwdParams p) {
     const uint4 ov = *reinterpret_cast<const uint4*>(p.out + tok * p.o_tok + h * p.o_kvh + row * p.o_grp + part * 8);
     *reinterpret_cast<uint4*>(&tq[row][part * 8]) = qv;
     *reinterpret_cast<uint4*>(&tdo[row][part * 8]) = dv;
+    {
+        const int unit = (part >> 2) * 64 + (part & 3) * 16 + row;            // chunk c = part / 4, k-group g = part % 4
+        const int64_t base = (static_cast<int64_t>(h) * p.total_q + tok) * kTImageElems + unit * 8;
+        *reinterpret_cast<uint4*>(p.qF + base) = qv;
+        *reinterpret_cast<uint4*>(p.doF + base) = dv;
+    }
     const uint32_t dw[4] = {dv.x, dv.y, dv.z, dv.w};
     const uint32_t ow[4] = {ov.x, ov.y, ov.z, ov.w};
     float acc = 0.f;
@@ -90,7 +100,12 @@ void bwd_prep_kernel(const BwdParams p) {
     }
 #pragma unroll
     for (int off = 1; off < 16; off <<= 1) acc += __shfl_xor(acc, off);
-    if (part == 0) p.dsum[static_cast<int64_t>(h) * p.total_q * 16 + tok * 16 + row] = acc;
+    if (part == 0) {
+        p.dsum[static_cast<int64_t>(h) * p.total_q * 16 + tok * 16 + row] = acc;
+        float* rs = p.rowstat + (static_cast<int64_t>(h) * p.total_q + tok) * 32;
+        rs[row] = p.lse[h * p.lse_kvh + tok * p.lse_tok + row * p.lse_grp] * kLog2e;
+        rs[16 + row] = acc;
+    }
     __syncthreads();
     bf16_bits* qdst = p.qT + (static_cast<int64_t>(h) * p.total_q + tok) * kTImageElems;
     bf16_bits* ddst = p.doT + (static_cast<int64_t>(h) * p.total_q + tok) * kTImageElems;
@@ -413,6 +428,267 @@ void bwd_dkdv_kernel(const BwdParams p) {
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// dK / dV, streamed variant: same work split (64-key block x 2048-token slice per workgroup) but the
+// workgroup is ONE token stream.  Four wavefronts each own 16 of the block's keys (their K and V
+// operands stay in registers for the whole kernel, their dK^T / dV^T tiles are 64 accumulator
+// registers), and every token pair's operands (q, dout, their transposed images, LSE and D) are
+// copied (flat 1 KiB transfers from fragment-major images the preprocessing kernel wrote) into a
+// 4-stage LDS ring by LDS-DMA loads issued three pairs ahead, so no wavefront
+// ever waits on global-memory latency and no operand passes through registers on its way in.
+// ---------------------------------------------------------------------------------------------
+constexpr int kStages = 4;
+constexpr int kStageBytes = 32768 + 1024;                      // 8 operand tiles of 4 KiB + 4 copies of the pair's 64 scalars
+constexpr int kMaxSliceWords = kSliceTokens / 64 + 1;
+
+__device__ __forceinline__ uint32_t lds_address(const void* ptr) {
+    return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const void*)ptr));
+}
+// LDS-DMA: lane l's 16 (or 4) bytes at its own global address land at lds_base + 16 l (4 l).  Invisible to
+// the compiler's wait-count tracking; ordered by hand with s_waitcnt vmcnt(n) + barrier.
+__device__ __forceinline__ void dma16(const void* src_lane, uint32_t lds_base) {
+    lds_base = __builtin_amdgcn_readfirstlane(lds_base);
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src_lane), "s"(lds_base) : "memory", "m0");
+}
+__device__ __forceinline__ void dma4(const void* src_lane, uint32_t lds_base) {
+    lds_base = __builtin_amdgcn_readfirstlane(lds_base);
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dword %0, off" : : "v"(src_lane), "s"(lds_base) : "memory", "m0");
+}
+
+struct PairCursor {                                            // walks the slice's mask words (in LDS) two tokens at a time
+    const unsigned long long* words;
+    int n_words, w;
+    uint64_t bits;
+    int64_t base0;                                             // packed token index of bit 0 of word 0
+    __device__ __forceinline__ void init(const unsigned long long* wd, int n, int64_t b0) {
+        words = wd; n_words = n; w = -1; bits = 0ull; base0 = b0;
+    }
+    __device__ __forceinline__ bool next(int64_t& ta, int64_t& tb, bool& has_b) {
+        while (bits == 0ull) {
+            if (++w >= n_words) return false;
+            const uint64_t v = words[w];
+            const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
+            const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
+            bits = (static_cast<uint64_t>(hi) << 32) | lo;
+        }
+        const int64_t base = base0 + (static_cast<int64_t>(w) << 6);
+        ta = base + __builtin_ctzll(bits);
+        bits &= bits - 1ull;
+        has_b = bits != 0ull;
+        tb = has_b ? base + __builtin_ctzll(bits) : ta;
+        bits &= bits - 1ull;
+        return true;
+    }
+};
+
+template <bool kCausal>
+__global__ __launch_bounds__(256)
+void bwd_dkdv_stream_kernel(const BwdParams p) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    unsigned char* ring = smem_raw;                                              // kStages * kStageBytes
+    unsigned long long* words = reinterpret_cast<unsigned long long*>(smem_raw + kStages * kStageBytes);
+    float* red = reinterpret_cast<float*>(smem_raw);                             // reused after the main loop: [128][65]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);                   // = key tile (16 keys); scalar, so branches on it are uniform
+    const int n = lane & 15, g = lane >> 4;
+    const int j = blockIdx.x / p.n_slices;
+    const int slice = blockIdx.x - j * p.n_slices;
+    const int b = blockIdx.y, h = blockIdx.z;
+    const int q0 = p.cu_seqlens_q[b];
+    const int Sq = p.cu_seqlens_q[b + 1] - q0;
+    const int k0 = p.cu_seqlens_k[b];
+    const int Sk = p.cu_seqlens_k[b + 1] - k0;
+    if (j * kBlockN >= Sk) return;                                               // uniform per workgroup
+    int i_lo = slice * kSliceTokens;
+    if (kCausal) {
+        const int first = j * kBlockN - (Sk - Sq);
+        if (first > i_lo) i_lo = first;
+    }
+    int i_hi = (slice + 1) * kSliceTokens;
+    if (i_hi > Sq) i_hi = Sq;
+    if (i_lo >= i_hi) return;                                                    // uniform per workgroup
+
+    // this wavefront's K and V operands (B side of S = Q K^T and dP = dO V^T), resident in registers
+    bf16x8 kreg[4], vreg[4];
+    {
+        const int64_t img = (static_cast<int64_t>(h) * p.n_slots + image_slot0(p.cu_seqlens_k, b) + j) * kImageElems;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            kreg[c] = *reinterpret_cast<const bf16x8*>(p.kimg + img + ((wave * 4 + c) * 64 + lane) * 8);
+            vreg[c] = *reinterpret_cast<const bf16x8*>(p.vimg_r + img + ((wave * 4 + c) * 64 + lane) * 8);
+        }
+    }
+    // the slice's mask words, clipped to [t_lo, t_hi), into LDS
+    const int64_t t_lo = static_cast<int64_t>(q0) + i_lo, t_hi = static_cast<int64_t>(q0) + i_hi;
+    const int w_lo = static_cast<int>(t_lo >> 6), w_hi = static_cast<int>((t_hi - 1) >> 6);
+    const int n_words = w_hi - w_lo + 1;                                         // <= kMaxSliceWords
+    const uint64_t* mrow = p.bwd_mask ? p.bwd_mask + (static_cast<int64_t>(h) * p.k_blocks + j) * p.n64_bwd : nullptr;
+    for (int w = tid; w < n_words; w += 256) {
+        uint64_t v = mrow ? mrow[w_lo + w] : ~0ull;
+        const int64_t base = static_cast<int64_t>(w_lo + w) << 6;
+        if (base < t_lo) v &= ~0ull << (t_lo - base);
+        if (base + 64 > t_hi) v &= ~0ull >> (base + 64 - t_hi);
+        words[w] = v;
+    }
+    __syncthreads();
+
+    const int64_t head_tok0 = static_cast<int64_t>(h) * p.total_q;
+    const uint32_t ring_lds = __builtin_amdgcn_readfirstlane(lds_address(ring));
+    // what this wavefront fetches for a pair: wave 0 q, wave 1 dout (both as gathered A-operand fragments),
+    // wave 2 the transposed q image, wave 3 the transposed dout image (flat copies); plus its own scalar copy
+    auto issue = [&](int64_t ta, int64_t tb, int stage) {
+        const uint32_t st = ring_lds + stage * kStageBytes;
+        const bf16_bits* src = wave == 0 ? p.qF : (wave == 1 ? p.doF : (wave == 2 ? p.qT : p.doT));
+        const bf16_bits* pa = src + (head_tok0 + ta) * kTImageElems + lane * 8;
+        const bf16_bits* pb = src + (head_tok0 + tb) * kTImageElems + lane * 8;
+        const uint32_t dst = st + wave * 8192;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            dma16(pa + 512 * c, dst + c * 1024);
+            dma16(pb + 512 * c, dst + 4096 + c * 1024);
+        }
+        // the pair's row statistics: [lse_a (16) | D_a (16) | lse_b (16) | D_b (16)], one private copy per wavefront
+        dma4(p.rowstat + (head_tok0 + (lane < 32 ? ta : tb)) * 32 + (lane & 31), st + 32768 + wave * 256);
+    };
+
+    floatx4 dKt[8], dVt[8];                                                       // lane (n, g): [16 dt + 4 g + e][16 wave + n]
+#pragma unroll
+    for (int dt = 0; dt < 8; ++dt) {
+        dKt[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+        dVt[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    PairCursor fetch_cur, use_cur;
+    fetch_cur.init(words, n_words, static_cast<int64_t>(w_lo) << 6);
+    use_cur.init(words, n_words, static_cast<int64_t>(w_lo) << 6);
+    // Every ordinary load issued so far must have landed before the first LDS-DMA goes out: the compiler
+    // would otherwise place its own "wait for kreg/vreg" inside the loop, and such a wait also drains the
+    // DMA loads that are meant to stay in flight.
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) asm volatile("" : "+v"(kreg[c]), "+v"(vreg[c]));
+    int ahead = 0;                                                                // pairs issued and not yet consumed
+    int fetch_stage = 0;
+    {
+        int64_t ta, tb; bool hb;
+        while (ahead < kStages - 1 && fetch_cur.next(ta, tb, hb)) {
+            issue(ta, tb, fetch_stage);
+            fetch_stage = fetch_stage == kStages - 1 ? 0 : fetch_stage + 1;
+            ++ahead;
+        }
+    }
+    int use_stage = 0;
+    int64_t ta, tb;
+    bool has_b;
+    while (use_cur.next(ta, tb, has_b)) {
+        // every wavefront issued 9 loads per pair, in order: allow the younger pairs' loads to stay in flight
+        if (ahead >= 3) __builtin_amdgcn_s_waitcnt(0x4F72);                       // vmcnt(18)
+        else if (ahead == 2) __builtin_amdgcn_s_waitcnt(0x0F79);                  // vmcnt(9)
+        else __builtin_amdgcn_s_waitcnt(0x0F70);                                  // vmcnt(0)
+        __syncthreads();                                                          // pair is in LDS for all; the stage consumed last turn is free
+        {
+            int64_t na, nb; bool hb;
+            if (fetch_cur.next(na, nb, hb)) {
+                issue(na, nb, fetch_stage);
+                fetch_stage = fetch_stage == kStages - 1 ? 0 : fetch_stage + 1;
+            } else {
+                --ahead;
+            }
+        }
+        const unsigned char* st = ring + use_stage * kStageBytes;
+        use_stage = use_stage == kStages - 1 ? 0 : use_stage + 1;
+
+        const float* scal = reinterpret_cast<const float*>(st + 32768 + wave * 256);
+        const float4 la = *reinterpret_cast<const float4*>(scal + 4 * g);
+        const float4 Da = *reinterpret_cast<const float4*>(scal + 16 + 4 * g);
+        const float4 lb = *reinterpret_cast<const float4*>(scal + 32 + 4 * g);
+        const float4 Db = *reinterpret_cast<const float4*>(scal + 48 + 4 * g);
+        const float lse_a[4] = {la.x, la.y, la.z, la.w};
+        const float lse_b[4] = {lb.x, lb.y, lb.z, lb.w};
+        const float D_a[4] = {Da.x, Da.y, Da.z, Da.w};
+        const float D_b[4] = {Db.x, Db.y, Db.z, Db.w};
+        int lim_a, lim_b;
+        {
+            const int valid = Sk - j * kBlockN - 1;
+            lim_a = valid; lim_b = valid;
+            if (kCausal) {
+                const int ca = static_cast<int>(ta - q0) + Sk - Sq - j * kBlockN;
+                const int cb = static_cast<int>(tb - q0) + Sk - Sq - j * kBlockN;
+                lim_a = ca < lim_a ? ca : lim_a;
+                lim_b = cb < lim_b ? cb : lim_b;
+            }
+            if (!has_b) lim_b = -1;
+        }
+        const uint4* frag = reinterpret_cast<const uint4*>(st) + lane;            // fragment c of tile t at frag[t*256 + c*64]
+        floatx4 sa = floatx4{0.f, 0.f, 0.f, 0.f}, sb = sa, dpa = sa, dpb = sa;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const uint4 ra = frag[0 * 256 + c * 64], rb = frag[1 * 256 + c * 64];
+            const uint4 rc = frag[2 * 256 + c * 64], rd = frag[3 * 256 + c * 64];
+            bf16x8 qa, qb, doa, dob;
+            __builtin_memcpy(&qa, &ra, 16);
+            __builtin_memcpy(&qb, &rb, 16);
+            __builtin_memcpy(&doa, &rc, 16);
+            __builtin_memcpy(&dob, &rd, 16);
+            sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa, kreg[c], sa, 0, 0, 0);
+            sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qb, kreg[c], sb, 0, 0, 0);
+            dpa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(doa, vreg[c], dpa, 0, 0, 0);
+            dpb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(dob, vreg[c], dpb, 0, 0, 0);
+        }
+        bf16x8 pfr, dsfr;
+        {
+            const int key = 16 * wave + n;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float xa = __builtin_amdgcn_exp2f(sa[e] * p.scale_log2 - lse_a[e]);
+                float xb = __builtin_amdgcn_exp2f(sb[e] * p.scale_log2 - lse_b[e]);
+                xa = key > lim_a ? 0.f : xa;
+                xb = key > lim_b ? 0.f : xb;
+                pfr[e] = static_cast<__bf16>(xa);
+                pfr[4 + e] = static_cast<__bf16>(xb);
+                dsfr[e] = static_cast<__bf16>(xa * (dpa[e] - D_a[e]));
+                dsfr[4 + e] = static_cast<__bf16>(xb * (dpb[e] - D_b[e]));
+            }
+        }
+        const uint2* timg = reinterpret_cast<const uint2*>(st + 16384) + lane;    // tile t, d-tile dt at timg[t*512 + dt*64]
+#pragma unroll
+        for (int dt = 0; dt < 8; ++dt) {
+            const uint2 a0 = timg[0 * 512 + dt * 64], a1 = timg[1 * 512 + dt * 64];
+            const uint2 d0 = timg[2 * 512 + dt * 64], d1 = timg[3 * 512 + dt * 64];
+            const uint4 aq_raw = make_uint4(a0.x, a0.y, a1.x, a1.y);
+            const uint4 ad_raw = make_uint4(d0.x, d0.y, d1.x, d1.y);
+            bf16x8 aq, ad;
+            __builtin_memcpy(&aq, &aq_raw, 16);
+            __builtin_memcpy(&ad, &ad_raw, 16);
+            dVt[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ad, pfr, dVt[dt], 0, 0, 0);
+            dKt[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aq, dsfr, dKt[dt], 0, 0, 0);
+        }
+    }
+
+    // each wavefront owns its 16 key columns: transpose through LDS for coalesced atomics
+    const int valid_keys = (Sk - j * kBlockN) < kBlockN ? (Sk - j * kBlockN) : kBlockN;
+    const int64_t row0 = static_cast<int64_t>(k0) + static_cast<int64_t>(j) * kBlockN;
+#pragma unroll
+    for (int which = 0; which < 2; ++which) {
+        __syncthreads();
+#pragma unroll
+        for (int dt = 0; dt < 8; ++dt)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                red[(16 * dt + 4 * g + e) * kRedPitch + 16 * wave + n] = which == 0 ? dKt[dt][e] : dVt[dt][e];
+        __syncthreads();
+        float* acc = which == 0 ? p.dk_acc : p.dv_acc;
+        const float mul = which == 0 ? p.scale : 1.f;
+        for (int idx = tid; idx < kBlockN * kHeadDim; idx += 256) {
+            const int key = idx >> 7, d = idx & 127;
+            if (key < valid_keys)
+                unsafeAtomicAdd(acc + ((row0 + key) * p.num_heads_k + h) * kHeadDim + d, red[d * kRedPitch + key] * mul);
+        }
+    }
+}
+
 __global__ __launch_bounds__(256)
 void zero_f32_kernel(float4* __restrict__ ptr, int64_t n4) {
     const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
@@ -442,7 +718,7 @@ void bwd_convert_dkdv_kernel(const BwdParams p) {
 static size_t align256(size_t x) { return (x + 255) & ~static_cast<size_t>(255); }
 
 struct BwdLayout {
-    size_t images, mask, dsum, qT, doT, dk_acc, dv_acc, total;
+    size_t images, mask, dsum, qT, doT, qF, doF, rowstat, dk_acc, dv_acc, total;
 };
 
 static BwdLayout bwd_layout(int batch, int64_t total_q, int64_t total_k, int num_heads_k, int max_seqlen_k) {
@@ -454,6 +730,9 @@ static BwdLayout bwd_layout(int batch, int64_t total_q, int64_t total_k, int num
     L.dsum = off; off += align256(static_cast<size_t>(num_heads_k) * total_q * 16 * 4);
     L.qT = off; off += align256(static_cast<size_t>(num_heads_k) * total_q * kTImageElems * 2);
     L.doT = off; off += align256(static_cast<size_t>(num_heads_k) * total_q * kTImageElems * 2);
+    L.qF = off; off += align256(static_cast<size_t>(num_heads_k) * total_q * kTImageElems * 2);
+    L.doF = off; off += align256(static_cast<size_t>(num_heads_k) * total_q * kTImageElems * 2);
+    L.rowstat = off; off += align256(static_cast<size_t>(num_heads_k) * total_q * 32 * 4);
     L.dk_acc = off; off += align256(static_cast<size_t>(total_k) * num_heads_k * kHeadDim * 4);
     L.dv_acc = off; off += align256(static_cast<size_t>(total_k) * num_heads_k * kHeadDim * 4);
     L.total = off;
@@ -512,6 +791,9 @@ extern "C" int infllmv2_varlen_bwd(void* stream, const void* dout, const void* q
     p.dsum = reinterpret_cast<float*>(ws + L.dsum);
     p.qT = reinterpret_cast<bf16_bits*>(ws + L.qT);
     p.doT = reinterpret_cast<bf16_bits*>(ws + L.doT);
+    p.qF = reinterpret_cast<bf16_bits*>(ws + L.qF);
+    p.doF = reinterpret_cast<bf16_bits*>(ws + L.doF);
+    p.rowstat = reinterpret_cast<float*>(ws + L.rowstat);
     const int64_t n_slots = image_slots(total_k, batch);
     const int64_t img_elems = n_slots * num_heads_k * kImageElems;
     p.kimg = reinterpret_cast<const bf16_bits*>(ws + L.images);
@@ -563,10 +845,24 @@ extern "C" int infllmv2_varlen_bwd(void* stream, const void* dout, const void* q
         if (is_causal) hipLaunchKernelGGL(bwd_dq_kernel<true>, gq, dim3(256), 0, st, p);
         else hipLaunchKernelGGL(bwd_dq_kernel<false>, gq, dim3(256), 0, st, p);
         IV2_LAUNCH_CHECK();
-        const size_t lds = kHeadDim * kRedPitch * sizeof(float);          // 33280 B >= the 32 KiB of staged images
         const dim3 gk(static_cast<unsigned>(p.k_blocks) * p.n_slices, batch, num_heads_k);
-        if (is_causal) hipLaunchKernelGGL(bwd_dkdv_kernel<true>, gk, dim3(512), lds, st, p);
-        else hipLaunchKernelGGL(bwd_dkdv_kernel<false>, gk, dim3(512), lds, st, p);
+        static const bool split_variant = [] {                 // experiment switch: 4 token streams x 2 key halves, operands through registers
+            const char* e = getenv("INFLLMV2_BWD_DKDV_SPLIT");
+            return e != nullptr && e[0] == '1';
+        }();
+        if (split_variant) {
+            const size_t lds = kHeadDim * kRedPitch * sizeof(float);      // 33280 B >= the 32 KiB of staged images
+            if (is_causal) hipLaunchKernelGGL(bwd_dkdv_kernel<true>, gk, dim3(512), lds, st, p);
+            else hipLaunchKernelGGL(bwd_dkdv_kernel<false>, gk, dim3(512), lds, st, p);
+        } else {
+            const size_t lds = kStages * kStageBytes + kMaxSliceWords * 8;
+            const void* fn = is_causal ? reinterpret_cast<const void*>(&bwd_dkdv_stream_kernel<true>)
+                                       : reinterpret_cast<const void*>(&bwd_dkdv_stream_kernel<false>);
+            hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+            IV2_CHECK(e == hipSuccess, "varlen_bwd: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+            if (is_causal) hipLaunchKernelGGL(bwd_dkdv_stream_kernel<true>, gk, dim3(256), lds, st, p);
+            else hipLaunchKernelGGL(bwd_dkdv_stream_kernel<false>, gk, dim3(256), lds, st, p);
+        }
         IV2_LAUNCH_CHECK();
     } else if (total_q > 0) {
         // no keys at all: dq = 0

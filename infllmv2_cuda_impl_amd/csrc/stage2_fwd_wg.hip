@@ -247,6 +247,13 @@ void stage2_fwd_shared_kernel(const FwdParams p, const SharedFwdExtra x) {
         return cw * 64 + bit;
     };
 
+    // all ordinary loads (Q operands) land before the first LDS-DMA: otherwise the compiler's own wait for
+    // them sits inside the loop and drains the DMA loads that are meant to stay in flight
+    __builtin_amdgcn_s_waitcnt(kWaitVm0);
+#pragma unroll
+    for (int t = 0; t < kTW; ++t)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) asm volatile("" : "+v"(qf[t][c]));
     int j0 = next_block();
     int j1 = j0 >= 0 ? next_block() : -1;
     if (j0 >= 0) issue(j0, 0);
