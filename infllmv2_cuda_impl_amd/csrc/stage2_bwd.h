@@ -1,0 +1,48 @@
+// Parameters shared by the Stage-2 backward kernels.
+#pragma once
+#include "common.h"
+
+namespace infllmv2 {
+
+constexpr int kSliceTokens = 2048;        // query tokens per dK/dV workgroup
+constexpr int kTImageElems = 2048;        // one token x 16 heads x 128, transposed image
+constexpr float kLog2e = 1.44269504088896340736f;
+
+struct BwdParams {
+    const bf16_bits* q;
+    const bf16_bits* dout;
+    const bf16_bits* out;
+    bf16_bits* dq;
+    const float* lse;
+    float* dsum;                    // (Hk, total_q * 16): D of head 16h+g of token t at [h][16 t + g]
+    bf16_bits* qT;                  // (Hk, total_q, 8, 64, 4): lane (r, g) of d-tile dt holds X[heads 4g..4g+3][16 dt + r]
+    bf16_bits* doT;
+    bf16_bits* qF;                  // (Hk, total_q, 4, 64, 8): q and dout as ready-made A-operand fragments, lane (r, g) of
+    bf16_bits* doF;                 //   chunk c holds X[head r][32 c + 8 g ..]
+    float* rowstat;                 // (Hk, total_q, 32): LSE * log2(e) of the 16 heads, then D of the 16 heads
+    const bf16_bits* kimg;          // K, K-image order
+    const bf16_bits* kimg_t;        // K, V-image order
+    const bf16_bits* vimg_r;        // V, K-image order
+    float* dk_acc;                  // (total_k, Hk, 128) fp32
+    float* dv_acc;
+    bf16_bits* dk;
+    bf16_bits* dv;
+    const uint64_t* fwd_mask;       // (Hk, total_q, n64_fwd) or null
+    const uint64_t* bwd_mask;       // (Hk, k_blocks, n64_bwd) or null
+    const int* cu_seqlens_q;
+    const int* cu_seqlens_k;
+    int64_t q_tok, q_grp, q_kvh;    // element strides {token, head-in-group, kv-head}
+    int64_t do_tok, do_grp, do_kvh;
+    int64_t o_tok, o_grp, o_kvh;
+    int64_t dq_tok, dq_grp, dq_kvh;
+    int64_t lse_tok, lse_grp, lse_kvh;
+    int64_t dk_row, dk_head, dv_row, dv_head;
+    int64_t n_slots, total_q, total_k;
+    int n64_fwd, n64_bwd, k_blocks, num_heads_k, n_slices;
+    float scale_log2, scale;
+};
+
+// dK/dV, one wavefront per (64-key block, 512-token slice): stage2_bwd_dkdv.hip
+int launch_bwd_dkdv_wave(hipStream_t st, const BwdParams& p, int batch, int max_seqlen_q, bool causal);
+
+}  // namespace infllmv2

@@ -24,49 +24,12 @@
 #include "common.h"
 #include "kv_image.h"
 #include "block_walker.h"
+#include "stage2_bwd.h"
 #include "../../include/infllmv2_hip.h"
 #include <math.h>
 #include <stdlib.h>
 
 namespace infllmv2 {
-
-constexpr int kSliceTokens = 2048;        // query tokens per dK/dV workgroup
-constexpr int kTImageElems = 2048;        // one token x 16 heads x 128, transposed image
-constexpr float kLog2e = 1.44269504088896340736f;
-
-struct BwdParams {
-    const bf16_bits* q;
-    const bf16_bits* dout;
-    const bf16_bits* out;
-    bf16_bits* dq;
-    const float* lse;
-    float* dsum;                    // (Hk, total_q * 16): D of head 16h+g of token t at [h][16 t + g]
-    bf16_bits* qT;                  // (Hk, total_q, 8, 64, 4): lane (r, g) of d-tile dt holds X[heads 4g..4g+3][16 dt + r]
-    bf16_bits* doT;
-    bf16_bits* qF;                  // (Hk, total_q, 4, 64, 8): q and dout as ready-made A-operand fragments, lane (r, g) of
-    bf16_bits* doF;                 //   chunk c holds X[head r][32 c + 8 g ..]
-    float* rowstat;                 // (Hk, total_q, 32): LSE * log2(e) of the 16 heads, then D of the 16 heads
-    const bf16_bits* kimg;          // K, K-image order
-    const bf16_bits* kimg_t;        // K, V-image order
-    const bf16_bits* vimg_r;        // V, K-image order
-    float* dk_acc;                  // (total_k, Hk, 128) fp32
-    float* dv_acc;
-    bf16_bits* dk;
-    bf16_bits* dv;
-    const uint64_t* fwd_mask;       // (Hk, total_q, n64_fwd) or null
-    const uint64_t* bwd_mask;       // (Hk, k_blocks, n64_bwd) or null
-    const int* cu_seqlens_q;
-    const int* cu_seqlens_k;
-    int64_t q_tok, q_grp, q_kvh;    // element strides {token, head-in-group, kv-head}
-    int64_t do_tok, do_grp, do_kvh;
-    int64_t o_tok, o_grp, o_kvh;
-    int64_t dq_tok, dq_grp, dq_kvh;
-    int64_t lse_tok, lse_grp, lse_kvh;
-    int64_t dk_row, dk_head, dv_row, dv_head;
-    int64_t n_slots, total_q, total_k;
-    int n64_fwd, n64_bwd, k_blocks, num_heads_k, n_slices;
-    float scale_log2, scale;
-};
 
 // ---------------------------------------------------------------------------------------------
 // preprocessing: D = rowsum(dO * O) and the transposed per-token images of Q and dO
@@ -846,11 +809,14 @@ extern "C" int infllmv2_varlen_bwd(void* stream, const void* dout, const void* q
         else hipLaunchKernelGGL(bwd_dq_kernel<false>, gq, dim3(256), 0, st, p);
         IV2_LAUNCH_CHECK();
         const dim3 gk(static_cast<unsigned>(p.k_blocks) * p.n_slices, batch, num_heads_k);
-        static const bool split_variant = [] {                 // experiment switch: 4 token streams x 2 key halves, operands through registers
-            const char* e = getenv("INFLLMV2_BWD_DKDV_SPLIT");
-            return e != nullptr && e[0] == '1';
+        static const int variant = [] {                         // experiment switch: 1 = workgroup-streamed, 2 = 4 streams x 2 key halves
+            const char* e = getenv("INFLLMV2_BWD_DKDV");
+            return e == nullptr ? 0 : atoi(e);
         }();
-        if (split_variant) {
+        if (variant == 0) {
+            rc = launch_bwd_dkdv_wave(st, p, batch, max_seqlen_q, is_causal != 0);
+            if (rc != 0) return rc;
+        } else if (variant == 2) {
             const size_t lds = kHeadDim * kRedPitch * sizeof(float);      // 33280 B >= the 32 KiB of staged images
             if (is_causal) hipLaunchKernelGGL(bwd_dkdv_kernel<true>, gk, dim3(512), lds, st, p);
             else hipLaunchKernelGGL(bwd_dkdv_kernel<false>, gk, dim3(512), lds, st, p);
