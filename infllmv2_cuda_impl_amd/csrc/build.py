@@ -16,7 +16,7 @@ LIB_PATH = os.path.join(PKG, "libinfllmv2_hip.so")
 OBJ_DIR = os.path.join(PKG, "build")
 
 HIPCC_FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffast-math", "-fno-finite-math-only",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffast-math", "-fno-finite-math-only", *os.environ.get("IV2_EXTRA_FLAGS", "").split(),
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-value",
     # keep MFMA accumulators in ordinary VGPRs: the default AGPR form makes this compiler shuffle accumulators

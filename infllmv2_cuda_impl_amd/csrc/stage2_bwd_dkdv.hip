@@ -29,7 +29,9 @@
 namespace infllmv2 {
 
 constexpr int kColSlice = 512;                                 // query tokens per work item
-constexpr int kColWords = kColSlice / 64 + 1;                  // mask words a slice can touch
+constexpr int kGroupSlices = 4;                                // slices that pool their light members
+constexpr int kGroupWords = kGroupSlices * kColSlice / 64;     // = 32: one mask word per lane of the lower half
+constexpr int kHeavyPairs = 128;                               // a slice with fewer selected tokens is "light"
 constexpr int kStage = 16384 + 512;                            // q a|b, dout a|b (4 KiB each) + the pair's 64 row scalars
 constexpr int kWaveLds = 2 * kStage;                           // = 64 rows x 132 floats: also the flush tile
 constexpr int kFlushPitch = 132;                               // floats per key row of the flush tile
@@ -51,31 +53,22 @@ __device__ __forceinline__ void dma16(const void* base, uint32_t lane_off, uint3
 __device__ __forceinline__ void dma4(const void* base, uint32_t lane_off, uint32_t lds_base) {
     asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %0, %1" : : "v"(lane_off), "s"(base), "s"(lds_base) : "memory", "m0");
 }
-// One d tile of the second GEMMs: dV^T[dt][kt] += ad * p[kt] and dK^T[dt][kt] += aq * ds[kt] for the four key tiles,
-// accumulators in AGPRs.  Written as one asm block because the compiler cannot see that these are MFMAs: an MFMA
-// must not read a VGPR in the two issue slots after a VALU instruction wrote it, so the block opens with the wait
-// states itself and contains nothing but MFMAs; only MFMAs touch these accumulators inside the main loop.
-__device__ __forceinline__ void mfma_dtile(floatx4 (&dv)[4], floatx4 (&dk)[4], const bf16x8& ad, const bf16x8& aq,
-                                           const bf16x8 (&p)[4], const bf16x8 (&ds)[4]) {
-    int4v adi, aqi, pi[4], dsi[4];
-    __builtin_memcpy(&adi, &ad, 16);
-    __builtin_memcpy(&aqi, &aq, 16);
+// One d tile of one of the second GEMMs: acc[kt] += a * b[kt] for the four key tiles, accumulators in AGPRs.
+// Written as one asm block because the compiler cannot see that these are MFMAs: an MFMA must not read a VGPR in
+// the two issue slots after a VALU instruction wrote it, so the block opens with the wait states itself and
+// contains nothing but MFMAs; only MFMAs touch these accumulators inside the main loop.
+__device__ __forceinline__ void mfma_dtile(floatx4 (&acc)[4], const bf16x8& a, const bf16x8 (&b)[4]) {
+    int4v ai, bi[4];
+    __builtin_memcpy(&ai, &a, 16);
 #pragma unroll
-    for (int kt = 0; kt < 4; ++kt) {
-        __builtin_memcpy(&pi[kt], &p[kt], 16);
-        __builtin_memcpy(&dsi[kt], &ds[kt], 16);
-    }
+    for (int kt = 0; kt < 4; ++kt) __builtin_memcpy(&bi[kt], &b[kt], 16);
     asm("s_nop 1\n\t"
-        "v_mfma_f32_16x16x32_bf16 %0, %8, %10, %0\n\t"
-        "v_mfma_f32_16x16x32_bf16 %4, %9, %14, %4\n\t"
-        "v_mfma_f32_16x16x32_bf16 %1, %8, %11, %1\n\t"
-        "v_mfma_f32_16x16x32_bf16 %5, %9, %15, %5\n\t"
-        "v_mfma_f32_16x16x32_bf16 %2, %8, %12, %2\n\t"
-        "v_mfma_f32_16x16x32_bf16 %6, %9, %16, %6\n\t"
-        "v_mfma_f32_16x16x32_bf16 %3, %8, %13, %3\n\t"
-        "v_mfma_f32_16x16x32_bf16 %7, %9, %17, %7"
-        : "+a"(dv[0]), "+a"(dv[1]), "+a"(dv[2]), "+a"(dv[3]), "+a"(dk[0]), "+a"(dk[1]), "+a"(dk[2]), "+a"(dk[3])
-        : "v"(adi), "v"(aqi), "v"(pi[0]), "v"(pi[1]), "v"(pi[2]), "v"(pi[3]), "v"(dsi[0]), "v"(dsi[1]), "v"(dsi[2]), "v"(dsi[3]));
+        "v_mfma_f32_16x16x32_bf16 %0, %4, %5, %0\n\t"
+        "v_mfma_f32_16x16x32_bf16 %1, %4, %6, %1\n\t"
+        "v_mfma_f32_16x16x32_bf16 %2, %4, %7, %2\n\t"
+        "v_mfma_f32_16x16x32_bf16 %3, %4, %8, %3"
+        : "+a"(acc[0]), "+a"(acc[1]), "+a"(acc[2]), "+a"(acc[3])
+        : "v"(ai), "v"(bi[0]), "v"(bi[1]), "v"(bi[2]), "v"(bi[3]));
 }
 // 16 lanes x 4 halfwords, transposed: lane (16 g + r) receives element r % 4 of the rows supplied by lanes
 // 16 g + r / 4 + {0, 4, 8, 12}.
@@ -85,7 +78,7 @@ __device__ __forceinline__ short4v lds_read_tr(const unsigned char* ptr) {
 
 template <bool kCausal>
 __global__ __launch_bounds__(64)
-void bwd_dkdv_wave_kernel(const BwdParams p, const int n_items_slices) {
+void bwd_dkdv_wave_kernel(const BwdParams p) {
     extern __shared__ __attribute__((aligned(16))) unsigned char ring[];
     const int lane = threadIdx.x;
     const int n = lane & 15, g = lane >> 4;
@@ -96,44 +89,76 @@ void bwd_dkdv_wave_kernel(const BwdParams p, const int n_items_slices) {
     const int Sk = p.cu_seqlens_k[b + 1] - k0;
     const int nb = (Sk + kBlockN - 1) / kBlockN;               // key blocks of this sequence
 
-    // ---- which (slice, block): the slices' shared first block, then the diagonal block and outwards, so the
-    //      long items (initial block, local window) are dispatched first ----
-    const int rel = blockIdx.x / n_items_slices;
-    const int slice = blockIdx.x - rel * n_items_slices;
-    int i_lo = slice * kColSlice;
-    int i_hi = i_lo + kColSlice;
-    if (i_hi > Sq) i_hi = Sq;
-    if (i_lo >= i_hi || rel >= nb) return;                     // uniform
+    // ---- which (512-token slice, block) ----
+    // Slices are cut on the packed token axis (so they are whole mask words) and clipped to the sequence.
+    // Workgroup ids go round-robin over the 8 XCDs: each XCD takes one slice at a time (latest first), so the
+    // wavefronts sharing an L2 stream the same tokens of q and dout; within a slice the shared first block
+    // comes first, then the diagonal block and outwards, so the long items are dispatched early.
+    const int xcd = blockIdx.x & 7, turn = blockIdx.x >> 3;
+    const int rel = turn % p.k_blocks;
+    if (Sq <= 0 || rel >= nb) return;                          // uniform
+    const int last_slice = (q0 + Sq - 1) / kColSlice;
+    const int top_slice = last_slice | (kGroupSlices - 1);     // last slice of the last group
+    const int round = turn / p.k_blocks;                       // an XCD works through one group of slices in consecutive rounds
+    const int slice = top_slice - (((round / kGroupSlices) * 8 + xcd) * kGroupSlices + round % kGroupSlices);
+    if (slice > last_slice || slice < q0 / kColSlice) return;  // uniform
     int j;
     if (rel == 0) {
         j = 0;
     } else {
-        int jd = kCausal ? (i_hi - 1 + Sk - Sq) / kBlockN : nb - 1;   // last block any token of the slice may see
+        int i_last = (slice + 1) * kColSlice - 1 - q0;         // last token of the slice, inside the sequence
+        if (i_last > Sq - 1) i_last = Sq - 1;
+        int jd = kCausal ? (i_last + Sk - Sq) / kBlockN : nb - 1;                // last block any token of the slice may see
         if (jd > nb - 1) jd = nb - 1;
         if (jd < 0) jd = 0;
         j = jd - rel + 1;
         if (j < 1) j += nb - 1;
     }
+    // tokens of the sequence that may see key 64 j at all
+    int64_t t_lo = q0, t_hi = static_cast<int64_t>(q0) + Sq;
     if (kCausal) {
-        const int first = j * kBlockN - (Sk - Sq);             // first token that can see key 64 j
-        if (first > i_lo) i_lo = first;
+        const int first = j * kBlockN - (Sk - Sq);
+        if (first > 0) t_lo += first;
     }
-    if (i_lo >= i_hi) return;                                  // uniform
+    if (t_lo >= t_hi) return;                                  // uniform
 
-    // ---- the slice's mask words, clipped to its tokens: word w lives in lane w ----
-    const int64_t t_lo = static_cast<int64_t>(q0) + i_lo, t_hi = static_cast<int64_t>(q0) + i_hi;
-    const int w_lo = static_cast<int>(t_lo >> 6), w_hi = static_cast<int>((t_hi - 1) >> 6);
-    const int n_words = w_hi - w_lo + 1;                       // <= kColWords
-    uint64_t my_word = 0ull;
-    if (lane < n_words) {
+    // ---- light slices are merged ----
+    // A flush costs 32768 fp32 atomics whatever the slice held, so a slice works on its own only if at least
+    // kHeavyPairs of its tokens selected the block; the other slices of the same group of 4 hand their tokens
+    // to the first non-empty one among them.  Every workgroup of the group takes the same decision from the
+    // group's 32 mask words (lane l < 32 holds word l; a slice is 8 words = 8 lanes).
+    unsigned long long* wbuf = reinterpret_cast<unsigned long long*>(ring + kWaveLds);      // [kGroupWords]
+    const int group = slice / kGroupSlices, sub = slice % kGroupSlices;
+    const int64_t w0 = static_cast<int64_t>(group) * kGroupWords;
+    {
         const uint64_t* mrow = p.bwd_mask ? p.bwd_mask + (static_cast<int64_t>(h) * p.k_blocks + j) * p.n64_bwd : nullptr;
-        uint64_t v = mrow ? mrow[w_lo + lane] : ~0ull;
-        const int64_t base = static_cast<int64_t>(w_lo + lane) << 6;
-        if (base < t_lo) v &= ~0ull << (t_lo - base);
-        if (base + 64 > t_hi) v &= ~0ull >> (base + 64 - t_hi);
-        my_word = v;
+        uint64_t wv = 0ull;
+        if (lane < kGroupWords) {
+            const int64_t w = w0 + lane;
+            const int64_t base = w << 6;
+            if (base < t_hi && base + 64 > t_lo) {
+                wv = mrow ? mrow[w] : ~0ull;
+                if (base < t_lo) wv &= ~0ull << (t_lo - base);
+                if (base + 64 > t_hi) wv &= ~0ull >> (base + 64 - t_hi);
+            }
+        }
+        int cnt = __builtin_popcountll(wv);
+        cnt += __shfl_xor(cnt, 1);
+        cnt += __shfl_xor(cnt, 2);
+        cnt += __shfl_xor(cnt, 4);                             // tokens of this lane's slice that selected the block
+        const uint64_t heavy = __ballot(cnt >= kHeavyPairs);   // 8 equal bits per slice
+        const uint64_t filled = __ballot(cnt > 0);
+        bool keep;
+        if ((heavy >> (8 * sub)) & 1ull) {
+            keep = (lane >> 3) == sub;
+        } else {
+            const uint64_t light = filled & ~heavy;
+            if (light == 0ull || (__builtin_ctzll(light) >> 3) != sub) return;   // uniform: empty, or another slice collects
+            keep = !((heavy >> lane) & 1ull);
+        }
+        if (lane < kGroupWords) wbuf[lane] = keep ? wv : 0ull;
     }
-    if (__ballot(my_word != 0ull) == 0ull) return;             // nobody in the slice selected this block
+    __syncthreads();
 
     // ---- K and V of the block: B operands, resident in registers ----
     bf16x8 kreg[4][4], vreg[4][4];
@@ -156,17 +181,18 @@ void bwd_dkdv_wave_kernel(const BwdParams p, const int n_items_slices) {
             dVt[dt][kt] = floatx4{0.f, 0.f, 0.f, 0.f};
         }
 
-    // ---- token-pair cursor over the mask words (scalar state) ----
+    // ---- token-pair cursor over the kept mask words (scalar state) ----
     int cw = -1;
     uint64_t bits = 0ull;
     auto next_pair = [&](int64_t& ta, int64_t& tb, bool& has_b) -> bool {
         while (bits == 0ull) {
-            if (++cw >= n_words) return false;
-            const uint32_t lo = __builtin_amdgcn_readlane(static_cast<uint32_t>(my_word), cw);
-            const uint32_t hi = __builtin_amdgcn_readlane(static_cast<uint32_t>(my_word >> 32), cw);
+            if (++cw >= kGroupWords) return false;
+            const uint64_t v = wbuf[cw];
+            const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
+            const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
             bits = (static_cast<uint64_t>(hi) << 32) | lo;
         }
-        const int64_t base = static_cast<int64_t>(w_lo + cw) << 6;
+        const int64_t base = (w0 + cw) << 6;
         ta = base + __builtin_ctzll(bits);
         bits &= bits - 1ull;
         has_b = bits != 0ull;
@@ -218,6 +244,9 @@ void bwd_dkdv_wave_kernel(const BwdParams p, const int n_items_slices) {
     int64_t ta, tb;
     bool has_b;
     bool more = next_pair(ta, tb, has_b);
+#ifdef IV2_EXP_NOLOOP
+    more = more && q0 < 0;
+#endif
     if (more) issue(ta, tb, 0);
     int stage = 0;
     while (more) {
@@ -225,7 +254,11 @@ void bwd_dkdv_wave_kernel(const BwdParams p, const int n_items_slices) {
         bool nhb;
         const bool have_next = next_pair(na, nb2, nhb);
         if (have_next) {
-            issue(na, nb2, stage ^ 1);                         // the other stage was consumed by the previous turn
+#ifndef IV2_EXP_NODMA
+            issue(na, nb2, stage ^ 1);
+#else
+            if (na < 0) issue(na, nb2, stage ^ 1);
+#endif                         // the other stage was consumed by the previous turn
             __builtin_amdgcn_s_waitcnt(0x4F72);                // vmcnt(18): this turn's 18 loads have landed
         } else {
             __builtin_amdgcn_s_waitcnt(0x0F70);
@@ -256,69 +289,104 @@ void bwd_dkdv_wave_kernel(const BwdParams p, const int n_items_slices) {
         const float D_b[4] = {Db.x, Db.y, Db.z, Db.w};
         const bool edge = (lim_a < kBlockN - 1) || (lim_b < kBlockN - 1);
 
-        // S = Q K^T and dP = dO V^T for both tokens, 32 keys at a time (bounds the live accumulators), then
-        // P = exp2(scale S - LSE) and dS = P (dP - D), packed to bf16 as the B operands of the second GEMMs
+        // Four phases, each 32 MFMAs, with the VALU work of the softmax backward hidden behind the matrix pipeline:
+        //   A  S = Q K^T                       (both tokens, all 64 keys; every fragment read from LDS feeds 4 MFMAs)
+        //   B  dP = dO V^T                     while the VALU turns S into P = exp2(scale S - LSE) (fp32 and bf16)
+        //   C  dV^T += dO^T P                  while the VALU forms dS = P (dP - D) (bf16)
+        //   D  dK^T += Q^T dS
         const uint4* frag = reinterpret_cast<const uint4*>(st) + lane;           // tile t, chunk c at frag[t * 256 + c * 64]
         bf16x8 pfr[4], dsfr[4];                                // per key tile: [token a heads 4g..4g+3 | token b heads 4g..4g+3]
+        floatx4 sa[4], sb[4], dpa[4], dpb[4];
 #pragma unroll
-        for (int hf = 0; hf < 2; ++hf) {
-            floatx4 sa[2], sb[2], dpa[2], dpb[2];
-#pragma unroll
-            for (int k2 = 0; k2 < 2; ++k2) {
-                sa[k2] = floatx4{0.f, 0.f, 0.f, 0.f};
-                sb[k2] = sa[k2]; dpa[k2] = sa[k2]; dpb[k2] = sa[k2];
-            }
+        for (int kt = 0; kt < 4; ++kt) {
+            sa[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
+            sb[kt] = sa[kt]; dpa[kt] = sa[kt]; dpb[kt] = sa[kt];
+        }
+        {   // A
+            uint4 fr[2][2];
+            fr[0][0] = frag[0]; fr[0][1] = frag[256];
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
-                const uint4 r0 = frag[0 * 256 + c * 64], r1 = frag[1 * 256 + c * 64];
-                const uint4 r2 = frag[2 * 256 + c * 64], r3 = frag[3 * 256 + c * 64];
-                bf16x8 qa, qb, doa, dob;
-                __builtin_memcpy(&qa, &r0, 16);
-                __builtin_memcpy(&qb, &r1, 16);
-                __builtin_memcpy(&doa, &r2, 16);
-                __builtin_memcpy(&dob, &r3, 16);
+                if (c < 3) { fr[(c + 1) & 1][0] = frag[(c + 1) * 64]; fr[(c + 1) & 1][1] = frag[256 + (c + 1) * 64]; }
+                bf16x8 qa, qb;
+                __builtin_memcpy(&qa, &fr[c & 1][0], 16);
+                __builtin_memcpy(&qb, &fr[c & 1][1], 16);
 #pragma unroll
-                for (int k2 = 0; k2 < 2; ++k2) {
-                    const int kt = 2 * hf + k2;
-                    sa[k2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa, kreg[kt][c], sa[k2], 0, 0, 0);
-                    sb[k2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qb, kreg[kt][c], sb[k2], 0, 0, 0);
-                    dpa[k2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(doa, vreg[kt][c], dpa[k2], 0, 0, 0);
-                    dpb[k2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(dob, vreg[kt][c], dpb[k2], 0, 0, 0);
+                for (int kt = 0; kt < 4; ++kt) {
+                    sa[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa, kreg[kt][c], sa[kt], 0, 0, 0);
+                    sb[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qb, kreg[kt][c], sb[kt], 0, 0, 0);
                 }
             }
-#pragma unroll
-            for (int k2 = 0; k2 < 2; ++k2) {
-                const int kt = 2 * hf + k2;
-                const int nlim_a = lim_a - 16 * kt, nlim_b = lim_b - 16 * kt;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    float xa = __builtin_amdgcn_exp2f(sa[k2][e] * p.scale_log2 - lse_a[e]);
-                    float xb = __builtin_amdgcn_exp2f(sb[k2][e] * p.scale_log2 - lse_b[e]);
-                    if (edge) {
-                        xa = n > nlim_a ? 0.f : xa;
-                        xb = n > nlim_b ? 0.f : xb;
-                    }
-                    pfr[kt][e] = static_cast<__bf16>(xa);
-                    pfr[kt][4 + e] = static_cast<__bf16>(xb);
-                    dsfr[kt][e] = static_cast<__bf16>(xa * (dpa[k2][e] - D_a[e]));
-                    dsfr[kt][4 + e] = static_cast<__bf16>(xb * (dpb[k2][e] - D_b[e]));
-                }
-            }
-            __builtin_amdgcn_sched_barrier(0);                 // keep the halves apart: interleaving them costs 32 more live registers
         }
-
-        // dV^T += dO^T P and dK^T += Q^T dS: the A operands are transposed reads of the same LDS tiles
-        const unsigned char* tr = st + tr_off;
+        __builtin_amdgcn_sched_barrier(0);
+        {   // B
+            uint4 fr[2][2];
+            fr[0][0] = frag[512]; fr[0][1] = frag[768];
 #pragma unroll
-        for (int dt = 0; dt < 8; ++dt) {
-            const short4v q_a = lds_read_tr(tr + dt * 512), q_b = lds_read_tr(tr + 4096 + dt * 512);
-            const short4v d_a = lds_read_tr(tr + 8192 + dt * 512), d_b = lds_read_tr(tr + 12288 + dt * 512);
-            bf16x8 aq, ad;
-            __builtin_memcpy(&aq, &q_a, 8);
-            __builtin_memcpy(reinterpret_cast<unsigned char*>(&aq) + 8, &q_b, 8);
-            __builtin_memcpy(&ad, &d_a, 8);
-            __builtin_memcpy(reinterpret_cast<unsigned char*>(&ad) + 8, &d_b, 8);
-            mfma_dtile(dVt[dt], dKt[dt], ad, aq, pfr, dsfr);
+            for (int c = 0; c < 4; ++c) {
+                if (c < 3) { fr[(c + 1) & 1][0] = frag[512 + (c + 1) * 64]; fr[(c + 1) & 1][1] = frag[768 + (c + 1) * 64]; }
+                bf16x8 doa, dob;
+                __builtin_memcpy(&doa, &fr[c & 1][0], 16);
+                __builtin_memcpy(&dob, &fr[c & 1][1], 16);
+#pragma unroll
+                for (int kt = 0; kt < 4; ++kt) {
+                    dpa[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(doa, vreg[kt][c], dpa[kt], 0, 0, 0);
+                    dpb[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(dob, vreg[kt][c], dpb[kt], 0, 0, 0);
+                }
+                {   // P of key tile c, kept in fp32 in place of S
+                    const int kt = c;
+                    const int nlim_a = lim_a - 16 * kt, nlim_b = lim_b - 16 * kt;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        float xa = __builtin_amdgcn_exp2f(sa[kt][e] * p.scale_log2 - lse_a[e]);
+                        float xb = __builtin_amdgcn_exp2f(sb[kt][e] * p.scale_log2 - lse_b[e]);
+                        if (edge) {
+                            xa = n > nlim_a ? 0.f : xa;
+                            xb = n > nlim_b ? 0.f : xb;
+                        }
+                        sa[kt][e] = xa;
+                        sb[kt][e] = xb;
+                        pfr[kt][e] = static_cast<__bf16>(xa);
+                        pfr[kt][4 + e] = static_cast<__bf16>(xb);
+                    }
+                }
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        const unsigned char* tr = st + tr_off;
+        {   // C: the A operands are transposed reads of the dout tiles, fetched one d tile ahead
+            short4v t_a[2], t_b[2];
+            t_a[0] = lds_read_tr(tr + 8192); t_b[0] = lds_read_tr(tr + 12288);
+#pragma unroll
+            for (int dt = 0; dt < 8; ++dt) {
+                if (dt < 7) { t_a[(dt + 1) & 1] = lds_read_tr(tr + 8192 + (dt + 1) * 512); t_b[(dt + 1) & 1] = lds_read_tr(tr + 12288 + (dt + 1) * 512); }
+                bf16x8 ad;
+                __builtin_memcpy(&ad, &t_a[dt & 1], 8);
+                __builtin_memcpy(reinterpret_cast<unsigned char*>(&ad) + 8, &t_b[dt & 1], 8);
+                mfma_dtile(dVt[dt], ad, pfr);
+                {   // dS of half a key tile
+                    const int kt = dt >> 1, e0 = (dt & 1) * 2;
+#pragma unroll
+                    for (int e = e0; e < e0 + 2; ++e) {
+                        dsfr[kt][e] = static_cast<__bf16>(sa[kt][e] * (dpa[kt][e] - D_a[e]));
+                        dsfr[kt][4 + e] = static_cast<__bf16>(sb[kt][e] * (dpb[kt][e] - D_b[e]));
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        {   // D: transposed reads of the q tiles
+            short4v t_a[2], t_b[2];
+            t_a[0] = lds_read_tr(tr); t_b[0] = lds_read_tr(tr + 4096);
+#pragma unroll
+            for (int dt = 0; dt < 8; ++dt) {
+                if (dt < 7) { t_a[(dt + 1) & 1] = lds_read_tr(tr + (dt + 1) * 512); t_b[(dt + 1) & 1] = lds_read_tr(tr + 4096 + (dt + 1) * 512); }
+                bf16x8 aq;
+                __builtin_memcpy(&aq, &t_a[dt & 1], 8);
+                __builtin_memcpy(reinterpret_cast<unsigned char*>(&aq) + 8, &t_b[dt & 1], 8);
+                mfma_dtile(dKt[dt], aq, dsfr);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
         more = have_next;
         ta = na; tb = nb2; has_b = nhb;
@@ -354,12 +422,14 @@ void bwd_dkdv_wave_kernel(const BwdParams p, const int n_items_slices) {
 }
 
 int launch_bwd_dkdv_wave(hipStream_t st, const BwdParams& p, int batch, int max_seqlen_q, bool causal) {
-    const int n_slices = (max_seqlen_q + kColSlice - 1) / kColSlice;
-    const int64_t items = static_cast<int64_t>(n_slices) * p.k_blocks;
+    const int n_slices = (max_seqlen_q + kColSlice - 1) / kColSlice + 1 + kGroupSlices;   // sequences need not start or end on group boundaries
+    const int n_slices8 = (n_slices + 8 * kGroupSlices - 1) / (8 * kGroupSlices) * (8 * kGroupSlices);
+    const int64_t items = static_cast<int64_t>(n_slices8) * p.k_blocks;
     IV2_CHECK(items <= 0x7fffffffll, "varlen_bwd: too many (slice, block) work items");
     const dim3 grid(static_cast<unsigned>(items), batch, p.num_heads_k);
-    if (causal) hipLaunchKernelGGL(bwd_dkdv_wave_kernel<true>, grid, dim3(64), kWaveLds, st, p, n_slices);
-    else hipLaunchKernelGGL(bwd_dkdv_wave_kernel<false>, grid, dim3(64), kWaveLds, st, p, n_slices);
+    const size_t lds = kWaveLds + kGroupWords * 8;
+    if (causal) hipLaunchKernelGGL(bwd_dkdv_wave_kernel<true>, grid, dim3(64), lds, st, p);
+    else hipLaunchKernelGGL(bwd_dkdv_wave_kernel<false>, grid, dim3(64), lds, st, p);
     IV2_LAUNCH_CHECK();
     return 0;
 }
