@@ -42,6 +42,8 @@ struct BwdParams {
     float scale_log2, scale;
 };
 
+// dQ, 8 consecutive tokens per workgroup sharing their common blocks through LDS: stage2_bwd_dq.hip
+int launch_bwd_dq_hybrid(hipStream_t st, const BwdParams& p, int batch, int max_seqlen_q, bool causal);
 // dK/dV, one wavefront per (64-key block, 512-token slice): stage2_bwd_dkdv.hip
 int launch_bwd_dkdv_wave(hipStream_t st, const BwdParams& p, int batch, int max_seqlen_q, bool causal);
 

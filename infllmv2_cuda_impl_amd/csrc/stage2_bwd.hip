@@ -804,10 +804,19 @@ extern "C" int infllmv2_varlen_bwd(void* stream, const void* dout, const void* q
         IV2_CHECK(total_q <= 0x7fffffffll, "varlen_bwd: too many query tokens");
         hipLaunchKernelGGL(bwd_prep_kernel, dim3(static_cast<unsigned>(total_q), num_heads_k), dim3(256), 0, st, p);
         IV2_LAUNCH_CHECK();
-        const dim3 gq((max_seqlen_q + 3) / 4, batch, num_heads_k);
-        if (is_causal) hipLaunchKernelGGL(bwd_dq_kernel<true>, gq, dim3(256), 0, st, p);
-        else hipLaunchKernelGGL(bwd_dq_kernel<false>, gq, dim3(256), 0, st, p);
-        IV2_LAUNCH_CHECK();
+        static const bool dq_per_token = [] {                  // diagnostic switch: one wavefront per token, no sharing
+            const char* e = getenv("INFLLMV2_BWD_DQ_PER_TOKEN");
+            return e != nullptr && e[0] == '1';
+        }();
+        if (dq_per_token) {
+            const dim3 gq((max_seqlen_q + 3) / 4, batch, num_heads_k);
+            if (is_causal) hipLaunchKernelGGL(bwd_dq_kernel<true>, gq, dim3(256), 0, st, p);
+            else hipLaunchKernelGGL(bwd_dq_kernel<false>, gq, dim3(256), 0, st, p);
+            IV2_LAUNCH_CHECK();
+        } else {
+            rc = launch_bwd_dq_hybrid(st, p, batch, max_seqlen_q, is_causal != 0);
+            if (rc != 0) return rc;
+        }
         const dim3 gk(static_cast<unsigned>(p.k_blocks) * p.n_slices, batch, num_heads_k);
         static const int variant = [] {                         // experiment switch: 1 = workgroup-streamed, 2 = 4 streams x 2 key halves
             const char* e = getenv("INFLLMV2_BWD_DKDV");

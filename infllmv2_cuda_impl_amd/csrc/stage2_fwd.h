@@ -22,9 +22,9 @@ struct FwdParams {
     float scale_log2;               // softmax_scale * log2(e)
 };
 
-// Workgroup-shared forward: 16 consecutive tokens per workgroup walk the union of their mask rows
-// and stage every K/V block image once in LDS.
-int launch_stage2_fwd_shared(hipStream_t st, const FwdParams& p, int batch, int num_heads_k, int max_seqlen_q,
+// Workgroup-hybrid forward (stage2_fwd_hybrid.hip): 8 consecutive tokens per workgroup stage the blocks they all
+// select once in LDS and walk the rest of their rows one wavefront each.
+int launch_stage2_fwd_hybrid(hipStream_t st, const FwdParams& p, int batch, int num_heads_k, int max_seqlen_q,
                              int max_seqlen_k, bool causal);
 
 }  // namespace infllmv2

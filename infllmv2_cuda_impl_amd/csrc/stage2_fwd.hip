@@ -349,11 +349,11 @@ extern "C" int infllmv2_varlen_fwd(void* stream, const void* q, const void* k, c
     fp.total_q = total_q;
     fp.n64 = n_uint64_per_row;
     fp.scale_log2 = softmax_scale * 1.44269504088896340736f;
-    static const bool shared_walk = [] {                       // experiment switch: workgroup-shared union walk (stage2_fwd_wg.hip)
-        const char* e = getenv("INFLLMV2_FWD_SHARED");
+    static const bool per_token = [] {                         // diagnostic switch: the one-wavefront-per-token kernel
+        const char* e = getenv("INFLLMV2_FWD_PER_TOKEN");
         return e != nullptr && e[0] == '1';
     }();
-    if (shared_walk) return launch_stage2_fwd_shared(st, fp, batch, num_heads_k, max_seqlen_q, max_seqlen_k, is_causal != 0);
+    if (!per_token) return launch_stage2_fwd_hybrid(st, fp, batch, num_heads_k, max_seqlen_q, max_seqlen_k, is_causal != 0);
     const dim3 grid((max_seqlen_q + 3) / 4, batch, num_heads_k);
     if (is_causal) hipLaunchKernelGGL(stage2_fwd_kernel<true>, grid, dim3(256), 0, st, fp);
     else hipLaunchKernelGGL(stage2_fwd_kernel<false>, grid, dim3(256), 0, st, fp);
