@@ -31,8 +31,9 @@ __device__ __forceinline__ int64_t image_slot0(const int* cu_seqlens_k, int b) {
     return cu_seqlens_k[b] / kBlockN + b;
 }
 
-// Launches the packing pre-pass.  workspace receives [K image | V image] and, with
-// backward_images, also [K in V-image order | V in K-image order].
+// Launches the packing pre-pass.  workspace receives [K image | V image] for the forward or, with
+// backward_images, [K image | V in K-image order] (the backward contracts V over d, and reads K^T out of the
+// K image by transposed LDS loads).
 int launch_pack(hipStream_t st, const void* k, const void* v, const int32_t* cu_seqlens_k, void* workspace,
                 size_t workspace_bytes, int batch, int64_t total_k, int num_heads_k, int max_seqlen_k,
                 const int64_t* k_strides, const int64_t* v_strides, bool backward_images);

@@ -4,8 +4,6 @@
 
 namespace infllmv2 {
 
-constexpr int kSliceTokens = 2048;        // query tokens per dK/dV workgroup
-constexpr int kTImageElems = 2048;        // one token x 16 heads x 128, transposed image
 constexpr float kLog2e = 1.44269504088896340736f;
 
 struct BwdParams {
@@ -15,13 +13,8 @@ struct BwdParams {
     bf16_bits* dq;
     const float* lse;
     float* dsum;                    // (Hk, total_q * 16): D of head 16h+g of token t at [h][16 t + g]
-    bf16_bits* qT;                  // (Hk, total_q, 8, 64, 4): lane (r, g) of d-tile dt holds X[heads 4g..4g+3][16 dt + r]
-    bf16_bits* doT;
-    bf16_bits* qF;                  // (Hk, total_q, 4, 64, 8): q and dout as ready-made A-operand fragments, lane (r, g) of
-    bf16_bits* doF;                 //   chunk c holds X[head r][32 c + 8 g ..]
     float* rowstat;                 // (Hk, total_q, 32): LSE * log2(e) of the 16 heads, then D of the 16 heads
     const bf16_bits* kimg;          // K, K-image order
-    const bf16_bits* kimg_t;        // K, V-image order
     const bf16_bits* vimg_r;        // V, K-image order
     float* dk_acc;                  // (total_k, Hk, 128) fp32
     float* dv_acc;
@@ -38,7 +31,7 @@ struct BwdParams {
     int64_t lse_tok, lse_grp, lse_kvh;
     int64_t dk_row, dk_head, dv_row, dv_head;
     int64_t n_slots, total_q, total_k;
-    int n64_fwd, n64_bwd, k_blocks, num_heads_k, n_slices;
+    int n64_fwd, n64_bwd, k_blocks, num_heads_k;
     float scale_log2, scale;
 };
 

@@ -29,16 +29,13 @@ namespace infllmv2 {
 struct PackParams {
     const bf16_bits* k;
     const bf16_bits* v;
-    bf16_bits* kimg;                // K in K-image order (A/B operand of a GEMM contracting over d)
-    bf16_bits* vimg;                // V in V-image order (A operand of a GEMM contracting over keys)
-    bf16_bits* kimg_t;              // optional: K in V-image order (backward: dQ^T = K^T dS^T)
-    bf16_bits* vimg_r;              // optional: V in K-image order (backward: dP = dO V^T)
-    const int* cu_seqlens_k;        // cumulative (batch + 1) or, for a cache, null
-    const int* seqlens_k;           // per-sequence lengths when cu_seqlens_k is null
-    int64_t k_batch_stride, k_row_stride, k_head_stride;
-    int64_t v_batch_stride, v_row_stride, v_head_stride;
+    bf16_bits* kimg;                // K in K-image order (operand of a GEMM contracting over d)
+    bf16_bits* vimg;                // forward: V in V-image order (A operand of a GEMM contracting over keys), else null
+    bf16_bits* vimg_r;              // backward: V in K-image order (dP = dO V^T contracts over d), else null
+    const int* cu_seqlens_k;
+    int64_t k_row_stride, k_head_stride;
+    int64_t v_row_stride, v_head_stride;
     int64_t n_slots;
-    int slots_per_batch;            // used when cu_seqlens_k is null
 };
 
 constexpr int kVPad = 8;            // LDS row padding (elements) for the V transposition
@@ -47,25 +44,14 @@ __global__ __launch_bounds__(256)
 void pack_kv_kernel(const PackParams p) {
     __shared__ __attribute__((aligned(16))) bf16_bits vt[kBlockN][kHeadDim + kVPad];
     const int j = blockIdx.x, b = blockIdx.y, h = blockIdx.z;
-    int64_t row0, slot;
-    int Sk;
-    if (p.cu_seqlens_k != nullptr) {
-        const int k0 = p.cu_seqlens_k[b];
-        Sk = p.cu_seqlens_k[b + 1] - k0;
-        row0 = k0;
-        slot = image_slot0(p.cu_seqlens_k, b) + j;
-    } else {
-        Sk = p.seqlens_k[b];
-        row0 = 0;
-        slot = static_cast<int64_t>(b) * p.slots_per_batch + j;
-    }
+    const int k0 = p.cu_seqlens_k[b];
+    const int Sk = p.cu_seqlens_k[b + 1] - k0;
     if (static_cast<int64_t>(j) * kBlockN >= Sk) return;
+    const int64_t slot = image_slot0(p.cu_seqlens_k, b) + j;
     const int tid = threadIdx.x;
-    const bf16_bits* kb = p.k + b * p.k_batch_stride + (row0 + static_cast<int64_t>(j) * kBlockN) * p.k_row_stride + h * p.k_head_stride;
-    const bf16_bits* vb = p.v + b * p.v_batch_stride + (row0 + static_cast<int64_t>(j) * kBlockN) * p.v_row_stride + h * p.v_head_stride;
+    const bf16_bits* kb = p.k + (k0 + static_cast<int64_t>(j) * kBlockN) * p.k_row_stride + h * p.k_head_stride;
+    const bf16_bits* vb = p.v + (k0 + static_cast<int64_t>(j) * kBlockN) * p.v_row_stride + h * p.v_head_stride;
     const int64_t img_off = (static_cast<int64_t>(h) * p.n_slots + slot) * kImageElems;
-    bf16_bits* kdst = p.kimg + img_off;
-    bf16_bits* vdst = p.vimg + img_off;
     const int valid = Sk - j * kBlockN;                       // keys of this block inside the sequence
     const uint4 zero = make_uint4(0, 0, 0, 0);
 
@@ -75,13 +61,14 @@ void pack_kv_kernel(const PackParams p) {
         const int key = 16 * kt + r;
         uint4 val = zero;
         if (key < valid) val = *reinterpret_cast<const uint4*>(kb + key * p.k_row_stride + 32 * c + 8 * g);
-        *reinterpret_cast<uint4*>(kdst + u * 8) = val;
+        *reinterpret_cast<uint4*>(p.kimg + img_off + u * 8) = val;
         if (p.vimg_r != nullptr) {
             uint4 vv = zero;
             if (key < valid) vv = *reinterpret_cast<const uint4*>(vb + key * p.v_row_stride + 32 * c + 8 * g);
             *reinterpret_cast<uint4*>(p.vimg_r + img_off + u * 8) = vv;
         }
     }
+    if (p.vimg == nullptr) return;                            // uniform per workgroup
     for (int u = tid; u < 1024; u += 256) {
         const int key = u >> 4, d0 = (u & 15) * 8;
         uint4 val = zero;
@@ -99,28 +86,7 @@ void pack_kv_kernel(const PackParams p) {
             const int key_a = 32 * cc + (jj < 4 ? 4 * g + jj : 16 + 4 * g + jj - 4);
             w[jj >> 1] = static_cast<uint32_t>(vt[key_a][d]) | (static_cast<uint32_t>(vt[key_a + 1][d]) << 16);
         }
-        *reinterpret_cast<uint4*>(vdst + u * 8) = make_uint4(w[0], w[1], w[2], w[3]);
-    }
-    if (p.kimg_t == nullptr) return;                          // uniform per workgroup
-    __syncthreads();
-    for (int u = tid; u < 1024; u += 256) {
-        const int key = u >> 4, d0 = (u & 15) * 8;
-        uint4 val = zero;
-        if (key < valid) val = *reinterpret_cast<const uint4*>(kb + key * p.k_row_stride + d0);
-        *reinterpret_cast<uint4*>(&vt[key][d0]) = val;
-    }
-    __syncthreads();
-    for (int u = tid; u < 1024; u += 256) {
-        const int dt = u >> 7, cc = (u >> 6) & 1, lane = u & 63;
-        const int r = lane & 15, g = lane >> 4;
-        const int d = 16 * dt + r;
-        uint32_t w[4];
-#pragma unroll
-        for (int jj = 0; jj < 8; jj += 2) {
-            const int key_a = 32 * cc + (jj < 4 ? 4 * g + jj : 16 + 4 * g + jj - 4);
-            w[jj >> 1] = static_cast<uint32_t>(vt[key_a][d]) | (static_cast<uint32_t>(vt[key_a + 1][d]) << 16);
-        }
-        *reinterpret_cast<uint4*>(p.kimg_t + img_off + u * 8) = make_uint4(w[0], w[1], w[2], w[3]);
+        *reinterpret_cast<uint4*>(p.vimg + img_off + u * 8) = make_uint4(w[0], w[1], w[2], w[3]);
     }
 }
 
@@ -267,8 +233,7 @@ int launch_pack(hipStream_t st, const void* k, const void* v, const int32_t* cu_
     IV2_CHECK(k && v && cu_seqlens_k && workspace, "pack_kv: null pointer");
     IV2_CHECK(batch > 0 && num_heads_k > 0 && total_k >= 0 && max_seqlen_k >= 0, "pack_kv: bad sizes");
     IV2_CHECK(num_heads_k <= 65535 && batch <= 65535, "pack_kv: batch and num_heads_k must not exceed 65535");
-    IV2_CHECK(workspace_bytes >= infllmv2_kv_image_bytes(total_k, batch, num_heads_k) * (backward_images ? 2 : 1),
-              "pack_kv: workspace too small");
+    IV2_CHECK(workspace_bytes >= infllmv2_kv_image_bytes(total_k, batch, num_heads_k), "pack_kv: workspace too small");
     IV2_CHECK(reinterpret_cast<uintptr_t>(k) % 16 == 0 && reinterpret_cast<uintptr_t>(v) % 16 == 0 &&
               reinterpret_cast<uintptr_t>(workspace) % 16 == 0, "pack_kv: k, v and workspace must be 16-byte aligned");
     IV2_CHECK(k_strides[0] % 8 == 0 && k_strides[1] % 8 == 0 && v_strides[0] % 8 == 0 && v_strides[1] % 8 == 0,
@@ -280,11 +245,8 @@ int launch_pack(hipStream_t st, const void* k, const void* v, const int32_t* cu_
     pp.k = static_cast<const bf16_bits*>(k);
     pp.v = static_cast<const bf16_bits*>(v);
     pp.kimg = static_cast<bf16_bits*>(workspace);
-    pp.vimg = pp.kimg + n_slots * num_heads_k * kImageElems;
-    if (backward_images) {
-        pp.kimg_t = pp.vimg + n_slots * num_heads_k * kImageElems;
-        pp.vimg_r = pp.kimg_t + n_slots * num_heads_k * kImageElems;
-    }
+    bf16_bits* second = pp.kimg + n_slots * num_heads_k * kImageElems;
+    if (backward_images) pp.vimg_r = second; else pp.vimg = second;
     pp.cu_seqlens_k = cu_seqlens_k;
     pp.k_row_stride = k_strides[0]; pp.k_head_stride = k_strides[1];
     pp.v_row_stride = v_strides[0]; pp.v_head_stride = v_strides[1];
