@@ -225,7 +225,7 @@ def main():
         kernel_only(0)
         k_ms = event_ms(torch, kernel_only, max(10, args.steps))
         achieved = fwd_flops / k_ms / 1e9
-        result["roofline"] = {"bound": "mfma", "kernel": "stage2_fwd_kernel<causal>", "achieved": achieved,
+        result["roofline"] = {"bound": "mfma", "kernel": "stage2_fwd_hybrid_kernel<causal>", "achieved": achieved,
                               "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS,
                               "traffic": None, "kernel_ms": k_ms}
         try:

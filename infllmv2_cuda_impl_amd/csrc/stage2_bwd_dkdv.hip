@@ -244,9 +244,6 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
     int64_t ta, tb;
     bool has_b;
     bool more = next_pair(ta, tb, has_b);
-#ifdef IV2_EXP_NOLOOP
-    more = more && q0 < 0;
-#endif
     if (more) issue(ta, tb, 0);
     int stage = 0;
     while (more) {
@@ -254,11 +251,7 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
         bool nhb;
         const bool have_next = next_pair(na, nb2, nhb);
         if (have_next) {
-#ifndef IV2_EXP_NODMA
-            issue(na, nb2, stage ^ 1);
-#else
-            if (na < 0) issue(na, nb2, stage ^ 1);
-#endif                         // the other stage was consumed by the previous turn
+            issue(na, nb2, stage ^ 1);                         // the other stage was consumed by the previous turn
             __builtin_amdgcn_s_waitcnt(0x4F72);                // vmcnt(18): this turn's 18 loads have landed
         } else {
             __builtin_amdgcn_s_waitcnt(0x0F70);
