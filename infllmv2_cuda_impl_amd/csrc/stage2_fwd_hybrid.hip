@@ -10,7 +10,9 @@
 //     copied once, by LDS-DMA, from its fragment-major image into a 3-deep LDS ring two blocks
 //     ahead, and each wavefront reads its MFMA operands with conflict-free ds_read_b128;
 //   * the remaining blocks of a row are walked by its wavefront alone, operands straight from
-//     global memory into registers, as in stage2_fwd_kernel.
+//     global memory into registers, as in stage2_fwd_kernel;
+//   * the two walks are interleaved, one common and one own block per turn: the first is bound by
+//     the matrix pipeline and the VALU, the second by the vector memory path.
 //
 // A per-token kernel is bound by what the vector memory path can deliver (32 KiB of operands per
 // 512 MFMA cycles); the shared walk takes the common half of the work off that path.  Online
@@ -31,7 +33,7 @@ constexpr int kHybTokens = 8;                                  // tokens (= wave
 constexpr int kHybChunk = 64;                                  // token groups per XCD chunk
 constexpr int kRingTiles = 3;
 constexpr int kTileBytes = 32768;                              // K image | V image of one block
-constexpr int kMaxMaskWords = 512;                             // LDS copy of the common row: up to 32768 key blocks
+constexpr int kMaxMaskWords = 256;                             // LDS copies of the mask rows: up to 16384 key blocks
 
 struct HybridExtra {
     int groups_per_seq;                                        // ceil(max_seqlen_q / kHybTokens)
@@ -107,7 +109,8 @@ __global__ __launch_bounds__(512)
 void stage2_fwd_hybrid_kernel(const FwdParams p, const HybridExtra x) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     uint4* ring = reinterpret_cast<uint4*>(smem_raw);                               // [kRingTiles][2048]: K units 0..1023, V units 1024..2047
-    unsigned long long* com = reinterpret_cast<unsigned long long*>(smem_raw + kRingTiles * kTileBytes);   // [nw]
+    unsigned long long* com = reinterpret_cast<unsigned long long*>(smem_raw + kRingTiles * kTileBytes);   // [kMaxMaskWords]
+    unsigned long long* rows = com + kMaxMaskWords;                                 // [kHybTokens][kMaxMaskWords]
 
     // ---- which tokens: XCD-chunked, heaviest first ----
     const int bid = blockIdx.x;
@@ -138,32 +141,32 @@ void stage2_fwd_hybrid_kernel(const FwdParams p, const HybridExtra x) {
     const int64_t tok = static_cast<int64_t>(q0) + (live ? i : i0);
     const uint64_t* mrow = p.mask ? p.mask + (static_cast<int64_t>(h) * p.total_q + tok) * p.n64 : nullptr;
 
-    // ---- the row words every live token of the group has in common ----
+    // ---- the row words every live token of the group has in common, and what is left of each row ----
     int nw;                                                                          // words that can hold an allowed block of any token
     {
         const int i_last = (i0 + kHybTokens - 1 < Sq) ? i0 + kHybTokens - 1 : Sq - 1;
         int lk = kCausal ? (i_last + Sk - Sq) : (Sk - 1);
         if (lk > Sk - 1) lk = Sk - 1;
         nw = lk < 0 ? 0 : (lk >> 12) + 1;
-        if (mrow && nw > p.n64) nw = p.n64;
-        if (nw > kMaxMaskWords) nw = kMaxMaskWords;                                  // beyond that, blocks are simply not shared
+        if (mrow && nw > p.n64) nw = p.n64;                                          // nw <= kMaxMaskWords: checked by the launcher
     }
+    unsigned long long* own = rows + wave * kMaxMaskWords;                           // this token's row, later minus the common part
     for (int w = tid; w < nw; w += 512) com[w] = ~0ull;
     __syncthreads();
-    if (live) {
-        for (int w = lane; w < nw; w += 64) {
-            uint64_t v = 0ull;
-            if (last_blk >= 0 && w <= (last_blk >> 6)) {
-                v = mrow ? mrow[w] : ~0ull;
-                if (w == (last_blk >> 6)) {
-                    const int tb = last_blk & 63;
-                    v &= (tb == 63) ? ~0ull : ((1ull << (tb + 1)) - 1ull);
-                }
+    for (int w = lane; w < nw; w += 64) {
+        uint64_t v = 0ull;
+        if (last_blk >= 0 && w <= (last_blk >> 6)) {
+            v = mrow ? mrow[w] : ~0ull;
+            if (w == (last_blk >> 6)) {
+                const int tb = last_blk & 63;
+                v &= (tb == 63) ? ~0ull : ((1ull << (tb + 1)) - 1ull);
             }
-            if (v != ~0ull) atomicAnd(&com[w], static_cast<unsigned long long>(v));
         }
+        own[w] = v;
+        if (live && v != ~0ull) atomicAnd(&com[w], static_cast<unsigned long long>(v));
     }
     __syncthreads();
+    for (int w = lane; w < nw; w += 64) own[w] &= ~com[w];
 
     // ---- Q operand ----
     bf16x8 qf[4];
@@ -179,35 +182,67 @@ void stage2_fwd_hybrid_kernel(const FwdParams p, const HybridExtra x) {
 
     const int64_t slot0 = static_cast<int64_t>(h) * p.n_slots + image_slot0(p.cu_seqlens_k, b);
 
-    // ---- phase 1: the common blocks, in lock step through the LDS ring ----
-    {
-        const uint4* src_lane = (wave < 4 ? reinterpret_cast<const uint4*>(p.kimg) + slot0 * 1024 + wave * 256
-                                          : reinterpret_cast<const uint4*>(p.vimg) + slot0 * 1024 + (wave - 4) * 256) + lane;
-        const uint32_t ring_base = __builtin_amdgcn_readfirstlane(lds_address_of(ring) + wave * 4096);
-        auto issue = [&](int jj, int tile) { dma_copy_4k(src_lane + static_cast<int64_t>(jj) * 1024, ring_base + tile * kTileBytes); };
-        int cw = -1;
-        uint64_t cbits = 0ull;
-        auto next_common = [&]() -> int {
-            while (cbits == 0ull) {
-                if (++cw >= nw) return -1;
-                cbits = uniform_u64(com[cw]);
-            }
-            const int bit = __builtin_ctzll(cbits);
-            cbits &= cbits - 1ull;
-            return cw * 64 + bit;
-        };
-        // all ordinary loads (Q operands, mask words) land before the first LDS-DMA: otherwise the compiler's own
-        // wait for them sits inside the loop and drains the DMA loads that are meant to stay in flight
-        __builtin_amdgcn_s_waitcnt(0x0F70);                                          // vmcnt(0)
+    // ---- the walk: one turn = one common block (lock step, operands from the LDS ring) + one own block (operands
+    //      from global memory into registers).  The own blocks' loads keep the vector memory path busy while the
+    //      matrix pipeline works on the common block, and the other way round. ----
+    const uint4* src_lane = (wave < 4 ? reinterpret_cast<const uint4*>(p.kimg) + slot0 * 1024 + wave * 256
+                                      : reinterpret_cast<const uint4*>(p.vimg) + slot0 * 1024 + (wave - 4) * 256) + lane;
+    const uint32_t ring_base = __builtin_amdgcn_readfirstlane(lds_address_of(ring) + wave * 4096);
+    auto issue = [&](int jj, int tile) { dma_copy_4k(src_lane + static_cast<int64_t>(jj) * 1024, ring_base + tile * kTileBytes); };
+    int cw = -1, ow = -1;
+    uint64_t cbits = 0ull, obits = 0ull;
+    auto next_common = [&]() -> int {
+        while (cbits == 0ull) {
+            if (++cw >= nw) return -1;
+            cbits = uniform_u64(com[cw]);
+        }
+        const int bit = __builtin_ctzll(cbits);
+        cbits &= cbits - 1ull;
+        return cw * 64 + bit;
+    };
+    auto next_own = [&]() -> int {
+        while (obits == 0ull) {
+            if (++ow >= nw) return -1;
+            obits = uniform_u64(own[ow]);
+        }
+        const int bit = __builtin_ctzll(obits);
+        obits &= obits - 1ull;
+        return ow * 64 + bit;
+    };
+    const bf16_bits* kimg = p.kimg + slot0 * kImageElems + lane * 8;
+    const bf16_bits* vimg = p.vimg + slot0 * kImageElems + lane * 8;
+    bf16x8 kreg[16], vreg[16];
+    int jp = live ? next_own() : -1;                           // own block of this turn; its K fragments are loaded a turn ahead
+    if (jp >= 0) {
+        const bf16_bits* src = kimg + static_cast<int64_t>(jp) * kImageElems;
 #pragma unroll
-        for (int c = 0; c < 4; ++c) asm volatile("" : "+v"(qf[c]));
-        int j0 = next_common();
-        int j1 = j0 >= 0 ? next_common() : -1;
-        if (j0 >= 0) issue(j0, 0);
-        if (j1 >= 0) issue(j1, 1);
-        int tile = 0;
-        while (j0 >= 0) {
-            if (j1 >= 0) __builtin_amdgcn_s_waitcnt(0x0F74); else __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(4) / vmcnt(0)
+        for (int f = 0; f < 16; ++f) kreg[f] = *reinterpret_cast<const bf16x8*>(src + f * 512);
+    }
+    // All ordinary loads so far (Q, mask words, first K fragments) land before the first LDS-DMA.  From here on the
+    // compiler's wait counts know nothing of the DMA loads; they stay correct because loads complete in order (an
+    // unknown younger load only makes a wait stricter), and the waits written by hand below count the ordinary
+    // loads that may be younger than the DMA they wait for.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int c = 0; c < 4; ++c) asm volatile("" : "+v"(qf[c]));
+#pragma unroll
+    for (int f = 0; f < 16; ++f) asm volatile("" : "+v"(kreg[f]));
+    int j0 = next_common();
+    int j1 = j0 >= 0 ? next_common() : -1;
+    if (j0 >= 0) issue(j0, 0);
+    if (j1 >= 0) issue(j1, 1);
+    int tile = 0;
+    bool k_ahead = false;                                      // the coming own block's 16 K-fragment loads were issued last turn
+    while (j0 >= 0 || jp >= 0) {
+        if (j0 >= 0) {                                         // uniform over the workgroup
+            // younger than this wavefront's 4 DMA loads of block j0: the 4 of j1 and last turn's 16 K loads
+            const int young = (j1 >= 0 ? 4 : 0) + (k_ahead ? 16 : 0);
+            switch (young) {
+                case 20: asm volatile("s_waitcnt vmcnt(20)" ::: "memory"); break;
+                case 16: asm volatile("s_waitcnt vmcnt(16)" ::: "memory"); break;
+                case 4:  asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
+                default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+            }
             __syncthreads();                                   // block j0 is in LDS for everyone; tile (tile + 2) % 3 is free
             const int j2 = j1 >= 0 ? next_common() : -1;
             if (j2 >= 0) issue(j2, tile >= 1 ? tile - 1 : 2);
@@ -242,43 +277,10 @@ void stage2_fwd_hybrid_kernel(const FwdParams p, const HybridExtra x) {
             j1 = j2;
             tile = tile == 2 ? 0 : tile + 1;
         }
-    }
-    if (!live) return;                                                               // no barrier below
-
-    // ---- phase 2: this token's own blocks, operands straight from global memory ----
-    {
-        const int my_words = last_blk < 0 ? 0 : ((last_blk >> 6) + 1 < nw ? (last_blk >> 6) + 1 : nw);
-        int w = -1;
-        uint64_t bits = 0ull;
-        // rows wider than the LDS copy of the common words keep their far blocks private: com is ~0 only up to nw
-        const int row_words = last_blk < 0 ? 0 : (mrow ? ((last_blk >> 6) + 1 < p.n64 ? (last_blk >> 6) + 1 : p.n64) : (last_blk >> 6) + 1);
-        auto next_own = [&]() -> int {
-            while (bits == 0ull) {
-                if (++w >= row_words) return -1;
-                uint64_t v = mrow ? mrow[w] : ~0ull;
-                if (w == (last_blk >> 6)) {
-                    const int tb = last_blk & 63;
-                    v &= (tb == 63) ? ~0ull : ((1ull << (tb + 1)) - 1ull);
-                }
-                if (w < my_words) v &= ~com[w];
-                bits = uniform_u64(v);
-            }
-            const int bit = __builtin_ctzll(bits);
-            bits &= bits - 1ull;
-            return w * 64 + bit;
-        };
-        const bf16_bits* kimg = p.kimg + slot0 * kImageElems + lane * 8;
-        const bf16_bits* vimg = p.vimg + slot0 * kImageElems + lane * 8;
-        bf16x8 kreg[16], vreg[16];
-        int j = next_own();
-        if (j >= 0) {
-            const bf16_bits* src = kimg + static_cast<int64_t>(j) * kImageElems;
-#pragma unroll
-            for (int f = 0; f < 16; ++f) kreg[f] = *reinterpret_cast<const bf16x8*>(src + f * 512);
-        }
-        while (j >= 0) {
+        k_ahead = false;
+        if (jp >= 0) {                                         // per wavefront
             {
-                const bf16_bits* src = vimg + static_cast<int64_t>(j) * kImageElems;
+                const bf16_bits* src = vimg + static_cast<int64_t>(jp) * kImageElems;
 #pragma unroll
                 for (int f = 0; f < 16; ++f) vreg[f] = *reinterpret_cast<const bf16x8*>(src + f * 512);
             }
@@ -290,22 +292,24 @@ void stage2_fwd_hybrid_kernel(const FwdParams p, const HybridExtra x) {
                 for (int c = 0; c < 4; ++c)
                     s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[kt * 4 + c], qf[c], s[kt], 0, 0, 0);
             }
-            const int jn = next_own();
-            if (jn >= 0) {
-                const bf16_bits* src = kimg + static_cast<int64_t>(jn) * kImageElems;
-#pragma unroll
-                for (int f = 0; f < 16; ++f) kreg[f] = *reinterpret_cast<const bf16x8*>(src + f * 512);
-            }
             bf16x8 pf[2];
-            softmax_step(s, m, l, o, pf, (j == last_blk) ? last_key - j * kBlockN : kBlockN, g, p.scale_log2);
+            softmax_step(s, m, l, o, pf, (jp == last_blk) ? last_key - jp * kBlockN : kBlockN, g, p.scale_log2);
 #pragma unroll
             for (int dt = 0; dt < 8; ++dt)
 #pragma unroll
                 for (int cc = 0; cc < 2; ++cc)
                     o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg[dt * 2 + cc], pf[cc], o[dt], 0, 0, 0);
-            j = jn;
+            const int jn = next_own();
+            if (jn >= 0) {                                     // K fragments of the next own block
+                const bf16_bits* src = kimg + static_cast<int64_t>(jn) * kImageElems;
+#pragma unroll
+                for (int f = 0; f < 16; ++f) kreg[f] = *reinterpret_cast<const bf16x8*>(src + f * 512);
+                k_ahead = true;
+            }
+            jp = jn;
         }
     }
+    if (!live) return;
 
     // ---- epilogue ----
     const float l_tot = wave_sum_over_g(l);
@@ -331,10 +335,11 @@ int launch_stage2_fwd_hybrid(hipStream_t st, const FwdParams& p, int batch, int 
     x.groups_per_seq = (max_seqlen_q + kHybTokens - 1) / kHybTokens;
     const int64_t total = static_cast<int64_t>(num_heads_k) * batch * x.groups_per_seq;
     IV2_CHECK(total <= 0x3fffffff, "varlen_fwd: too many token groups");
+    IV2_CHECK((max_seqlen_k + kBlockN - 1) / kBlockN <= kMaxMaskWords * 64, "varlen_fwd: more than %d key blocks per sequence", kMaxMaskWords * 64);
     x.total_groups = static_cast<int>(total);
     const int64_t per_round = 8 * kHybChunk;
     const int64_t grid = (total + per_round - 1) / per_round * per_round;
-    const size_t lds = kRingTiles * kTileBytes + kMaxMaskWords * 8;
+    const size_t lds = kRingTiles * kTileBytes + (1 + kHybTokens) * kMaxMaskWords * 8;
     const void* fn = causal ? reinterpret_cast<const void*>(&stage2_fwd_hybrid_kernel<true>)
                             : reinterpret_cast<const void*>(&stage2_fwd_hybrid_kernel<false>);
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
@@ -342,7 +347,6 @@ int launch_stage2_fwd_hybrid(hipStream_t st, const FwdParams& p, int batch, int 
     if (causal) hipLaunchKernelGGL(stage2_fwd_hybrid_kernel<true>, dim3(static_cast<unsigned>(grid)), dim3(512), lds, st, p, x);
     else hipLaunchKernelGGL(stage2_fwd_hybrid_kernel<false>, dim3(static_cast<unsigned>(grid)), dim3(512), lds, st, p, x);
     IV2_LAUNCH_CHECK();
-    (void)max_seqlen_k;
     return 0;
 }
 
