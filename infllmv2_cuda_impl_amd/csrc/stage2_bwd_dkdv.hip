@@ -201,10 +201,14 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
         return true;
     };
 
-    // ---- LDS-DMA of one pair: lane (r, g') of chunk c gathers X[token][head r][32 c + 8 g' ..] ----
+    // ---- LDS-DMA of one pair: per 64-byte chunk c of the 16 head rows, one 1 KiB transfer ----
     const uint32_t ring_lds = __builtin_amdgcn_readfirstlane(lds_addr(ring));
-    const uint32_t q_lane = static_cast<uint32_t>((n * p.q_grp + 8 * g) * 2);       // byte offsets inside one token and KV head
-    const uint32_t do_lane = static_cast<uint32_t>((n * p.do_grp + 8 * g) * 2);
+    // Which 16 bytes a lane fetches: the four lanes of a quad take the four 16-byte pieces of one head's 64-byte
+    // chunk, so a quad is one contiguous 64-byte request.  LDS unit l = 4 * head + j of a chunk then holds piece
+    // (j + head / 4) % 4: the rotation makes the operand reads below bank-conflict free.
+    const int dma_head = lane >> 2, dma_piece = ((lane & 3) + (lane >> 4)) & 3;
+    const uint32_t q_lane = static_cast<uint32_t>((dma_head * p.q_grp + 8 * dma_piece) * 2);   // byte offsets inside one token and KV head
+    const uint32_t do_lane = static_cast<uint32_t>((dma_head * p.do_grp + 8 * dma_piece) * 2);
     const uint32_t stat_lane = static_cast<uint32_t>((lane & 31) * 4);
     const bf16_bits* q_head = p.q + static_cast<int64_t>(h) * p.q_kvh;
     const bf16_bits* do_head = p.dout + static_cast<int64_t>(h) * p.do_kvh;
@@ -239,7 +243,12 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
 
     // lane's byte offset inside a token's 4 KiB fragment tile for the transposed reads: row rho = lane % 16 of
     // the 16 x 4 group is X[head 4 g + rho / 4][16 dt + 4 (rho % 4) ..]
-    const int tr_off = ((n & 3) >> 1) * 256 + (4 * g + (n >> 2)) * 16 + (n & 1) * 8;
+    // piece g' = 2 (dt % 2) + (rho % 4) / 2 of head 4 g + rho / 4 sits in unit 4 * head + (g' - g) % 4
+    const int tr_head = 4 * g + (n >> 2);
+    const int tr_off_even = (4 * tr_head + ((((n & 3) >> 1) - g) & 3)) * 16 + (n & 1) * 8;
+    const int tr_off_odd = (4 * tr_head + ((2 + ((n & 3) >> 1) - g) & 3)) * 16 + (n & 1) * 8;
+    // operand fragment (head n, piece g) of a chunk: unit 4 n + (g - n / 4) % 4
+    const int frag_unit = 4 * n + ((g - (n >> 2)) & 3);
 
     int64_t ta, tb;
     bool has_b;
@@ -287,7 +296,7 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
         //   B  dP = dO V^T                     while the VALU turns S into P = exp2(scale S - LSE) (fp32 and bf16)
         //   C  dV^T += dO^T P                  while the VALU forms dS = P (dP - D) (bf16)
         //   D  dK^T += Q^T dS
-        const uint4* frag = reinterpret_cast<const uint4*>(st) + lane;           // tile t, chunk c at frag[t * 256 + c * 64]
+        const uint4* frag = reinterpret_cast<const uint4*>(st) + frag_unit;      // tile t, chunk c at frag[t * 256 + c * 64]
         bf16x8 pfr[4], dsfr[4];                                // per key tile: [token a heads 4g..4g+3 | token b heads 4g..4g+3]
         floatx4 sa[4], sb[4], dpa[4], dpb[4];
 #pragma unroll
@@ -346,13 +355,15 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
             }
         }
         __builtin_amdgcn_sched_barrier(0);
-        const unsigned char* tr = st + tr_off;
+        const unsigned char* tr_e = st + tr_off_even;
+        const unsigned char* tr_o = st + tr_off_odd;
+        auto tr_at = [&](int tile_bytes, int dt) { return ((dt & 1) ? tr_o : tr_e) + tile_bytes + (dt >> 1) * 1024; };
         {   // C: the A operands are transposed reads of the dout tiles, fetched one d tile ahead
             short4v t_a[2], t_b[2];
-            t_a[0] = lds_read_tr(tr + 8192); t_b[0] = lds_read_tr(tr + 12288);
+            t_a[0] = lds_read_tr(tr_at(8192, 0)); t_b[0] = lds_read_tr(tr_at(12288, 0));
 #pragma unroll
             for (int dt = 0; dt < 8; ++dt) {
-                if (dt < 7) { t_a[(dt + 1) & 1] = lds_read_tr(tr + 8192 + (dt + 1) * 512); t_b[(dt + 1) & 1] = lds_read_tr(tr + 12288 + (dt + 1) * 512); }
+                if (dt < 7) { t_a[(dt + 1) & 1] = lds_read_tr(tr_at(8192, dt + 1)); t_b[(dt + 1) & 1] = lds_read_tr(tr_at(12288, dt + 1)); }
                 bf16x8 ad;
                 __builtin_memcpy(&ad, &t_a[dt & 1], 8);
                 __builtin_memcpy(reinterpret_cast<unsigned char*>(&ad) + 8, &t_b[dt & 1], 8);
@@ -370,10 +381,10 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
         }
         {   // D: transposed reads of the q tiles
             short4v t_a[2], t_b[2];
-            t_a[0] = lds_read_tr(tr); t_b[0] = lds_read_tr(tr + 4096);
+            t_a[0] = lds_read_tr(tr_at(0, 0)); t_b[0] = lds_read_tr(tr_at(4096, 0));
 #pragma unroll
             for (int dt = 0; dt < 8; ++dt) {
-                if (dt < 7) { t_a[(dt + 1) & 1] = lds_read_tr(tr + (dt + 1) * 512); t_b[(dt + 1) & 1] = lds_read_tr(tr + 4096 + (dt + 1) * 512); }
+                if (dt < 7) { t_a[(dt + 1) & 1] = lds_read_tr(tr_at(0, dt + 1)); t_b[(dt + 1) & 1] = lds_read_tr(tr_at(4096, dt + 1)); }
                 bf16x8 aq;
                 __builtin_memcpy(&aq, &t_a[dt & 1], 8);
                 __builtin_memcpy(reinterpret_cast<unsigned char*>(&aq) + 8, &t_b[dt & 1], 8);
