@@ -24,6 +24,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
+# HBM bytes per launch of the dominant kernel at the default workload: 2.00 x FETCH_SIZE + 1.00 x WRITE_SIZE of the two
+# rocprofv3 --pmc runs summarised in profiles/stage2_fwd_config2_hbm_traffic.md (counters cannot be read from inside
+# this process); null for any other workload
+MEASURED_FWD_TRAFFIC_BYTES = 5.40e9
 PEAK_BF16_TFLOPS = 2500.0      # MI355X dense bf16 MFMA peak (vendor figure, no sparsity)
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E peak
 
@@ -227,7 +231,7 @@ def main():
         achieved = fwd_flops / k_ms / 1e9
         result["roofline"] = {"bound": "mfma", "kernel": "stage2_fwd_hybrid_kernel<causal>", "achieved": achieved,
                               "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS,
-                              "traffic": None, "kernel_ms": k_ms}
+                              "traffic": MEASURED_FWD_TRAFFIC_BYTES if (S, topk) == (32768, 64) else None, "kernel_ms": k_ms}
         try:
             from infllmv2_cuda_impl_amd.backward import HAVE_BACKWARD  # noqa: F401
             qg, kg, vg = [t.clone().requires_grad_(True) for t in (q, k, v)]
