@@ -42,13 +42,35 @@ struct BlockWalker {
     }
 };
 
+// Cross-row exchanges with gfx950's v_permlane16_swap / v_permlane32_swap (VALU speed; a ds_bpermute takes a trip
+// through the LDS crossbar): swapping a register with itself hands every lane its own row's value and the partner
+// row's value.
+__device__ __forceinline__ void row_pair_xor16(float x, float& mine, float& other) {
+    typedef unsigned u2 __attribute__((ext_vector_type(2)));
+    const u2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    mine = __uint_as_float(r[0]);
+    other = __uint_as_float(r[1]);
+}
+__device__ __forceinline__ void row_pair_xor32(float x, float& mine, float& other) {
+    typedef unsigned u2 __attribute__((ext_vector_type(2)));
+    const u2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    mine = __uint_as_float(r[0]);
+    other = __uint_as_float(r[1]);
+}
+// reductions over the four 16-lane groups g of a wavefront (lanes l, l ^ 16, l ^ 32, l ^ 48)
 __device__ __forceinline__ float wave_max_over_g(float x) {
-    x = fmaxf(x, __shfl_xor(x, 16));
-    return fmaxf(x, __shfl_xor(x, 32));
+    float a, b;
+    row_pair_xor16(x, a, b);
+    x = fmaxf(a, b);
+    row_pair_xor32(x, a, b);
+    return fmaxf(a, b);
 }
 __device__ __forceinline__ float wave_sum_over_g(float x) {
-    x += __shfl_xor(x, 16);
-    return x + __shfl_xor(x, 32);
+    float a, b;
+    row_pair_xor16(x, a, b);
+    x = a + b;
+    row_pair_xor32(x, a, b);
+    return a + b;
 }
 
 }  // namespace infllmv2

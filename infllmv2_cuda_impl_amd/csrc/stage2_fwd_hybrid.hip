@@ -93,8 +93,10 @@ __device__ __forceinline__ void softmax_step(floatx4 (&s)[4], float& m, float& l
         }
     l = l * alpha + rs;
     m = m_new;
+    if (__ballot(alpha != 1.f) != 0ull) {                      // the running maxima moved (rare after the first blocks)
 #pragma unroll
-    for (int dt = 0; dt < 8; ++dt) o[dt] *= alpha;
+        for (int dt = 0; dt < 8; ++dt) o[dt] *= alpha;
+    }
 #pragma unroll
     for (int cc = 0; cc < 2; ++cc)
 #pragma unroll
@@ -247,31 +249,35 @@ void stage2_fwd_hybrid_kernel(const FwdParams p, const HybridExtra x) {
             const int j2 = j1 >= 0 ? next_common() : -1;
             if (j2 >= 0) issue(j2, tile >= 1 ? tile - 1 : 2);
             if (live) {
+                // all 16 fragments of a tile are fetched before the MFMAs that use them (vreg is free between own
+                // blocks), and the MFMAs run over independent accumulators first
                 const uint4* kb = ring + tile * 2048 + lane;
                 const uint4* vb = kb + 1024;
+#pragma unroll
+                for (int f = 0; f < 16; ++f) {
+                    const uint4 raw = kb[f * 64];
+                    __builtin_memcpy(&vreg[f], &raw, 16);
+                }
                 floatx4 s[4];
 #pragma unroll
-                for (int kt = 0; kt < 4; ++kt) {
-                    s[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
+                for (int kt = 0; kt < 4; ++kt) s[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                    for (int c = 0; c < 4; ++c) {
-                        const uint4 raw = kb[(kt * 4 + c) * 64];
-                        bf16x8 kf;
-                        __builtin_memcpy(&kf, &raw, 16);
-                        s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[c], s[kt], 0, 0, 0);
-                    }
+                for (int c = 0; c < 4; ++c)
+#pragma unroll
+                    for (int kt = 0; kt < 4; ++kt)
+                        s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg[kt * 4 + c], qf[c], s[kt], 0, 0, 0);
+#pragma unroll
+                for (int f = 0; f < 16; ++f) {
+                    const uint4 raw = vb[f * 64];
+                    __builtin_memcpy(&vreg[f], &raw, 16);
                 }
                 bf16x8 pf[2];
                 softmax_step(s, m, l, o, pf, (j0 == last_blk) ? last_key - j0 * kBlockN : kBlockN, g, p.scale_log2);
 #pragma unroll
-                for (int dt = 0; dt < 8; ++dt)
+                for (int cc = 0; cc < 2; ++cc)
 #pragma unroll
-                    for (int cc = 0; cc < 2; ++cc) {
-                        const uint4 raw = vb[(dt * 2 + cc) * 64];
-                        bf16x8 vf;
-                        __builtin_memcpy(&vf, &raw, 16);
-                        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[cc], o[dt], 0, 0, 0);
-                    }
+                    for (int dt = 0; dt < 8; ++dt)
+                        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg[dt * 2 + cc], pf[cc], o[dt], 0, 0, 0);
             }
             j0 = j1;
             j1 = j2;
@@ -286,18 +292,18 @@ void stage2_fwd_hybrid_kernel(const FwdParams p, const HybridExtra x) {
             }
             floatx4 s[4];
 #pragma unroll
-            for (int kt = 0; kt < 4; ++kt) {
-                s[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
+            for (int kt = 0; kt < 4; ++kt) s[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int c = 0; c < 4; ++c)
+            for (int c = 0; c < 4; ++c)
+#pragma unroll
+                for (int kt = 0; kt < 4; ++kt)
                     s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[kt * 4 + c], qf[c], s[kt], 0, 0, 0);
-            }
             bf16x8 pf[2];
             softmax_step(s, m, l, o, pf, (jp == last_blk) ? last_key - jp * kBlockN : kBlockN, g, p.scale_log2);
 #pragma unroll
-            for (int dt = 0; dt < 8; ++dt)
+            for (int cc = 0; cc < 2; ++cc)
 #pragma unroll
-                for (int cc = 0; cc < 2; ++cc)
+                for (int dt = 0; dt < 8; ++dt)
                     o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg[dt * 2 + cc], pf[cc], o[dt], 0, 0, 0);
             const int jn = next_own();
             if (jn >= 0) {                                     // K fragments of the next own block
