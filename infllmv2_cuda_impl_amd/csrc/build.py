@@ -18,7 +18,7 @@ OBJ_DIR = os.path.join(PKG, "build")
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffast-math", "-fno-finite-math-only", *os.environ.get("IV2_EXTRA_FLAGS", "").split(),
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-Wno-unused-value",
+    "-Wno-unused-value", "-Wno-inline-asm",
     # keep MFMA accumulators in ordinary VGPRs: the default AGPR form makes this compiler shuffle accumulators
     # through v_accvgpr_read/write around every MFMA whose result the VALU touches
     "-mllvm", "-amdgpu-mfma-vgpr-form",

@@ -7,11 +7,11 @@
 // no atomics, no conversion pass, bit-reproducible.
 //
 // Schedule as in stage2_fwd_hybrid.hip: 8 wavefronts = 8 consecutive tokens; the blocks all 8
-// mask rows select go once through a 3-deep LDS ring ([K image | V in K-image order], 32 KiB),
+// mask rows select go once through a 2-tile LDS ring ([K image | V in K-image order], 32 KiB),
 // and there the K^T operand of dQ^T = K^T dS^T is a transposed read (ds_read_b64_tr_b16) of
 // the same K tile; the remaining blocks of each row are walked by its wavefront alone, K and V
 // fragments straight from global memory into registers, the K fragments parked in a private LDS
-// tile for the same transposed read.
+// tile for the same transposed read.  The two walks are interleaved, one block of each per turn.
 #include "common.h"
 #include "kv_image.h"
 #include "block_walker.h"
@@ -23,8 +23,8 @@ namespace infllmv2 {
 constexpr int kDqTokens = 8;
 constexpr int kDqChunk = 64;                                   // token groups per XCD chunk
 constexpr int kDqTileBytes = 32768;
-constexpr int kDqMaskWords = 512;
-constexpr int kDqLdsTiles = 8 * 16384;                         // max(3-tile ring, 8 private K tiles)
+constexpr int kDqMaskWords = 256;                              // LDS copies of the mask rows: up to 16384 key blocks
+constexpr int kDqLdsTiles = 2 * kDqTileBytes + 8 * 8192;       // 2-tile ring + 8 private half K tiles
 
 typedef short short4q __attribute__((ext_vector_type(4)));
 
@@ -74,8 +74,9 @@ template <bool kCausal>
 __global__ __launch_bounds__(512)
 void bwd_dq_hybrid_kernel(const BwdParams p, const DqExtra x) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-    uint4* ring = reinterpret_cast<uint4*>(smem_raw);                               // [3][2048]: K units 0..1023, V (K-image order) 1024..2047
-    unsigned long long* com = reinterpret_cast<unsigned long long*>(smem_raw + kDqLdsTiles);
+    uint4* ring = reinterpret_cast<uint4*>(smem_raw);                               // [2][2048]: K units 0..1023, V (K-image order) 1024..2047
+    unsigned long long* com = reinterpret_cast<unsigned long long*>(smem_raw + kDqLdsTiles);       // [kDqMaskWords]
+    unsigned long long* rows = com + kDqMaskWords;                                                  // [kDqTokens][kDqMaskWords]
 
     const int bid = blockIdx.x;
     const int xcd = bid & 7, sidx = bid >> 3;
@@ -105,32 +106,32 @@ void bwd_dq_hybrid_kernel(const BwdParams p, const DqExtra x) {
     const int64_t tok = static_cast<int64_t>(q0) + (live ? i : i0);
     const uint64_t* mrow = p.fwd_mask ? p.fwd_mask + (static_cast<int64_t>(h) * p.total_q + tok) * p.n64_fwd : nullptr;
 
-    // ---- the row words every live token of the group has in common ----
+    // ---- the row words every live token of the group has in common, and what is left of each row ----
     int nw;
     {
         const int i_last = (i0 + kDqTokens - 1 < Sq) ? i0 + kDqTokens - 1 : Sq - 1;
         int lk = kCausal ? (i_last + Sk - Sq) : (Sk - 1);
         if (lk > Sk - 1) lk = Sk - 1;
         nw = lk < 0 ? 0 : (lk >> 12) + 1;
-        if (mrow && nw > p.n64_fwd) nw = p.n64_fwd;
-        if (nw > kDqMaskWords) nw = kDqMaskWords;
+        if (mrow && nw > p.n64_fwd) nw = p.n64_fwd;                                  // nw <= kDqMaskWords: checked by the launcher
     }
+    unsigned long long* own = rows + wave * kDqMaskWords;
     for (int w = tid; w < nw; w += 512) com[w] = ~0ull;
     __syncthreads();
-    if (live) {
-        for (int w = lane; w < nw; w += 64) {
-            uint64_t v = 0ull;
-            if (last_blk >= 0 && w <= (last_blk >> 6)) {
-                v = mrow ? mrow[w] : ~0ull;
-                if (w == (last_blk >> 6)) {
-                    const int tb = last_blk & 63;
-                    v &= (tb == 63) ? ~0ull : ((1ull << (tb + 1)) - 1ull);
-                }
+    for (int w = lane; w < nw; w += 64) {
+        uint64_t v = 0ull;
+        if (last_blk >= 0 && w <= (last_blk >> 6)) {
+            v = mrow ? mrow[w] : ~0ull;
+            if (w == (last_blk >> 6)) {
+                const int tb = last_blk & 63;
+                v &= (tb == 63) ? ~0ull : ((1ull << (tb + 1)) - 1ull);
             }
-            if (v != ~0ull) atomicAnd(&com[w], static_cast<unsigned long long>(v));
         }
+        own[w] = v;
+        if (live && v != ~0ull) atomicAnd(&com[w], static_cast<unsigned long long>(v));
     }
     __syncthreads();
+    for (int w = lane; w < nw; w += 64) own[w] &= ~com[w];
 
     // ---- this token's operands ----
     bf16x8 qf[4], dof[4];
@@ -154,39 +155,64 @@ void bwd_dq_hybrid_kernel(const BwdParams p, const DqExtra x) {
     // dt and key chunk kt2 is K[16 kt2 + 4 g + rho / 4][16 dt + 4 (rho % 4) ..]
     const int tr_lane = (((n & 3) >> 1) * 16 + 4 * g + (n >> 2)) * 16 + (n & 1) * 8;
 
-    // ---- phase 1: the common blocks, in lock step through the LDS ring ----
-    {
-        const uint4* src_lane = (wave < 4 ? reinterpret_cast<const uint4*>(p.kimg) + slot0 * 1024 + wave * 256
-                                          : reinterpret_cast<const uint4*>(p.vimg_r) + slot0 * 1024 + (wave - 4) * 256) + lane;
-        const uint32_t ring_base = __builtin_amdgcn_readfirstlane(lds_address_dq(ring) + wave * 4096);
-        auto issue = [&](int jj, int tile) { dq_dma_copy_4k(src_lane + static_cast<int64_t>(jj) * 1024, ring_base + tile * kDqTileBytes); };
-        int cw = -1;
-        uint64_t cbits = 0ull;
-        auto next_common = [&]() -> int {
-            while (cbits == 0ull) {
-                if (++cw >= nw) return -1;
-                cbits = dq_uniform_u64(com[cw]);
-            }
-            const int bit = __builtin_ctzll(cbits);
-            cbits &= cbits - 1ull;
-            return cw * 64 + bit;
-        };
-        // all ordinary loads land before the first LDS-DMA (the compiler's own wait for them would otherwise sit
-        // inside the loop and drain the DMA loads that are meant to stay in flight)
-        __builtin_amdgcn_s_waitcnt(0x0F70);                                          // vmcnt(0)
+    // ---- the walk: one turn = one common block (lock step, operands from the 2-tile LDS ring) + one own block
+    //      (K and V fragments from global memory into registers, prefetched a turn ahead).  The K fragments of an own
+    //      block feed S from registers and are parked, 32 keys at a time, in this wavefront's 8 KiB LDS tile, from
+    //      which dQ's K^T operand is a transposed read: an own block costs 32 KiB of global loads, not 48. ----
+    const uint4* src_lane = (wave < 4 ? reinterpret_cast<const uint4*>(p.kimg) + slot0 * 1024 + wave * 256
+                                      : reinterpret_cast<const uint4*>(p.vimg_r) + slot0 * 1024 + (wave - 4) * 256) + lane;
+    const uint32_t ring_base = __builtin_amdgcn_readfirstlane(lds_address_dq(ring) + wave * 4096);
+    auto issue = [&](int jj, int tile) { dq_dma_copy_4k(src_lane + static_cast<int64_t>(jj) * 1024, ring_base + tile * kDqTileBytes); };
+    int cw = -1, ow = -1;
+    uint64_t cbits = 0ull, obits = 0ull;
+    auto next_common = [&]() -> int {
+        while (cbits == 0ull) {
+            if (++cw >= nw) return -1;
+            cbits = dq_uniform_u64(com[cw]);
+        }
+        const int bit = __builtin_ctzll(cbits);
+        cbits &= cbits - 1ull;
+        return cw * 64 + bit;
+    };
+    auto next_own = [&]() -> int {
+        while (obits == 0ull) {
+            if (++ow >= nw) return -1;
+            obits = dq_uniform_u64(own[ow]);
+        }
+        const int bit = __builtin_ctzll(obits);
+        obits &= obits - 1ull;
+        return ow * 64 + bit;
+    };
+    const int64_t img0 = slot0 * kImageElems + lane * 8;
+    uint4* mine = reinterpret_cast<uint4*>(smem_raw + 2 * kDqTileBytes + wave * 8192) + lane;     // 32 keys of K: 8 fragments
+    const unsigned char* mine_tr = smem_raw + 2 * kDqTileBytes + wave * 8192 + tr_lane;
+    bf16x8 kreg[16], vreg[16];
+    int jp = live ? next_own() : -1;
+    if (jp >= 0) {
+        const bf16_bits* ksrc = p.kimg + img0 + static_cast<int64_t>(jp) * kImageElems;
 #pragma unroll
-        for (int c = 0; c < 4; ++c) asm volatile("" : "+v"(qf[c]), "+v"(dof[c]));
-        asm volatile("" : "+v"(lse2), "+v"(dsum));
-        int j0 = next_common();
-        int j1 = j0 >= 0 ? next_common() : -1;
-        if (j0 >= 0) issue(j0, 0);
-        if (j1 >= 0) issue(j1, 1);
-        int tile = 0;
-        while (j0 >= 0) {
-            if (j1 >= 0) __builtin_amdgcn_s_waitcnt(0x0F74); else __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(4) / vmcnt(0)
-            __syncthreads();                                   // block j0 is in LDS for everyone; tile (tile + 2) % 3 is free
-            const int j2 = j1 >= 0 ? next_common() : -1;
-            if (j2 >= 0) issue(j2, tile >= 1 ? tile - 1 : 2);
+        for (int f = 0; f < 16; ++f) kreg[f] = *reinterpret_cast<const bf16x8*>(ksrc + f * 512);
+    }
+    // All ordinary loads so far land before the first LDS-DMA.  From here on the compiler's wait counts know nothing
+    // of the DMA loads; they stay correct because loads complete in order, and the waits written by hand below
+    // count the ordinary loads that may be younger than the DMA they wait for.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int c = 0; c < 4; ++c) asm volatile("" : "+v"(qf[c]), "+v"(dof[c]));
+#pragma unroll
+    for (int f = 0; f < 16; ++f) asm volatile("" : "+v"(kreg[f]));
+    asm volatile("" : "+v"(lse2), "+v"(dsum));
+    int j0 = next_common();
+    if (j0 >= 0) issue(j0, 0);
+    int tile = 0;
+    bool k_ahead = false;                                      // the coming own block's 16 K-fragment loads were issued last turn
+    while (j0 >= 0 || jp >= 0) {
+        if (j0 >= 0) {                                         // uniform over the workgroup
+            // younger than this wavefront's 4 DMA loads of block j0: last turn's 16 K loads
+            if (k_ahead) asm volatile("s_waitcnt vmcnt(16)" ::: "memory"); else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();                                   // block j0 is in LDS for everyone; the other tile is free
+            const int j1 = next_common();
+            if (j1 >= 0) issue(j1, tile ^ 1);
             if (live) {
                 const uint4* kb = ring + tile * 2048 + lane;
                 const uint4* vb = kb + 1024;
@@ -195,23 +221,35 @@ void bwd_dq_hybrid_kernel(const BwdParams p, const DqExtra x) {
                 for (int kt = 0; kt < 4; ++kt) {
                     s[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
                     dp[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                    for (int c = 0; c < 4; ++c) {
-                        const uint4 kraw = kb[(kt * 4 + c) * 64], vraw = vb[(kt * 4 + c) * 64];
-                        bf16x8 kf, vf;
-                        __builtin_memcpy(&kf, &kraw, 16);
-                        __builtin_memcpy(&vf, &vraw, 16);
-                        s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[c], s[kt], 0, 0, 0);
-                        dp[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, dof[c], dp[kt], 0, 0, 0);
-                    }
                 }
+                // vreg is free between own blocks: it stages 16 fragments at a time
+#pragma unroll
+                for (int f = 0; f < 16; ++f) {
+                    const uint4 raw = kb[f * 64];
+                    __builtin_memcpy(&vreg[f], &raw, 16);
+                }
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+#pragma unroll
+                    for (int kt = 0; kt < 4; ++kt)
+                        s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg[kt * 4 + c], qf[c], s[kt], 0, 0, 0);
+#pragma unroll
+                for (int f = 0; f < 16; ++f) {
+                    const uint4 raw = vb[f * 64];
+                    __builtin_memcpy(&vreg[f], &raw, 16);
+                }
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+#pragma unroll
+                    for (int kt = 0; kt < 4; ++kt)
+                        dp[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg[kt * 4 + c], dof[c], dp[kt], 0, 0, 0);
                 bf16x8 dsf[2];
                 ds_tile(s, dp, dsf, (j0 == last_blk) ? last_key - j0 * kBlockN : kBlockN, g, p.scale_log2, lse2, dsum);
                 const unsigned char* ktile = reinterpret_cast<const unsigned char*>(ring + tile * 2048) + tr_lane;
 #pragma unroll
-                for (int dt = 0; dt < 8; ++dt)
+                for (int cc = 0; cc < 2; ++cc)
 #pragma unroll
-                    for (int cc = 0; cc < 2; ++cc) {
+                    for (int dt = 0; dt < 8; ++dt) {
                         // K image unit (kt2, c, g', r') sits at ((kt2 * 4 + c) * 64 + g' * 16 + r') * 16 bytes
                         const unsigned char* at = ktile + ((2 * cc) * 4 + (dt >> 1)) * 1024 + (dt & 1) * 512;
                         const short4q lo = dq_read_tr(at), hi = dq_read_tr(at + 4096);
@@ -222,94 +260,72 @@ void bwd_dq_hybrid_kernel(const BwdParams p, const DqExtra x) {
                     }
             }
             j0 = j1;
-            j1 = j2;
-            tile = tile == 2 ? 0 : tile + 1;
+            tile ^= 1;
         }
-    }
-    __syncthreads();                                           // the ring is dead: its memory becomes 8 private K tiles
-    if (!live) return;                                         // no barrier below
-
-    // ---- phase 2: this token's own blocks ----
-    // K and V (K-image order) of the next block are prefetched into registers while the current block computes.
-    // The K fragments feed S from registers and are also parked in this wavefront's private 16 KiB LDS tile, from
-    // which dQ's K^T operand is a transposed read: the block costs 32 KiB of global loads, not 48.
-    {
-        const int row_words = last_blk < 0 ? 0 : (mrow ? ((last_blk >> 6) + 1 < p.n64_fwd ? (last_blk >> 6) + 1 : p.n64_fwd) : (last_blk >> 6) + 1);
-        int w = -1;
-        uint64_t bits = 0ull;
-        auto next_own = [&]() -> int {
-            while (bits == 0ull) {
-                if (++w >= row_words) return -1;
-                uint64_t v = mrow ? mrow[w] : ~0ull;
-                if (w == (last_blk >> 6)) {
-                    const int tb = last_blk & 63;
-                    v &= (tb == 63) ? ~0ull : ((1ull << (tb + 1)) - 1ull);
-                }
-                if (w < nw) v &= ~com[w];
-                bits = dq_uniform_u64(v);
-            }
-            const int bit = __builtin_ctzll(bits);
-            bits &= bits - 1ull;
-            return w * 64 + bit;
-        };
-        const int64_t img0 = slot0 * kImageElems + lane * 8;
-        uint4* mine = reinterpret_cast<uint4*>(smem_raw + wave * 16384) + lane;
-        const unsigned char* mine_tr = smem_raw + wave * 16384 + tr_lane;
-        bf16x8 kreg[16], vreg[16];
-        int j = next_own();
-        if (j >= 0) {
-            const bf16_bits* ksrc = p.kimg + img0 + static_cast<int64_t>(j) * kImageElems;
-            const bf16_bits* vsrc = p.vimg_r + img0 + static_cast<int64_t>(j) * kImageElems;
+        k_ahead = false;
+        if (jp >= 0) {                                         // per wavefront
+            {
+                const bf16_bits* vsrc = p.vimg_r + img0 + static_cast<int64_t>(jp) * kImageElems;
 #pragma unroll
-            for (int f = 0; f < 16; ++f) {
-                kreg[f] = *reinterpret_cast<const bf16x8*>(ksrc + f * 512);
-                vreg[f] = *reinterpret_cast<const bf16x8*>(vsrc + f * 512);
-            }
-        }
-        while (j >= 0) {
-#pragma unroll
-            for (int f = 0; f < 16; ++f) {
-                uint4 raw;
-                __builtin_memcpy(&raw, &kreg[f], 16);
-                mine[f * 64] = raw;
+                for (int f = 0; f < 16; ++f) vreg[f] = *reinterpret_cast<const bf16x8*>(vsrc + f * 512);
             }
             floatx4 s[4], dp[4];
 #pragma unroll
             for (int kt = 0; kt < 4; ++kt) {
                 s[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
                 dp[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
+            }
 #pragma unroll
-                for (int c = 0; c < 4; ++c) {
+            for (int c = 0; c < 4; ++c)
+#pragma unroll
+                for (int kt = 0; kt < 4; ++kt)
                     s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[kt * 4 + c], qf[c], s[kt], 0, 0, 0);
+#pragma unroll
+            for (int f = 0; f < 8; ++f) {                      // keys 0..31 of K -> private tile
+                uint4 raw;
+                __builtin_memcpy(&raw, &kreg[f], 16);
+                mine[f * 64] = raw;
+            }
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+#pragma unroll
+                for (int kt = 0; kt < 4; ++kt)
                     dp[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg[kt * 4 + c], dof[c], dp[kt], 0, 0, 0);
-                }
-            }
-            const int jn = next_own();
-            if (jn >= 0) {
-                const bf16_bits* ksrc = p.kimg + img0 + static_cast<int64_t>(jn) * kImageElems;
-                const bf16_bits* vsrc = p.vimg_r + img0 + static_cast<int64_t>(jn) * kImageElems;
-#pragma unroll
-                for (int f = 0; f < 16; ++f) {
-                    kreg[f] = *reinterpret_cast<const bf16x8*>(ksrc + f * 512);
-                    vreg[f] = *reinterpret_cast<const bf16x8*>(vsrc + f * 512);
-                }
-            }
             bf16x8 dsf[2];
-            ds_tile(s, dp, dsf, (j == last_blk) ? last_key - j * kBlockN : kBlockN, g, p.scale_log2, lse2, dsum);
+            ds_tile(s, dp, dsf, (jp == last_blk) ? last_key - jp * kBlockN : kBlockN, g, p.scale_log2, lse2, dsum);
 #pragma unroll
-            for (int dt = 0; dt < 8; ++dt)
+            for (int cc = 0; cc < 2; ++cc) {
+                if (cc == 1) {
 #pragma unroll
-                for (int cc = 0; cc < 2; ++cc) {
-                    const unsigned char* at = mine_tr + ((2 * cc) * 4 + (dt >> 1)) * 1024 + (dt & 1) * 512;
+                    for (int f = 0; f < 8; ++f) {              // keys 32..63 (LDS executes a wavefront's accesses in order)
+                        uint4 raw;
+                        __builtin_memcpy(&raw, &kreg[8 + f], 16);
+                        mine[f * 64] = raw;
+                    }
+                }
+#pragma unroll
+                for (int dt = 0; dt < 8; ++dt) {
+                    const unsigned char* at = mine_tr + (dt >> 1) * 1024 + (dt & 1) * 512;
                     const short4q lo = dq_read_tr(at), hi = dq_read_tr(at + 4096);
                     bf16x8 kt_f;
                     __builtin_memcpy(&kt_f, &lo, 8);
                     __builtin_memcpy(reinterpret_cast<unsigned char*>(&kt_f) + 8, &hi, 8);
                     dq[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kt_f, dsf[cc], dq[dt], 0, 0, 0);
                 }
-            j = jn;
+            }
+            // the K fragments of the next own block go out last: they are the only ordinary loads in flight when the
+            // next turn waits for its DMA
+            const int jn = next_own();
+            if (jn >= 0) {
+                const bf16_bits* ksrc = p.kimg + img0 + static_cast<int64_t>(jn) * kImageElems;
+#pragma unroll
+                for (int f = 0; f < 16; ++f) kreg[f] = *reinterpret_cast<const bf16x8*>(ksrc + f * 512);
+                k_ahead = true;
+            }
+            jp = jn;
         }
     }
+    if (!live) return;
 
     bf16_bits* op = p.dq + tok * p.dq_tok + h * p.dq_kvh + n * p.dq_grp + 4 * g;
 #pragma unroll
@@ -327,10 +343,11 @@ int launch_bwd_dq_hybrid(hipStream_t st, const BwdParams& p, int batch, int max_
     x.groups_per_seq = (max_seqlen_q + kDqTokens - 1) / kDqTokens;
     const int64_t total = static_cast<int64_t>(p.num_heads_k) * batch * x.groups_per_seq;
     IV2_CHECK(total <= 0x3fffffff, "varlen_bwd: too many token groups");
+    IV2_CHECK(p.k_blocks <= kDqMaskWords * 64, "varlen_bwd: more than %d key blocks per sequence", kDqMaskWords * 64);
     x.total_groups = static_cast<int>(total);
     const int64_t per_round = 8 * kDqChunk;
     const int64_t grid = (total + per_round - 1) / per_round * per_round;
-    const size_t lds = kDqLdsTiles + kDqMaskWords * 8;
+    const size_t lds = kDqLdsTiles + (1 + kDqTokens) * kDqMaskWords * 8;
     const void* fn = causal ? reinterpret_cast<const void*>(&bwd_dq_hybrid_kernel<true>)
                             : reinterpret_cast<const void*>(&bwd_dq_hybrid_kernel<false>);
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
