@@ -287,8 +287,6 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
         const float4 Db = *reinterpret_cast<const float4*>(scal + 80 + 4 * g);
         const float lse_a[4] = {la.x, la.y, la.z, la.w};
         const float lse_b[4] = {lb.x, lb.y, lb.z, lb.w};
-        const float D_a[4] = {Da.x, Da.y, Da.z, Da.w};
-        const float D_b[4] = {Db.x, Db.y, Db.z, Db.w};
         const bool edge = (lim_a < kBlockN - 1) || (lim_b < kBlockN - 1);
 
         // Four phases, each 32 MFMAs, with the VALU work of the softmax backward hidden behind the matrix pipeline:
@@ -299,10 +297,12 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
         const uint4* frag = reinterpret_cast<const uint4*>(st) + frag_unit;      // tile t, chunk c at frag[t * 256 + c * 64]
         bf16x8 pfr[4], dsfr[4];                                // per key tile: [token a heads 4g..4g+3 | token b heads 4g..4g+3]
         floatx4 sa[4], sb[4], dpa[4], dpb[4];
+        // the dP accumulators start at -D, so that dS = P (dP - D) is one multiplication per element
+        const floatx4 negD_a = {-Da.x, -Da.y, -Da.z, -Da.w}, negD_b = {-Db.x, -Db.y, -Db.z, -Db.w};
 #pragma unroll
         for (int kt = 0; kt < 4; ++kt) {
             sa[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
-            sb[kt] = sa[kt]; dpa[kt] = sa[kt]; dpb[kt] = sa[kt];
+            sb[kt] = sa[kt]; dpa[kt] = negD_a; dpb[kt] = negD_b;
         }
         {   // A
             uint4 fr[2][2];
@@ -337,20 +337,30 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
                 }
                 {   // P of key tile c, kept in fp32 in place of S
                     const int kt = c;
-                    const int nlim_a = lim_a - 16 * kt, nlim_b = lim_b - 16 * kt;
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         float xa = __builtin_amdgcn_exp2f(sa[kt][e] * p.scale_log2 - lse_a[e]);
                         float xb = __builtin_amdgcn_exp2f(sb[kt][e] * p.scale_log2 - lse_b[e]);
-                        if (edge) {
-                            xa = n > nlim_a ? 0.f : xa;
-                            xb = n > nlim_b ? 0.f : xb;
-                        }
                         sa[kt][e] = xa;
                         sb[kt][e] = xb;
                         pfr[kt][e] = static_cast<__bf16>(xa);
                         pfr[kt][4 + e] = static_cast<__bf16>(xb);
                     }
+                }
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (edge) {
+            // a block cut by the causal diagonal or by the sequence end (rare): keys beyond the limit get P = 0
+#pragma unroll
+            for (int kt = 0; kt < 4; ++kt) {
+                const bool off_a = n > lim_a - 16 * kt, off_b = n > lim_b - 16 * kt;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    sa[kt][e] = off_a ? 0.f : sa[kt][e];
+                    sb[kt][e] = off_b ? 0.f : sb[kt][e];
+                    pfr[kt][e] = static_cast<__bf16>(sa[kt][e]);
+                    pfr[kt][4 + e] = static_cast<__bf16>(sb[kt][e]);
                 }
             }
         }
@@ -372,8 +382,8 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
                     const int kt = dt >> 1, e0 = (dt & 1) * 2;
 #pragma unroll
                     for (int e = e0; e < e0 + 2; ++e) {
-                        dsfr[kt][e] = static_cast<__bf16>(sa[kt][e] * (dpa[kt][e] - D_a[e]));
-                        dsfr[kt][4 + e] = static_cast<__bf16>(sb[kt][e] * (dpb[kt][e] - D_b[e]));
+                        dsfr[kt][e] = static_cast<__bf16>(sa[kt][e] * dpa[kt][e]);
+                        dsfr[kt][4 + e] = static_cast<__bf16>(sb[kt][e] * dpb[kt][e]);
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);
