@@ -58,16 +58,26 @@ __device__ __forceinline__ short4q dq_read_tr(const unsigned char* ptr) {
 }
 
 // dS^T of one block as the B operand of dQ^T = K^T dS^T, from the S^T and dP^T accumulators
+// dS^T of one block as the B operand of dQ^T += K^T dS^T.  The dP accumulators were started at -D, so dp holds dP - D.
+// lim: last in-block key index the token may see (>= 63 for a whole block, which is the common case).
 __device__ __forceinline__ void ds_tile(const floatx4 (&s)[4], const floatx4 (&dp)[4], bf16x8 (&dsf)[2], int lim, int g,
-                                        float scale_log2, float lse2, float dsum) {
+                                        float scale_log2, float lse2) {
+    if (lim >= kBlockN - 1) {                                  // uniform per wavefront
 #pragma unroll
-    for (int kt = 0; kt < 4; ++kt)
+        for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            float pv = __builtin_amdgcn_exp2f(s[kt][e] * scale_log2 - lse2);
-            if (16 * kt + 4 * g + e > lim) pv = 0.f;
-            dsf[kt >> 1][(kt & 1) * 4 + e] = static_cast<__bf16>(pv * (dp[kt][e] - dsum));
-        }
+            for (int e = 0; e < 4; ++e)
+                dsf[kt >> 1][(kt & 1) * 4 + e] = static_cast<__bf16>(__builtin_amdgcn_exp2f(s[kt][e] * scale_log2 - lse2) * dp[kt][e]);
+    } else {
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float pv = __builtin_amdgcn_exp2f(s[kt][e] * scale_log2 - lse2);
+                if (16 * kt + 4 * g + e > lim) pv = 0.f;
+                dsf[kt >> 1][(kt & 1) * 4 + e] = static_cast<__bf16>(pv * dp[kt][e]);
+            }
+    }
 }
 
 template <bool kCausal>
@@ -146,6 +156,7 @@ void bwd_dq_hybrid_kernel(const BwdParams p, const DqExtra x) {
     }
     float lse2 = p.lse[h * p.lse_kvh + tok * p.lse_tok + n * p.lse_grp] * kLog2e;
     float dsum = p.dsum[static_cast<int64_t>(h) * p.total_q * 16 + tok * 16 + n];
+    const floatx4 neg_dsum = {-dsum, -dsum, -dsum, -dsum};     // the dP accumulators start here: dS = P (dP - D) is then one product
     floatx4 dq[8];
 #pragma unroll
     for (int dt = 0; dt < 8; ++dt) dq[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -220,7 +231,7 @@ void bwd_dq_hybrid_kernel(const BwdParams p, const DqExtra x) {
 #pragma unroll
                 for (int kt = 0; kt < 4; ++kt) {
                     s[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
-                    dp[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
+                    dp[kt] = neg_dsum;
                 }
                 // vreg is free between own blocks: it stages 16 fragments at a time
 #pragma unroll
@@ -244,7 +255,7 @@ void bwd_dq_hybrid_kernel(const BwdParams p, const DqExtra x) {
                     for (int kt = 0; kt < 4; ++kt)
                         dp[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg[kt * 4 + c], dof[c], dp[kt], 0, 0, 0);
                 bf16x8 dsf[2];
-                ds_tile(s, dp, dsf, (j0 == last_blk) ? last_key - j0 * kBlockN : kBlockN, g, p.scale_log2, lse2, dsum);
+                ds_tile(s, dp, dsf, (j0 == last_blk) ? last_key - j0 * kBlockN : kBlockN - 1, g, p.scale_log2, lse2);
                 const unsigned char* ktile = reinterpret_cast<const unsigned char*>(ring + tile * 2048) + tr_lane;
 #pragma unroll
                 for (int cc = 0; cc < 2; ++cc)
@@ -273,7 +284,7 @@ void bwd_dq_hybrid_kernel(const BwdParams p, const DqExtra x) {
 #pragma unroll
             for (int kt = 0; kt < 4; ++kt) {
                 s[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
-                dp[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
+                dp[kt] = neg_dsum;
             }
 #pragma unroll
             for (int c = 0; c < 4; ++c)
@@ -292,7 +303,7 @@ void bwd_dq_hybrid_kernel(const BwdParams p, const DqExtra x) {
                 for (int kt = 0; kt < 4; ++kt)
                     dp[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg[kt * 4 + c], dof[c], dp[kt], 0, 0, 0);
             bf16x8 dsf[2];
-            ds_tile(s, dp, dsf, (jp == last_blk) ? last_key - jp * kBlockN : kBlockN, g, p.scale_log2, lse2, dsum);
+            ds_tile(s, dp, dsf, (jp == last_blk) ? last_key - jp * kBlockN : kBlockN - 1, g, p.scale_log2, lse2);
 #pragma unroll
             for (int cc = 0; cc < 2; ++cc) {
                 if (cc == 1) {
