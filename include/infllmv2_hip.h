@@ -124,6 +124,22 @@ int infllmv2_varlen_fwd_stage1(void* stream, const void* q, const void* k, const
                                const int64_t* v_strides, int64_t score_head_stride,
                                int64_t score_row_stride, float softmax_scale, int is_causal);
 
+/* Stage 1 and the max-pooling onto key blocks in one launch: what infllmv2_max_pooling_1d(_varlen) returns for the
+ * score tensor of infllmv2_varlen_fwd_stage1, bit for bit, without that tensor ever reaching memory.  Replaces the
+ * caller's pair of calls `infllmv2_attn_stage1` (infllm_v2/infllmv2_sparse_attention.py:483-606) followed by
+ * `max_pooling_1d` / `max_pooling_1d_varlen` (infllm_v2/max_pooling_1d.py:4-46, 49-137; csrc/max_pooling_1d.cuh:12-160)
+ * for the pooling window those callers use (kernel 5, stride 4, padding 1 on 64-token blocks; anything else is
+ * rejected).  q/k/v, cu_seqlens and strides as in infllmv2_varlen_fwd_stage1; cache_lens (batch) or null with one
+ * cache_len for all sequences; pooled (Hk, total_q, out_len) bf16, dense. */
+int infllmv2_varlen_fwd_stage1_pooled(void* stream, const void* q, const void* k, const void* v, void* pooled,
+                                      const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                                      const int32_t* cu_seqlens_v, const int32_t* cache_lens, int cache_len,
+                                      int batch, int64_t total_q, int num_heads, int num_heads_k, int head_dim,
+                                      int max_seqlen_q, int max_seqlen_k, const int64_t* q_strides,
+                                      const int64_t* k_strides, const int64_t* v_strides, int out_len,
+                                      float softmax_scale, int is_causal, int kernel_size, int stride, int padding,
+                                      int block_size, int local_blocks, int init_blocks);
+
 /* ---- Stage 2: block-sparse attention -------------------------------------------------------- */
 
 /* Scratch needed by infllmv2_varlen_fwd / _bwd for the fragment-major K/V block images. */

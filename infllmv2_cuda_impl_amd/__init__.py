@@ -12,11 +12,13 @@ from .selection import topk_blocks
 from .attention import (
     infllmv2_attn_varlen_func,
     infllmv2_attn_stage1,
+    infllmv2_attn_stage1_pooled,
     infllmv2_attn_with_kvcache,
 )
 
 __all__ = [
     "blockmask_to_uint64", "topk_to_uint64", "uint64_to_bool", "transpose_blockmask",
     "max_pooling_1d", "max_pooling_1d_varlen", "topk_blocks",
-    "infllmv2_attn_varlen_func", "infllmv2_attn_stage1", "infllmv2_attn_with_kvcache",
+    "infllmv2_attn_varlen_func", "infllmv2_attn_stage1", "infllmv2_attn_stage1_pooled",
+    "infllmv2_attn_with_kvcache",
 ]

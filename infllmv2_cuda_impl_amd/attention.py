@@ -212,6 +212,39 @@ def infllmv2_attn_stage1(q, k, v, cu_seqlens_q, cu_seqlens_k, cu_seqlens_v, max_
                          softmax_scale, causal)
 
 
+def infllmv2_attn_stage1_pooled(q, k, v, cu_seqlens_q, cu_seqlens_k, cu_seqlens_v, max_seqlen_q, max_seqlen_k,
+                                local_blocks, init_blocks, cache_lens=None, cache_len=0, max_cache_len=None,
+                                block_size=64, stride=16, softmax_scale=None, causal=False):
+    """Stage-1 scoring and the max-pooling onto key blocks, fused (no counterpart in the reference's API).
+
+    Returns exactly what ``max_pooling_1d(infllmv2_attn_stage1(...), cache_len, local_blocks, init_blocks)`` (one
+    sequence, ``cache_lens`` None) or ``max_pooling_1d_varlen(infllmv2_attn_stage1(...), cu_seqlens_q, cu_seqlens_k,
+    cache_lens, max_seqlen_q, max_seqlen_k, local_blocks, init_blocks)`` (packed) return, bit for bit, in one
+    launch and without materialising the ``(nheads_k, total_q, max_seqlen_k)`` score tensor: bf16
+    ``(nheads_k, total_q, ceil((max_seqlen_q + cache) / block_size))`` with ``cache`` = ``cache_len`` or
+    ``max(cache_lens)`` (pass ``max_cache_len`` to avoid the host read).  Only ``block_size`` 64 over stride-16
+    compressed keys is fused.
+    """
+    from .stage1 import stage1_pooled
+    if softmax_scale is None:
+        softmax_scale = q.shape[-1] ** (-0.5)
+    q, k, v = [_dense_last_dim(x) for x in (q, k, v)]
+    _check_qkv(q, k, v, cu_seqlens_q, cu_seqlens_k, same_kv_len=False)
+    if cu_seqlens_v.dtype != torch.int32:
+        raise RuntimeError("cu_seqlens_v must have dtype int32")
+    if cache_lens is not None:
+        if max_cache_len is None:
+            max_cache_len = int(cache_lens.max().item()) if cache_lens.numel() > 0 else 0
+    else:
+        if cu_seqlens_q.numel() != 2:
+            raise RuntimeError("packed sequences need cache_lens (as max_pooling_1d_varlen does)")
+        max_cache_len = cache_len
+    out_len = (max_seqlen_q + max_cache_len + block_size - 1) // block_size
+    return stage1_pooled(q, k, v, cu_seqlens_q, cu_seqlens_k, cu_seqlens_v, max_seqlen_q, max_seqlen_k,
+                         softmax_scale, causal, out_len, cache_lens, cache_len, local_blocks, init_blocks,
+                         block_size, stride)
+
+
 def infllmv2_attn_with_kvcache(q, k_cache, v_cache, k=None, v=None, rotary_cos=None, rotary_sin=None,
                                cache_seqlens: Optional[Union[int, torch.Tensor]] = None,
                                cache_batch_idx: Optional[torch.Tensor] = None,

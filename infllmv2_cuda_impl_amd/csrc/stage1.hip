@@ -19,6 +19,7 @@
 // in MFMA-operand order (conflict-free ds_read_b128) and reused by all 16 tokens, and inside a
 // wavefront one operand read feeds four MFMAs.
 #include "common.h"
+#include "block_walker.h"
 #include "../../include/infllmv2_hip.h"
 #include <math.h>
 
@@ -28,7 +29,7 @@ struct Stage1Params {
     const bf16_bits* q;
     const bf16_bits* k;              // fine compressed keys   (sum Lk, Hk, d)
     const bf16_bits* c;              // coarse compressed keys (sum Lc, Hk, d)
-    bf16_bits* score;                // (Hk, total_q, row_stride)
+    bf16_bits* score;                // (Hk, total_q, row_stride); pooled output: (Hk, total_q, pool_len), dense
     const int* cu_seqlens_q;
     const int* cu_seqlens_k;
     const int* cu_seqlens_c;
@@ -38,11 +39,17 @@ struct Stage1Params {
     int score_cols;                  // columns to define in every row (max_seqlen_k)
     float scale_log2;
     int causal;
+    // pooled output only
+    const int* cache_lens;           // per sequence, or null: cache_len for all
+    int cache_len;
+    int pool_len;                    // key blocks per output row
+    int local_blocks, init_blocks;
 };
 
 constexpr int kTokPerWave = 4;
 constexpr int kWavesS1 = 4;
 constexpr int kTokPerBlock = kTokPerWave * kWavesS1;   // 16
+constexpr int kKeysPerBlock = 4;                       // compressed keys (stride 16) per 64-token key block
 
 __device__ __forceinline__ int trunc_div(int a, int b) { return a / b; }   // C++ semantics on purpose
 
@@ -77,7 +84,30 @@ __device__ __forceinline__ void store_tile_lds(const uint4 (&r)[4], uint4* lds, 
     }
 }
 
-template <bool kCausal>
+// x, y -> (x's even 16-lane rows interleaved with y's even rows, x's odd rows interleaved with y's odd rows), summed:
+// row 2r of the result is x.row(2r) + x.row(2r+1), row 2r+1 is y.row(2r) + y.row(2r+1).
+__device__ __forceinline__ float fold_rows16(float x, float y) {
+    typedef unsigned u2 __attribute__((ext_vector_type(2)));
+    const u2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(y), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+// rows 0,1 of the result are x.row(r) + x.row(r+2), rows 2,3 are y.row(r-2) + y.row(r)
+__device__ __forceinline__ float fold_rows32(float x, float y) {
+    typedef unsigned u2 __attribute__((ext_vector_type(2)));
+    const u2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(y), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float dpp_quad_xor1(float x) {
+    return __uint_as_float(__builtin_amdgcn_mov_dpp(__float_as_uint(x), 0xB1, 0xF, 0xF, false));    // quad_perm:[1,0,3,2]
+}
+__device__ __forceinline__ float dpp_quad_xor2(float x) {
+    return __uint_as_float(__builtin_amdgcn_mov_dpp(__float_as_uint(x), 0x4E, 0xF, 0xF, false));    // quad_perm:[2,3,0,1]
+}
+
+// kPool: instead of the score rows, write their 1-D max-pooling onto 64-token key blocks (window of 5 compressed
+// keys, stride 4, padding 1, forced blocks +inf, empty windows -inf: the rule of csrc/max_pooling_1d.cuh:12-160
+// applied to the scores this kernel would have written, which never reach memory).
+template <bool kCausal, bool kPool>
 __global__ __launch_bounds__(256)
 void stage1_kernel(const Stage1Params p) {
     __shared__ uint4 tile[2][1024];                            // two 16 KiB operand-ordered key tiles
@@ -87,7 +117,8 @@ void stage1_kernel(const Stage1Params p) {
     const int b = blockIdx.y, h = blockIdx.z;
     const int q0 = p.cu_seqlens_q[b];
     const int Sq = p.cu_seqlens_q[b + 1] - q0;
-    const int tok_block0 = blockIdx.x * kTokPerBlock;
+    // late tokens see the most keys: they go first, so the long workgroups do not form the tail of the launch
+    const int tok_block0 = (static_cast<int>(gridDim.x) - 1 - static_cast<int>(blockIdx.x)) * kTokPerBlock;
     if (tok_block0 >= Sq) return;                              // uniform per workgroup
     const int k0 = p.cu_seqlens_k[b], Lk = p.cu_seqlens_k[b + 1] - k0;
     const int c0 = p.cu_seqlens_c[b], Lc = p.cu_seqlens_c[b + 1] - c0;
@@ -96,6 +127,7 @@ void stage1_kernel(const Stage1Params p) {
     const int tok0 = tok_block0 + wave * kTokPerWave;          // first token of this wavefront
     int vis_f[kTokPerWave], vis_c[kTokPerWave];
     bool live[kTokPerWave];
+    int min_vis_c = 0x7fffffff;
 #pragma unroll
     for (int t = 0; t < kTokPerWave; ++t) {
         const int i = tok0 + t;
@@ -103,6 +135,8 @@ void stage1_kernel(const Stage1Params p) {
         vis_f[t] = live[t] ? stage1_visible(i, 16, Lk, Sq, kCausal) : 0;
         vis_c[t] = live[t] ? stage1_visible(i, s1, Lc, Sq, kCausal) : 0;
         if (vis_c[t] == 0) vis_f[t] = 0;                       // early exit of flash_fwd_kernel.h:1271-1276
+        if (kPool && vis_f[t] > p.score_cols) vis_f[t] = p.score_cols;               // the score row the pooling would have read ends there
+        min_vis_c = vis_c[t] < min_vis_c ? vis_c[t] : min_vis_c;
     }
     // tile counts are taken over the whole workgroup (its last live token sees the most keys)
     const int i_last = (tok_block0 + kTokPerBlock - 1 < Sq ? tok_block0 + kTokPerBlock - 1 : Sq - 1);
@@ -111,7 +145,7 @@ void stage1_kernel(const Stage1Params p) {
     const int tiles_c = (wg_vis_c + 63) >> 6;
     const int tiles_f = (wg_vis_f + 63) >> 6;
 
-    // Q as the A operand: lane (row = head n... here r = lane % 16 is the head, g the k-group)
+    // Q as the A operand: r = lane % 16 is the head, g the k-group
     bf16x8 qf[kTokPerWave][4];
 #pragma unroll
     for (int t = 0; t < kTokPerWave; ++t) {
@@ -155,18 +189,20 @@ void stage1_kernel(const Stage1Params p) {
                     s[t][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[t][c], kf, s[t][kt], 0, 0, 0);
             }
         }
+        // only the tile that holds a token's last visible key needs the per-key test
+        const bool cut = (ti + 1) * 64 > min_vis_c;            // uniform per wavefront
 #pragma unroll
         for (int t = 0; t < kTokPerWave; ++t) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 float v[4];
-                float mx = -INFINITY;
 #pragma unroll
-                for (int kt = 0; kt < 4; ++kt) {
-                    const int j = ti * 64 + kt * 16 + n;
-                    v[kt] = (j < vis_c[t]) ? s[t][kt][e] * p.scale_log2 : -INFINITY;
-                    mx = fmaxf(mx, v[kt]);
+                for (int kt = 0; kt < 4; ++kt) v[kt] = s[t][kt][e] * p.scale_log2;
+                if (cut) {
+#pragma unroll
+                    for (int kt = 0; kt < 4; ++kt) v[kt] = (ti * 64 + kt * 16 + n < vis_c[t]) ? v[kt] : -INFINITY;
                 }
+                const float mx = fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3]));
                 const float m_new = fmaxf(m[t][e], mx);
                 const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
                 float acc = l[t][e] * __builtin_amdgcn_exp2f(m[t][e] - m_use);
@@ -205,17 +241,32 @@ void stage1_kernel(const Stage1Params p) {
     }
     __syncthreads();
     bf16_bits* out_rows[kTokPerWave];
+    int bq[kTokPerWave];                                       // pooled output: the key block the token itself sits in
+    float carry[kTokPerWave];                                  // pooled output: score of the last key of the previous tile
+    {
+        const int cache_len = kPool ? (p.cache_lens ? p.cache_lens[b] : p.cache_len) : 0;
 #pragma unroll
-    for (int t = 0; t < kTokPerWave; ++t)
-        out_rows[t] = p.score + h * p.score_head_stride + (static_cast<int64_t>(q0) + tok0 + t) * p.score_row_stride;
+        for (int t = 0; t < kTokPerWave; ++t) {
+            const int64_t row = static_cast<int64_t>(q0) + tok0 + t;
+            out_rows[t] = kPool ? p.score + (static_cast<int64_t>(h) * p.score_head_stride + row * p.pool_len)
+                                : p.score + h * p.score_head_stride + row * p.score_row_stride;
+            bq[t] = (tok0 + t + cache_len) / kBlockN;
+            carry[t] = 0.f;
+        }
+    }
+    // value of a pooled entry that no visible key reaches
+    auto pool_rest = [&](int kb, int bq_t, float reached) -> bf16_bits {
+        const bool forced = (kb < p.init_blocks) || (bq_t >= kb && bq_t <= kb + p.local_blocks);
+        const int first = kb * kKeysPerBlock - 1;              // first key of the window (before clipping at 0)
+        const bool empty = (first < 0 ? 0 : first) >= (Lk < p.score_cols ? Lk : p.score_cols);
+        return forced ? bf16_bits{0x7f80} : (empty ? bf16_bits{0xff80} : f32_to_bf16(reached));
+    };
 
     for (int ti = 0; ti < tiles_f; ++ti) {
         const bool more = ti + 1 < tiles_f;
         if (more) load_tile_regs(stage, kbase, p.k_row_stride, (ti + 1) * 64, Lk, tid);
         const uint4* cur = tile[ti & 1];
-        float mine[kTokPerWave];                               // the score this lane will store: key 16*g + n
-#pragma unroll
-        for (int t = 0; t < kTokPerWave; ++t) mine[t] = 0.f;
+        float part[kTokPerWave][4];                            // [t][kt]: this lane's four heads summed, key 16 kt + n
 #pragma unroll
         for (int kt = 0; kt < 4; ++kt) {
             floatx4 s[kTokPerWave];
@@ -230,37 +281,112 @@ void stage1_kernel(const Stage1Params p) {
                 for (int t = 0; t < kTokPerWave; ++t)
                     s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[t][c], kf, s[t], 0, 0, 0);
             }
-            const int j = ti * 64 + kt * 16 + n;
 #pragma unroll
             for (int t = 0; t < kTokPerWave; ++t) {
                 float sum = 0.f;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) sum += __builtin_amdgcn_exp2f(s[t][e] * p.scale_log2 - lse2[t][e]);
-                sum = (j < vis_f[t]) ? sum : 0.f;
-                sum += __shfl_xor(sum, 16);
-                sum += __shfl_xor(sum, 32);                    // all four g-groups now hold the 16-head sum
-                if (g == kt) mine[t] = sum;
+                part[t][kt] = sum;
             }
         }
+        const int col = ti * 64 + lane;                        // lane = 16*g + n  <->  key 16*g + n of this tile
 #pragma unroll
         for (int t = 0; t < kTokPerWave; ++t) {
-            const int col = ti * 64 + lane;                    // lane = 16*g + n  <->  key 16*g + n of this tile
-            if (live[t] && col < p.score_cols) out_rows[t][col] = f32_to_bf16(mine[t]);
+            // sum over the four 16-lane rows (the head groups) and hand row kt the total of key tile kt, in three
+            // exchanges: (row0 + row1 | row2 + row3) of tiles 0/1 and of tiles 2/3, then the two halves
+            float mine = fold_rows32(fold_rows16(part[t][0], part[t][1]), fold_rows16(part[t][2], part[t][3]));
+            mine = (col < vis_f[t]) ? mine : 0.f;              // keys the token may not see score 0
+            if (!kPool) {
+                if (live[t] && col < p.score_cols) out_rows[t][col] = f32_to_bf16(mine);
+            } else {
+                // block kb = col / 4 pools keys 4 kb - 1 .. 4 kb + 3: its quad and the last key of the quad before
+                float left = __shfl_up(mine, 1);
+                if (lane == 0) left = carry[t];
+                carry[t] = __shfl(mine, 63);
+                float best = fmaxf(mine, dpp_quad_xor1(mine));
+                best = fmaxf(best, dpp_quad_xor2(best));
+                best = fmaxf(best, left);
+                const int kb = col >> 2;
+                if (live[t] && (lane & 3) == 0 && kb < p.pool_len) out_rows[t][kb] = pool_rest(kb, bq[t], best);
+            }
         }
         if (more) store_tile_lds(stage, tile[(ti + 1) & 1], tid);
         __syncthreads();
     }
-    // columns no tile covered are zero
+    // columns no tile covered
 #pragma unroll
     for (int t = 0; t < kTokPerWave; ++t) {
         if (!live[t]) continue;
-        for (int col = tiles_f * 64 + lane; col < p.score_cols; col += 64) out_rows[t][col] = 0;
+        if (!kPool) {
+            for (int col = tiles_f * 64 + lane; col < p.score_cols; col += 64) out_rows[t][col] = 0;
+        } else {
+            // the first of them still sees the last key of the last tile
+            for (int kb = tiles_f * 16 + lane; kb < p.pool_len; kb += 64)
+                out_rows[t][kb] = pool_rest(kb, bq[t], kb == tiles_f * 16 ? carry[t] : 0.f);
+        }
     }
 }
 
 }  // namespace infllmv2
 
 using namespace infllmv2;
+
+namespace {
+
+struct Stage1Pool {                  // pooled-output mode of the launch below
+    const int32_t* cache_lens;
+    int cache_len, pool_len, local_blocks, init_blocks;
+};
+
+int launch_stage1(const char* who, void* stream, const void* q, const void* k, const void* v, void* out,
+                  const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, const int32_t* cu_seqlens_v, int batch,
+                  int64_t total_q, int num_heads, int num_heads_k, int head_dim, int max_seqlen_q, int max_seqlen_k,
+                  const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                  int64_t out_head_stride, int64_t out_row_stride, float softmax_scale, int is_causal,
+                  const Stage1Pool* pool) {
+    IV2_CHECK(head_dim == kHeadDim, "%s: this build only supports head_dim 128 (got %d)", who, head_dim);
+    IV2_CHECK(num_heads_k > 0 && num_heads == num_heads_k * kGroup,
+              "%s: requires num_heads == 16 * num_heads_k (got %d and %d)", who, num_heads, num_heads_k);
+    IV2_CHECK(batch > 0 && total_q >= 0 && max_seqlen_q >= 0 && max_seqlen_k >= 0, "%s: bad sizes", who);
+    IV2_CHECK(q && k && v && out && cu_seqlens_q && cu_seqlens_k && cu_seqlens_v, "%s: null pointer", who);
+    IV2_CHECK(num_heads_k <= 65535 && batch <= 65535, "%s: batch and num_heads_k must not exceed 65535", who);
+    IV2_CHECK(reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(k) % 16 == 0 &&
+              reinterpret_cast<uintptr_t>(v) % 16 == 0, "%s: q, k, v must be 16-byte aligned", who);
+    for (int s = 0; s < 3; ++s) IV2_CHECK(q_strides[s] % 8 == 0, "%s: q strides must be multiples of 8 elements", who);
+    IV2_CHECK(k_strides[0] % 8 == 0 && k_strides[1] % 8 == 0 && v_strides[0] % 8 == 0 && v_strides[1] % 8 == 0,
+              "%s: k/v strides must be multiples of 8 elements", who);
+    if (total_q == 0 || max_seqlen_q == 0) return 0;
+    Stage1Params p{};
+    p.q = static_cast<const bf16_bits*>(q);
+    p.k = static_cast<const bf16_bits*>(k);
+    p.c = static_cast<const bf16_bits*>(v);
+    p.score = static_cast<bf16_bits*>(out);
+    p.cu_seqlens_q = cu_seqlens_q; p.cu_seqlens_k = cu_seqlens_k; p.cu_seqlens_c = cu_seqlens_v;
+    p.q_tok_stride = q_strides[0]; p.q_grp_stride = q_strides[1]; p.q_kvh_stride = q_strides[2];
+    p.k_row_stride = k_strides[0]; p.k_head_stride = k_strides[1];
+    p.c_row_stride = v_strides[0]; p.c_head_stride = v_strides[1];
+    p.score_head_stride = out_head_stride; p.score_row_stride = out_row_stride;
+    p.score_cols = max_seqlen_k;
+    p.scale_log2 = softmax_scale * 1.44269504088896340736f;
+    p.causal = is_causal;
+    if (pool) {
+        p.cache_lens = pool->cache_lens; p.cache_len = pool->cache_len; p.pool_len = pool->pool_len;
+        p.local_blocks = pool->local_blocks; p.init_blocks = pool->init_blocks;
+    }
+    const dim3 grid((max_seqlen_q + kTokPerBlock - 1) / kTokPerBlock, batch, num_heads_k);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (pool) {
+        if (is_causal) hipLaunchKernelGGL((stage1_kernel<true, true>), grid, dim3(256), 0, st, p);
+        else hipLaunchKernelGGL((stage1_kernel<false, true>), grid, dim3(256), 0, st, p);
+    } else {
+        if (is_causal) hipLaunchKernelGGL((stage1_kernel<true, false>), grid, dim3(256), 0, st, p);
+        else hipLaunchKernelGGL((stage1_kernel<false, false>), grid, dim3(256), 0, st, p);
+    }
+    IV2_LAUNCH_CHECK();
+    return 0;
+}
+
+}  // namespace
 
 extern "C" int infllmv2_varlen_fwd_stage1(void* stream, const void* q, const void* k, const void* v, void* score,
                                           const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
@@ -269,36 +395,29 @@ extern "C" int infllmv2_varlen_fwd_stage1(void* stream, const void* q, const voi
                                           const int64_t* q_strides, const int64_t* k_strides,
                                           const int64_t* v_strides, int64_t score_head_stride,
                                           int64_t score_row_stride, float softmax_scale, int is_causal) {
-    IV2_CHECK(head_dim == kHeadDim, "varlen_fwd_stage1: this build only supports head_dim 128 (got %d)", head_dim);
-    IV2_CHECK(num_heads_k > 0 && num_heads == num_heads_k * kGroup,
-              "varlen_fwd_stage1: requires num_heads == 16 * num_heads_k (got %d and %d)", num_heads, num_heads_k);
-    IV2_CHECK(batch > 0 && total_q >= 0 && max_seqlen_q >= 0 && max_seqlen_k >= 0, "varlen_fwd_stage1: bad sizes");
-    IV2_CHECK(q && k && v && score && cu_seqlens_q && cu_seqlens_k && cu_seqlens_v, "varlen_fwd_stage1: null pointer");
-    IV2_CHECK(num_heads_k <= 65535 && batch <= 65535, "varlen_fwd_stage1: batch and num_heads_k must not exceed 65535");
-    IV2_CHECK(reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(k) % 16 == 0 &&
-              reinterpret_cast<uintptr_t>(v) % 16 == 0, "varlen_fwd_stage1: q, k, v must be 16-byte aligned");
-    for (int s = 0; s < 3; ++s) IV2_CHECK(q_strides[s] % 8 == 0, "varlen_fwd_stage1: q strides must be multiples of 8 elements");
-    IV2_CHECK(k_strides[0] % 8 == 0 && k_strides[1] % 8 == 0 && v_strides[0] % 8 == 0 && v_strides[1] % 8 == 0,
-              "varlen_fwd_stage1: k/v strides must be multiples of 8 elements");
     IV2_CHECK(score_row_stride >= max_seqlen_k, "varlen_fwd_stage1: score row stride shorter than max_seqlen_k");
-    if (total_q == 0 || max_seqlen_q == 0) return 0;
-    Stage1Params p{};
-    p.q = static_cast<const bf16_bits*>(q);
-    p.k = static_cast<const bf16_bits*>(k);
-    p.c = static_cast<const bf16_bits*>(v);
-    p.score = static_cast<bf16_bits*>(score);
-    p.cu_seqlens_q = cu_seqlens_q; p.cu_seqlens_k = cu_seqlens_k; p.cu_seqlens_c = cu_seqlens_v;
-    p.q_tok_stride = q_strides[0]; p.q_grp_stride = q_strides[1]; p.q_kvh_stride = q_strides[2];
-    p.k_row_stride = k_strides[0]; p.k_head_stride = k_strides[1];
-    p.c_row_stride = v_strides[0]; p.c_head_stride = v_strides[1];
-    p.score_head_stride = score_head_stride; p.score_row_stride = score_row_stride;
-    p.score_cols = max_seqlen_k;
-    p.scale_log2 = softmax_scale * 1.44269504088896340736f;
-    p.causal = is_causal;
-    const dim3 grid((max_seqlen_q + kTokPerBlock - 1) / kTokPerBlock, batch, num_heads_k);
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    if (is_causal) hipLaunchKernelGGL(stage1_kernel<true>, grid, dim3(256), 0, st, p);
-    else hipLaunchKernelGGL(stage1_kernel<false>, grid, dim3(256), 0, st, p);
-    IV2_LAUNCH_CHECK();
-    return 0;
+    return launch_stage1("varlen_fwd_stage1", stream, q, k, v, score, cu_seqlens_q, cu_seqlens_k, cu_seqlens_v, batch,
+                         total_q, num_heads, num_heads_k, head_dim, max_seqlen_q, max_seqlen_k, q_strides, k_strides,
+                         v_strides, score_head_stride, score_row_stride, softmax_scale, is_causal, nullptr);
+}
+
+extern "C" int infllmv2_varlen_fwd_stage1_pooled(void* stream, const void* q, const void* k, const void* v,
+                                                 void* pooled, const int32_t* cu_seqlens_q,
+                                                 const int32_t* cu_seqlens_k, const int32_t* cu_seqlens_v,
+                                                 const int32_t* cache_lens, int cache_len, int batch,
+                                                 int64_t total_q, int num_heads, int num_heads_k, int head_dim,
+                                                 int max_seqlen_q, int max_seqlen_k, const int64_t* q_strides,
+                                                 const int64_t* k_strides, const int64_t* v_strides, int out_len,
+                                                 float softmax_scale, int is_causal, int kernel_size, int stride,
+                                                 int padding, int block_size, int local_blocks, int init_blocks) {
+    IV2_CHECK(kernel_size == 5 && stride == 4 && padding == 1 && block_size == kBlockN,
+              "varlen_fwd_stage1_pooled: only the 5/4/1 window on 64-token blocks is fused (got %d/%d/%d on %d); "
+              "use varlen_fwd_stage1 and max_pooling_1d", kernel_size, stride, padding, block_size);
+    IV2_CHECK(out_len >= 0 && cache_len >= 0, "varlen_fwd_stage1_pooled: negative out_len or cache_len");
+    if (out_len == 0) return 0;
+    const Stage1Pool pool{cache_lens, cache_len, out_len, local_blocks, init_blocks};
+    return launch_stage1("varlen_fwd_stage1_pooled", stream, q, k, v, pooled, cu_seqlens_q, cu_seqlens_k, cu_seqlens_v,
+                         batch, total_q, num_heads, num_heads_k, head_dim, max_seqlen_q, max_seqlen_k, q_strides,
+                         k_strides, v_strides, total_q * static_cast<int64_t>(out_len), out_len, softmax_scale,
+                         is_causal, &pool);
 }

@@ -39,3 +39,33 @@ def stage1_scores(q, k, v, cu_seqlens_q, cu_seqlens_k, cu_seqlens_v, max_seqlen_
                   _lib.i64_array([k.stride(0), k.stride(1)]), _lib.i64_array([v.stride(0), v.stride(1)]),
                   buf.stride(0), buf.stride(1), float(softmax_scale), int(bool(causal)))
     return buf if row == max_seqlen_k else buf[:, :, :max_seqlen_k]
+
+
+def stage1_pooled(q, k, v, cu_seqlens_q, cu_seqlens_k, cu_seqlens_v, max_seqlen_q, max_seqlen_k, softmax_scale,
+                  causal, out_len, cache_lens, cache_len, local_blocks, init_blocks, block_size, stride):
+    """Stage-1 scores pooled onto key blocks in the same launch: bf16 ``(nheads_k, total_q, out_len)``."""
+    for t in (cu_seqlens_q, cu_seqlens_k, cu_seqlens_v):
+        if not t.is_contiguous():
+            raise RuntimeError("cu_seqlens must be contiguous")
+    batch = cu_seqlens_q.numel() - 1
+    if cu_seqlens_v.numel() != batch + 1:
+        raise RuntimeError("cu_seqlens_v must have shape (batch_size + 1)")
+    if cache_lens is not None and (cache_lens.dtype != torch.int32 or cache_lens.numel() != batch
+                                   or not cache_lens.is_contiguous()):
+        raise RuntimeError("cache_lens must be a contiguous int32 tensor of shape (batch_size)")
+    total_q, Hq, d = q.shape
+    Hk = k.shape[1]
+    if v.shape[1] != Hk or v.shape[2] != d:
+        raise RuntimeError("v must have shape (total_v, num_heads_k, head_size)")
+    per_block = block_size // stride
+    out = torch.empty((Hk, total_q, out_len), dtype=torch.bfloat16, device=q.device)
+    with torch.cuda.device(q.device):
+        _lib.call("infllmv2_varlen_fwd_stage1_pooled", stream_ptr(q.device), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                  out.data_ptr(), cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), cu_seqlens_v.data_ptr(),
+                  cache_lens.data_ptr() if cache_lens is not None else None, int(cache_len), batch, total_q, Hq, Hk, d,
+                  max_seqlen_q, max_seqlen_k,
+                  _lib.i64_array([q.stride(0), q.stride(1), GROUP * q.stride(1)]),
+                  _lib.i64_array([k.stride(0), k.stride(1)]), _lib.i64_array([v.stride(0), v.stride(1)]),
+                  out_len, float(softmax_scale), int(bool(causal)), per_block + 1, per_block, 1, block_size,
+                  local_blocks, init_blocks)
+    return out
