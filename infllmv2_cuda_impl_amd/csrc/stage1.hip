@@ -16,8 +16,8 @@
 // pass 1 stay lane-local until one 16-lane butterfly at the end, and the sum over the 16 heads
 // in pass 2 is an in-lane add of four values plus two cross-lane adds.  A workgroup is 4
 // wavefronts x 4 consecutive tokens; each 64-key tile of compressed keys is staged once in LDS
-// in MFMA-operand order (conflict-free ds_read_b128) and reused by all 16 tokens, and inside a
-// wavefront one operand read feeds four MFMAs.
+// (LDS-DMA, straight into MFMA-operand order, read back with conflict-free ds_read_b128) and reused
+// by all 16 tokens, and inside a wavefront one operand read feeds four MFMAs.
 #include "common.h"
 #include "block_walker.h"
 #include "../../include/infllmv2_hip.h"
@@ -61,26 +61,28 @@ __device__ __forceinline__ int stage1_visible(int i, int s, int L, int Sq, bool 
     return v < L ? v : L;
 }
 
-// global (64 keys x 128 d) tile -> registers; thread t of 256 owns 16-byte units t, t+256, ...
-__device__ __forceinline__ void load_tile_regs(uint4 (&r)[4], const bf16_bits* base, int64_t row_stride,
-                                               int key0, int L, int tid) {
-#pragma unroll
-    for (int it = 0; it < 4; ++it) {
-        const int u = tid + it * 256;
-        const int key = u >> 4, chunk = u & 15;
-        r[it] = make_uint4(0, 0, 0, 0);
-        if (key0 + key < L) r[it] = *reinterpret_cast<const uint4*>(base + (key0 + key) * row_stride + chunk * 8);
-    }
+// A (64 keys x 128 d) tile goes from global memory to LDS by LDS-DMA, in MFMA-operand order: 16-byte unit
+// u = (kt*4 + c)*64 + 16*g + n holds K[16*kt + n][32*c + 8*g ..].  Thread tid of 256 moves units tid + 256*it, i.e.
+// wavefront w moves, for key tile kt = it, the chunk c = w of its 16 keys: lane l's unit lands at
+// lds_base + 16 l, which is exactly operand order, so the operand reads are linear and free of bank conflicts.
+// Keys beyond the last one are read from the last row (finite values that every consumer masks).
+// The compiler's wait counts do not see these loads: the code waits for them by hand before the barrier that
+// publishes the tile.
+__device__ __forceinline__ uint32_t s1_lds_addr(const void* ptr) {
+    return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const void*)ptr));
 }
-
-// registers -> LDS in operand order: unit ((kt*4 + c)*64 + 16*g + n) holds K[16*kt + n][32*c + 8*g ..]
-__device__ __forceinline__ void store_tile_lds(const uint4 (&r)[4], uint4* lds, int tid) {
+__device__ __forceinline__ void s1_dma16(const void* base, uint32_t lane_off, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
+                 : : "v"(lane_off), "s"(base), "s"(lds_base) : "memory", "m0");
+}
+__device__ __forceinline__ void issue_tile(const bf16_bits* base, int row_stride, int key0, int L, uint32_t lds_tile,
+                                           int wave, int n, int g) {
 #pragma unroll
     for (int it = 0; it < 4; ++it) {
-        const int u = tid + it * 256;
-        const int key = u >> 4, chunk = u & 15;
-        const int kt = key >> 4, n = key & 15, c = chunk >> 2, g = chunk & 3;
-        lds[(kt * 4 + c) * 64 + 16 * g + n] = r[it];
+        int row = key0 + 16 * it + n;
+        row = row < L ? row : L - 1;
+        const uint32_t off = static_cast<uint32_t>(row * row_stride + 32 * wave + 8 * g) * 2u;
+        s1_dma16(base, off, lds_tile + (it * 4 + wave) * 1024);
     }
 }
 
@@ -164,15 +166,20 @@ void stage1_kernel(const Stage1Params p) {
 
     const bf16_bits* cbase = p.c + static_cast<int64_t>(c0) * p.c_row_stride + h * p.c_head_stride;
     const bf16_bits* kbase = p.k + static_cast<int64_t>(k0) * p.k_row_stride + h * p.k_head_stride;
-    uint4 stage[4];
-    if (tiles_c > 0) {
-        load_tile_regs(stage, cbase, p.c_row_stride, 0, Lc, tid);
-        store_tile_lds(stage, tile[0], tid);
-    }
+    const uint32_t lds_tiles = __builtin_amdgcn_readfirstlane(s1_lds_addr(tile));
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const int c_stride = static_cast<int>(p.c_row_stride), k_stride = static_cast<int>(p.k_row_stride);
+    // every ordinary load so far (q) lands before the first LDS-DMA goes out
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int t = 0; t < kTokPerWave; ++t)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) asm volatile("" : "+v"(qf[t][c]));
+    if (tiles_c > 0) issue_tile(cbase, c_stride, 0, Lc, lds_tiles, wave_u, n, g);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     for (int ti = 0; ti < tiles_c; ++ti) {
-        const bool more = ti + 1 < tiles_c;
-        if (more) load_tile_regs(stage, cbase, p.c_row_stride, (ti + 1) * 64, Lc, tid);
+        if (ti + 1 < tiles_c) issue_tile(cbase, c_stride, (ti + 1) * 64, Lc, lds_tiles + ((ti + 1) & 1) * 16384, wave_u, n, g);
         const uint4* cur = tile[ti & 1];
         floatx4 s[kTokPerWave][4];
 #pragma unroll
@@ -212,7 +219,7 @@ void stage1_kernel(const Stage1Params p) {
                 m[t][e] = m_new;
             }
         }
-        if (more) store_tile_lds(stage, tile[(ti + 1) & 1], tid);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");         // this wavefront's share of the next tile has landed
         __syncthreads();
     }
     // merge the 16 key-column lanes of each head: lse2 = m + log2(l) in log2 units
@@ -235,10 +242,8 @@ void stage1_kernel(const Stage1Params p) {
         }
 
     // ---------------- pass 2: scores over the fine keys ----------------
-    if (tiles_f > 0) {
-        load_tile_regs(stage, kbase, p.k_row_stride, 0, Lk, tid);
-        store_tile_lds(stage, tile[0], tid);
-    }
+    if (tiles_f > 0) issue_tile(kbase, k_stride, 0, Lk, lds_tiles, wave_u, n, g);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     bf16_bits* out_rows[kTokPerWave];
     int bq[kTokPerWave];                                       // pooled output: the key block the token itself sits in
@@ -263,8 +268,7 @@ void stage1_kernel(const Stage1Params p) {
     };
 
     for (int ti = 0; ti < tiles_f; ++ti) {
-        const bool more = ti + 1 < tiles_f;
-        if (more) load_tile_regs(stage, kbase, p.k_row_stride, (ti + 1) * 64, Lk, tid);
+        if (ti + 1 < tiles_f) issue_tile(kbase, k_stride, (ti + 1) * 64, Lk, lds_tiles + ((ti + 1) & 1) * 16384, wave_u, n, g);
         const uint4* cur = tile[ti & 1];
         float part[kTokPerWave][4];                            // [t][kt]: this lane's four heads summed, key 16 kt + n
 #pragma unroll
@@ -310,7 +314,7 @@ void stage1_kernel(const Stage1Params p) {
                 if (live[t] && (lane & 3) == 0 && kb < p.pool_len) out_rows[t][kb] = pool_rest(kb, bq[t], best);
             }
         }
-        if (more) store_tile_lds(stage, tile[(ti + 1) & 1], tid);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
     }
     // columns no tile covered
@@ -355,6 +359,11 @@ int launch_stage1(const char* who, void* stream, const void* q, const void* k, c
     for (int s = 0; s < 3; ++s) IV2_CHECK(q_strides[s] % 8 == 0, "%s: q strides must be multiples of 8 elements", who);
     IV2_CHECK(k_strides[0] % 8 == 0 && k_strides[1] % 8 == 0 && v_strides[0] % 8 == 0 && v_strides[1] % 8 == 0,
               "%s: k/v strides must be multiples of 8 elements", who);
+    // a lane's byte offset from its sequence's first compressed key is a 32-bit LDS-DMA operand
+    IV2_CHECK(k_strides[0] > 0 && v_strides[0] > 0 &&
+              (static_cast<int64_t>(max_seqlen_k) + 64) * k_strides[0] < (1ll << 30) &&
+              (static_cast<int64_t>(max_seqlen_k) + 64) * v_strides[0] < (1ll << 30),
+              "%s: compressed-key rows too far apart (row stride x max_seqlen_k must stay below 2^30 elements)", who);
     if (total_q == 0 || max_seqlen_q == 0) return 0;
     Stage1Params p{};
     p.q = static_cast<const bf16_bits*>(q);
