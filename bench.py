@@ -4,7 +4,8 @@
 A step is one end-to-end prefill forward of BASELINE config 2: one sequence of 32768 tokens, bf16,
 GQA 32 query / 2 KV heads, d = 128, compressed keys kernel 32 / stride 16 (LSE over kernel 128 /
 stride 64), block 64, topk = 64 (1 init + 32 local blocks forced), causal:
-Stage-1 scores -> max-pool -> top-k -> mask packing -> Stage-2 block-sparse forward.
+Stage-1 scores -> max-pool (one fused launch; --unfused-front-end times the two separate calls) -> top-k ->
+mask packing -> Stage-2 block-sparse forward.
 Inputs (q, k, v and the caller-side compressed keys) are resident in HBM before the timed region.
 
 `value` = Stage-2 algorithmic sparse FLOPs (4*16*64*128 per selected causal block per token and KV head)
@@ -40,6 +41,8 @@ def parse_args():
     ap.add_argument("--seqlen", type=int, default=32768)
     ap.add_argument("--topk", type=int, default=64)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--unfused-front-end", action="store_true",
+                    help="time the reference's call sequence (Stage-1 scores, then max_pooling_1d) instead of the fused launch")
     ap.add_argument("--no-stages", action="store_true", help="skip the per-stage and kernel-only timings")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three plain 1 GiB device copies (a kernel of known traffic for scaling rocprofv3 --pmc counters)")
@@ -154,8 +157,12 @@ def main():
     Lk = kf.shape[0]
 
     def step():
-        score = ops.infllmv2_attn_stage1(q, kf, kc, cu_q, cu_f, cu_c, S, Lk, causal=True)
-        pooled = ops.max_pooling_1d(score, 0, local_blocks, init_blocks)
+        if args.unfused_front_end:      # the reference's own call sequence
+            score = ops.infllmv2_attn_stage1(q, kf, kc, cu_q, cu_f, cu_c, S, Lk, causal=True)
+            pooled = ops.max_pooling_1d(score, 0, local_blocks, init_blocks)
+        else:                           # same pooled tensor, bit for bit, in one launch
+            pooled = ops.infllmv2_attn_stage1_pooled(q, kf, kc, cu_q, cu_f, cu_c, S, Lk, local_blocks, init_blocks,
+                                                     causal=True)
         idx = ops.topk_blocks(pooled, topk)
         return ops.infllmv2_attn_varlen_func(q, k, v, cu_q, cu_q, S, S, causal=True, topk_idx=idx), idx
 
@@ -182,7 +189,9 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"BASELINE config 2: prefill forward, 1 x {S} tokens, GQA 32q/2kv, d=128, "
                                f"kernel 32/stride 16 compressed keys, block 64, topk={topk} "
-                               f"(1 init + 32 local forced), causal; Stage-1 + pool + top-k + pack + Stage-2 fwd",
+                               f"(1 init + 32 local forced), causal; "
+                               + ("Stage-1 + pool" if args.unfused_front_end else "fused Stage-1/pool")
+                               + " + top-k + pack + Stage-2 fwd",
                    "seqlen": S, "topk": topk, "selected_causal_blocks_per_token_head": nsel / (2 * S)},
         "stage2_fwd_algorithmic_flops": fwd_flops, "stage1_algorithmic_flops": s1_flops,
         "frac_bf16_mfma_peak_whole_step": fwd_flops / ms_per_step / 1e9 / PEAK_BF16_TFLOPS,
@@ -195,6 +204,8 @@ def main():
         stages = {
             "stage1": event_ms(torch, lambda: ops.infllmv2_attn_stage1(q, kf, kc, cu_q, cu_f, cu_c, S, Lk, causal=True), 10),
             "pool": event_ms(torch, lambda: ops.max_pooling_1d(score, 0, local_blocks, init_blocks), 10),
+            "stage1_pooled_fused": event_ms(torch, lambda: ops.infllmv2_attn_stage1_pooled(
+                q, kf, kc, cu_q, cu_f, cu_c, S, Lk, local_blocks, init_blocks, causal=True), 10),
             "topk": event_ms(torch, lambda: ops.topk_blocks(pooled, topk), 10),
             "pack_mask": event_ms(torch, lambda: ops.topk_to_uint64(idx, S, 64), 10),
             "stage2_fwd_op": event_ms(torch, lambda: ops.infllmv2_attn_varlen_func(q, k, v, cu_q, cu_q, S, S, causal=True, topk_idx=idx), 10),
@@ -212,6 +223,8 @@ def main():
         result["stage1_tflops"] = s1_flops / stages["stage1"] / 1e9
         sel_ms = stages["stage1"] + stages["pool"] + stages["topk"]
         result["stage1_pool_topk_share_of_fwd"] = sel_ms / (sel_ms + stages["pack_mask"] + stages["stage2_fwd_op"])
+        sel_ms = stages["stage1_pooled_fused"] + stages["topk"]
+        result["fused_front_end_share_of_fwd"] = sel_ms / (sel_ms + stages["pack_mask"] + stages["stage2_fwd_op"])
 
         # the dominant kernel alone: K/V images prepacked, mask packed, HIP events on the launch stream
         out_k = torch.empty_like(q)
