@@ -107,6 +107,19 @@ int infllmv2_topk(void* stream, int num_tokens, int dim, int top, int dtype, con
 int infllmv2_topk_blocks(void* stream, const void* pooled, int64_t row_stride, int32_t* topk_idx,
                          int64_t rows, int n, int k);
 
+/* ---- Compressed keys (caller-side in the reference) ----------------------------------------- */
+
+/* The Stage-1 inputs are means of K over sliding windows; the reference leaves their construction to its callers,
+ * and its tests build them with compress_tensor / calc_chunks_with_stride
+ * (tests/test_stage1_compressed_lse.py:16-99): row j of a sequence = mean of K rows [stride*j, stride*j+kernel_size),
+ * full windows only.  k (total_k, Hk, d) bf16 with strides {row, head}; out (sum_b L_b, Hk, d) bf16, dense, where
+ * L_b = (len_b - kernel_size) / stride + 1 (0 if len_b < kernel_size); cu_seqlens_out (batch + 1) is written by
+ * the call.  Rows j < first_row of every sequence are left untouched (first_row > 0 appends to compressed keys
+ * built earlier, as a decode loop does every `stride` tokens).  fp32 sum in window order, one rounding. */
+int infllmv2_compress_keys(void* stream, const void* k, void* out, const int32_t* cu_seqlens_k,
+                           int32_t* cu_seqlens_out, int batch, int max_seqlen_k, int num_heads_k, int head_dim,
+                           int64_t k_row_stride, int64_t k_head_stride, int kernel_size, int stride, int first_row);
+
 /* ---- Stage 1: scoring over compressed keys --------------------------------------------------- */
 
 /* csrc/entry.cu:15,211 `varlen_fwd_stage1` = mha_varlen_fwd_stage1

@@ -28,6 +28,7 @@ SIGNATURES = {
     "infllmv2_max_pooling_1d_varlen_strided": [_p, _p, _p, _p, _p, _p] + [_i] * 6 + [_i64, _i64] + [_i] * 7,
     "infllmv2_topk": [_p, _i, _i, _i, _i, _p, _p, _p],
     "infllmv2_topk_blocks": [_p, _p, _i64, _p, _i64, _i, _i],
+    "infllmv2_compress_keys": [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i64, _i64, _i, _i, _i],
     "infllmv2_varlen_fwd_stage1": [_p, _p, _p, _p, _p, _p, _p, _p, _i, _i64, _i, _i, _i, _i, _i, _p, _p, _p, _i64, _i64, _f, _i],
     "infllmv2_varlen_fwd_stage1_pooled": [_p] * 9 + [_i, _i, _i64, _i, _i, _i, _i, _i, _p, _p, _p, _i, _f] + [_i] * 7,
     "infllmv2_varlen_fwd": [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _sz, _i, _i, _i64, _i64, _i, _i, _i, _i, _i,

@@ -60,7 +60,7 @@ def _check_qkv(q, k, v, cu_seqlens_q, cu_seqlens_k, same_kv_len=True):
     for name, t in (("q", q), ("k", k), ("v", v), ("cu_seqlens_q", cu_seqlens_q), ("cu_seqlens_k", cu_seqlens_k)):
         require_gpu(t, name)
     for t in (q, k, v):
-        if t.stride(-1) != 1:
+        if t.numel() > 0 and t.stride(-1) != 1:
             raise RuntimeError("Input tensor must have contiguous last dimension")
     if not cu_seqlens_q.is_contiguous():
         raise RuntimeError("cu_seqlens_q must be contiguous")

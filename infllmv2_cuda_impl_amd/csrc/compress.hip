@@ -1,0 +1,111 @@
+// Compressed keys for Stage 1 (gfx950): row j of a sequence is the mean of its K rows
+// [stride*j, stride*j + kernel_size), full windows only.
+//
+// The reference leaves this step to its callers; the rule is the one its tests use to build the
+// Stage-1 inputs (compress_tensor / calc_chunks_with_stride, tests/test_stage1_compressed_lse.py:16-99:
+// windows that fit entirely inside a sequence, mean over the window, result in the input dtype).
+// The mean is an fp32 sum taken in window order divided by kernel_size, rounded once to bf16.
+//
+// HBM-bound and small: K is read once from memory (the overlapping windows hit in cache) and
+// the output is 1/stride of its size.  A thread owns 8 contiguous d values (16 bytes) of one output row.
+#include "common.h"
+#include "../../include/infllmv2_hip.h"
+
+namespace infllmv2 {
+
+__device__ __forceinline__ int compressed_rows(int len, int kernel_size, int stride) {
+    return len >= kernel_size ? (len - kernel_size) / stride + 1 : 0;
+}
+
+// cu_out[b] = rows of the sequences before b; one thread (batch is small)
+__global__ void compressed_cu_seqlens_kernel(const int* __restrict__ cu_k, int* __restrict__ cu_out, int batch,
+                                             int kernel_size, int stride) {
+    if (blockIdx.x != 0 || threadIdx.x != 0) return;
+    int acc = 0;
+    cu_out[0] = 0;
+    for (int b = 0; b < batch; ++b) {
+        acc += compressed_rows(cu_k[b + 1] - cu_k[b], kernel_size, stride);
+        cu_out[b + 1] = acc;
+    }
+}
+
+struct CompressParams {
+    const bf16_bits* k;
+    bf16_bits* out;
+    const int* cu_k;
+    const int* cu_out;
+    int64_t k_row_stride, k_head_stride;
+    int units_per_row;               // num_heads * head_dim / 8
+    int units_per_head;              // head_dim / 8
+    int kernel_size, stride;
+    int first_row;                   // rows before this one are left alone (appending to a cache of compressed keys)
+};
+
+__global__ __launch_bounds__(256)
+void compress_keys_kernel(const CompressParams p) {
+    const int b = blockIdx.y;
+    const int k0 = p.cu_k[b];
+    const int rows = compressed_rows(p.cu_k[b + 1] - k0, p.kernel_size, p.stride);
+    const int rows_per_wg = 256 / p.units_per_row;             // units_per_row divides 256 (checked by the launcher)
+    const int j = p.first_row + blockIdx.x * rows_per_wg + threadIdx.x / p.units_per_row;
+    if (j >= rows) return;
+    const int u = threadIdx.x % p.units_per_row;
+    const int head = u / p.units_per_head, piece = u % p.units_per_head;
+    const bf16_bits* src = p.k + (static_cast<int64_t>(k0) + static_cast<int64_t>(j) * p.stride) * p.k_row_stride +
+                           head * p.k_head_stride + piece * 8;
+    float acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+    for (int i = 0; i < p.kernel_size; ++i) {
+        const uint4 raw = *reinterpret_cast<const uint4*>(src + i * p.k_row_stride);
+        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            acc[2 * e] += __uint_as_float(w[e] << 16);
+            acc[2 * e + 1] += __uint_as_float(w[e] & 0xffff0000u);
+        }
+    }
+    const float n = static_cast<float>(p.kernel_size);
+    uint4 o;
+    o.x = pack_bf16x2(acc[0] / n, acc[1] / n);
+    o.y = pack_bf16x2(acc[2] / n, acc[3] / n);
+    o.z = pack_bf16x2(acc[4] / n, acc[5] / n);
+    o.w = pack_bf16x2(acc[6] / n, acc[7] / n);
+    *reinterpret_cast<uint4*>(p.out + (static_cast<int64_t>(p.cu_out[b]) + j) * p.units_per_row * 8 + u * 8) = o;
+}
+
+}  // namespace infllmv2
+
+using namespace infllmv2;
+
+extern "C" int infllmv2_compress_keys(void* stream, const void* k, void* out, const int32_t* cu_seqlens_k,
+                                      int32_t* cu_seqlens_out, int batch, int max_seqlen_k, int num_heads_k,
+                                      int head_dim, int64_t k_row_stride, int64_t k_head_stride, int kernel_size,
+                                      int stride, int first_row) {
+    IV2_CHECK(batch > 0 && batch <= 65535 && max_seqlen_k >= 0, "compress_keys: bad batch or max_seqlen_k");
+    IV2_CHECK(kernel_size > 0 && stride > 0 && first_row >= 0, "compress_keys: kernel_size and stride must be positive");
+    IV2_CHECK(k && out && cu_seqlens_k && cu_seqlens_out, "compress_keys: null pointer");
+    IV2_CHECK(head_dim > 0 && head_dim % 8 == 0 && num_heads_k > 0, "compress_keys: head_dim must be a multiple of 8");
+    const int units = num_heads_k * head_dim / 8;
+    IV2_CHECK(units <= 256 && 256 % units == 0, "compress_keys: num_heads_k * head_dim / 8 = %d must divide 256", units);
+    IV2_CHECK(reinterpret_cast<uintptr_t>(k) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 &&
+              k_row_stride % 8 == 0 && k_head_stride % 8 == 0, "compress_keys: k and out must be 16-byte aligned, strides multiples of 8");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    hipLaunchKernelGGL(compressed_cu_seqlens_kernel, dim3(1), dim3(64), 0, st, cu_seqlens_k, cu_seqlens_out, batch,
+                       kernel_size, stride);
+    IV2_LAUNCH_CHECK();
+    const int max_rows = max_seqlen_k >= kernel_size ? (max_seqlen_k - kernel_size) / stride + 1 : 0;
+    if (max_rows <= first_row) return 0;
+    CompressParams p{};
+    p.k = static_cast<const bf16_bits*>(k);
+    p.out = static_cast<bf16_bits*>(out);
+    p.cu_k = cu_seqlens_k; p.cu_out = cu_seqlens_out;
+    p.k_row_stride = k_row_stride; p.k_head_stride = k_head_stride;
+    p.units_per_row = units; p.units_per_head = head_dim / 8;
+    p.kernel_size = kernel_size; p.stride = stride; p.first_row = first_row;
+    const int rows_per_wg = 256 / units;
+    const dim3 grid((max_rows - first_row + rows_per_wg - 1) / rows_per_wg, batch);
+    hipLaunchKernelGGL(compress_keys_kernel, grid, dim3(256), 0, st, p);
+    IV2_LAUNCH_CHECK();
+    return 0;
+}

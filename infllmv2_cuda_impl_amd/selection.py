@@ -1,4 +1,4 @@
-"""Block selection (top-k over pooled block scores).
+"""Block selection: compressed keys, top-k over pooled block scores, and the whole front end in one call.
 
 The reference leaves this step to its callers (README.md:42,125-126 use ``torch.topk``); the only
 order it states is the comparator of csrc/topk.cuh:17,26,37, which this operator implements:
@@ -24,3 +24,67 @@ def topk_blocks(pooled: torch.Tensor, k: int) -> torch.Tensor:
         _lib.call("infllmv2_topk_blocks", stream_ptr(x.device), x.data_ptr(), n, out.data_ptr(),
                   flat_rows(x.shape[:-1]), n, k)
     return out
+
+
+def compress_keys(k: torch.Tensor, cu_seqlens_k: torch.Tensor, max_seqlen_k: int, kernel_size: int, stride: int,
+                  out: torch.Tensor | None = None, first_row: int = 0):
+    """Mean of ``k`` ``(total_k, nheads_k, d)`` bf16 over the full windows ``[stride*j, stride*j + kernel_size)`` of
+    every packed sequence: the compressed keys of Stage 1, which the reference's callers build themselves
+    (compress_tensor, tests/test_stage1_compressed_lse.py:56-99).
+
+    Returns ``(k_cmp, cu_seqlens_cmp)``: ``k_cmp`` ``(rows, nheads_k, d)`` bf16 whose first ``cu_seqlens_cmp[-1]``
+    rows are defined (``rows`` is that count for one sequence and an upper bound, ``total_k // stride + 1``, for a
+    packed batch, so that no host read is needed) and ``cu_seqlens_cmp`` int32 ``(batch + 1)``.  With ``out`` (a
+    buffer returned by an earlier call) and ``first_row`` only rows ``>= first_row`` of each sequence are written.
+    """
+    require_gpu(k, "k")
+    if k.dtype != torch.bfloat16:
+        raise RuntimeError("this build only has bf16 kernels")
+    if k.dim() != 3 or k.stride(-1) != 1:
+        raise RuntimeError("k must have shape (total_k, num_heads_k, head_size) with a contiguous last dimension")
+    if cu_seqlens_k.dtype != torch.int32 or not cu_seqlens_k.is_contiguous():
+        raise RuntimeError("cu_seqlens_k must be a contiguous int32 tensor")
+    batch = cu_seqlens_k.numel() - 1
+    total_k, Hk, d = k.shape
+    if batch == 1:
+        rows = (max_seqlen_k - kernel_size) // stride + 1 if max_seqlen_k >= kernel_size else 0
+    else:
+        rows = total_k // stride + 1
+    if out is None:
+        backing = torch.empty((max(rows, 1), Hk, d), dtype=k.dtype, device=k.device)      # never a null pointer
+        out = backing[:rows]
+    elif out.shape[0] < rows or tuple(out.shape[1:]) != (Hk, d) or not out.is_contiguous() or out.dtype != k.dtype:
+        raise RuntimeError("out must be a contiguous (rows, num_heads_k, head_size) buffer of k's dtype")
+    else:
+        backing = out
+    cu_out = torch.empty(batch + 1, dtype=torch.int32, device=k.device)
+    with torch.cuda.device(k.device):
+        _lib.call("infllmv2_compress_keys", stream_ptr(k.device), k.data_ptr(), backing.data_ptr(), cu_seqlens_k.data_ptr(),
+                  cu_out.data_ptr(), batch, max_seqlen_k, Hk, d, k.stride(0), k.stride(1), kernel_size, stride, first_row)
+    return out, cu_out
+
+
+def select_blocks(q: torch.Tensor, k: torch.Tensor, cu_seqlens_q: torch.Tensor, cu_seqlens_k: torch.Tensor,
+                  max_seqlen_q: int, max_seqlen_k: int, topk: int, local_blocks: int, init_blocks: int,
+                  cache_lens: torch.Tensor | None = None, max_cache_len: int | None = None, softmax_scale=None,
+                  causal: bool = True, kernel_size: int = 32, stride: int = 16, block_size: int = 64,
+                  exact_lse: bool = False) -> torch.Tensor:
+    """The selection front end in one call: compressed keys (kernel ``kernel_size`` / stride ``stride``; the
+    log-sum-exp over the 4x coarser set, or over the same set with ``exact_lse``), Stage-1 scores pooled onto
+    ``block_size``-token key blocks in one launch, top-k.  Returns ``topk_idx`` int32 ``(nheads_k, total_q, topk)``
+    for :func:`infllmv2_attn_varlen_func`, equal to what the reference's sequence of calls
+    (compress, ``infllmv2_attn_stage1``, ``max_pooling_1d(_varlen)``, top-k) selects; the score tensor is never
+    materialised.  Packed batches need ``cache_lens`` (zeros for plain prefill), as ``max_pooling_1d_varlen`` does.
+    """
+    from .attention import infllmv2_attn_stage1_pooled
+    kf, cu_f = compress_keys(k, cu_seqlens_k, max_seqlen_k, kernel_size, stride)
+    if exact_lse:
+        kc, cu_c = kf, cu_f
+    else:
+        kc, cu_c = compress_keys(k, cu_seqlens_k, max_seqlen_k, 4 * kernel_size, 4 * stride)
+    max_lk = (max_seqlen_k - kernel_size) // stride + 1 if max_seqlen_k >= kernel_size else 0
+    pooled = infllmv2_attn_stage1_pooled(q, kf, kc, cu_seqlens_q, cu_f, cu_c, max_seqlen_q, max_lk, local_blocks,
+                                         init_blocks, cache_lens=cache_lens, max_cache_len=max_cache_len,
+                                         block_size=block_size, stride=stride, softmax_scale=softmax_scale,
+                                         causal=causal)
+    return topk_blocks(pooled, topk)

@@ -9,6 +9,11 @@ from ._util import stream_ptr
 GROUP = 16
 
 
+def _readable(t: torch.Tensor) -> torch.Tensor:
+    """A key set with no rows (sequences shorter than one window) still needs a valid pointer; no row of it is read."""
+    return t if t.shape[0] > 0 else t.new_zeros((1,) + tuple(t.shape[1:]))
+
+
 def stage1_scores(q, k, v, cu_seqlens_q, cu_seqlens_k, cu_seqlens_v, max_seqlen_q, max_seqlen_k, softmax_scale,
                   causal, row_pad_to: int = 1):
     """Returns bf16 ``(nheads_k, total_q, max_seqlen_k)``.
@@ -29,6 +34,7 @@ def stage1_scores(q, k, v, cu_seqlens_q, cu_seqlens_k, cu_seqlens_v, max_seqlen_
     Hk = k.shape[1]
     if v.shape[1] != Hk or v.shape[2] != d:
         raise RuntimeError("v must have shape (total_v, num_heads_k, head_size)")
+    k, v = _readable(k), _readable(v)
     row = (max_seqlen_k + row_pad_to - 1) // row_pad_to * row_pad_to
     buf = torch.empty((Hk, total_q, row), dtype=torch.bfloat16, device=q.device)
     with torch.cuda.device(q.device):
@@ -57,6 +63,7 @@ def stage1_pooled(q, k, v, cu_seqlens_q, cu_seqlens_k, cu_seqlens_v, max_seqlen_
     Hk = k.shape[1]
     if v.shape[1] != Hk or v.shape[2] != d:
         raise RuntimeError("v must have shape (total_v, num_heads_k, head_size)")
+    k, v = _readable(k), _readable(v)
     per_block = block_size // stride
     out = torch.empty((Hk, total_q, out_len), dtype=torch.bfloat16, device=q.device)
     with torch.cuda.device(q.device):
