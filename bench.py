@@ -245,6 +245,16 @@ def main():
         result["roofline"] = {"bound": "mfma", "kernel": "stage2_fwd_hybrid_kernel<causal>", "achieved": achieved,
                               "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS,
                               "traffic": MEASURED_FWD_TRAFFIC_BYTES if (S, topk) == (32768, 64) else None, "kernel_ms": k_ms}
+        if S % 8 == 0:
+            # the K/V gather bound reported beside the MFMA one: a block common to the 8 tokens of a workgroup is
+            # fetched once per workgroup, every other selected block once per token, 32 KiB each, and a CU's
+            # vector-memory return path moves 64 B/clk (256 CUs, 2.4 GHz peak clock)
+            sel = (bits & causal_blk[None]).view(2, S // 8, 8, nblk)
+            n_common = int(sel.all(dim=2).sum())
+            gather_bytes = 32768 * (n_common + int(sel.sum()) - 8 * n_common)
+            peak_l1 = 256 * 64 * 2.4e9 / 1e12
+            result["roofline"]["gather"] = {"bound": "l1", "bytes": gather_bytes, "achieved": gather_bytes / k_ms / 1e9,
+                                            "peak": peak_l1, "unit": "TB/s", "frac": gather_bytes / k_ms / 1e9 / peak_l1}
         try:
             from infllmv2_cuda_impl_amd.backward import HAVE_BACKWARD  # noqa: F401
             qg, kg, vg = [t.clone().requires_grad_(True) for t in (q, k, v)]

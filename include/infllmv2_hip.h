@@ -23,7 +23,7 @@
 extern "C" {
 #endif
 
-#define INFLLMV2_ABI_VERSION 1
+#define INFLLMV2_ABI_VERSION 2
 
 /* ---- library ------------------------------------------------------------------------------ */
 
@@ -216,17 +216,28 @@ int infllmv2_varlen_bwd(void* stream, const void* dout, const void* q, const voi
 /* The split count infllmv2_fwd_kvcache will use: `requested` if > 0 (capped at 64), else a heuristic
  * (replaces num_splits_heuristic, csrc/flash_attn/flash_api.cpp:261-295). */
 int infllmv2_fwd_kvcache_num_splits(int batch, int num_heads_k, int requested);
-/* fp32 partial outputs and LSEs of the splits (0 bytes for one split). */
+/* fp32 partial outputs and LSEs of the splits, plus room for the query turned by the rotary embedding. */
 size_t infllmv2_fwd_kvcache_workspace_bytes(int batch, int num_heads_k, int num_splits);
 
 /* csrc/entry.cu:18,214 `fwd_kvcache` = mha_fwd_kvcache (csrc/flash_attn/flash_api.cpp:1549-1843; kernels
- * flash_fwd_kernel.h:606-1199 and 1794-1975) for seqlen_q == 1 without rotary / paged KV / cache_batch_idx /
- * leftpad.  q, out (batch, 1, Hq, 128): strides {batch, head}.  kcache, vcache (batch, capacity, Hk, 128),
+ * flash_fwd_kernel.h:606-1199 and 1794-1975) for seqlen_q == 1.
+ * q, out (batch, 1, Hq, 128): strides {batch, head}.  kcache, vcache (cache_batch, capacity, Hk, 128),
  * k_new, v_new (batch, seqlen_new, Hk, 128) or null: strides {batch, row, head}.  cache_seqlens (batch) int32
- * or null (= capacity).  New rows are written at cache_seqlens[b] + t first, then attention runs over
- * [0, cache_seqlens[b] + seqlen_new) restricted to the blocks set in blockmask (batch, Hk, n_uint64_per_row),
- * or all blocks when it is null.  softmax_lse (batch, Hq) fp32.  num_splits >= 1 as returned by
- * infllmv2_fwd_kvcache_num_splits. */
+ * or null (= capacity).  New rows are written at cache rows cache_seqlens[b] + t first, then attention runs
+ * over the sequence's keys restricted to the blocks set in blockmask (batch, Hk, n_uint64_per_row), or all
+ * blocks when it is null.  softmax_lse (batch, Hq) fp32.  num_splits >= 1 as returned by
+ * infllmv2_fwd_kvcache_num_splits.  Options, each null / 0 when unused:
+ *  - cache_batch_idx (batch) int32: sequence b lives in cache row cache_batch_idx[b] (flash_api.cpp:1800-1808);
+ *  - cache_leftpad (batch) int32: the sequence's keys are cache rows [leftpad[b], cache_seqlens[b] + seqlen_new)
+ *    and mask block j covers the 64 keys from row leftpad[b] + 64 j (flash_api.cpp:1762-1771, block_info.h:23-43);
+ *  - block_table (batch, pages per sequence) int32 with its batch stride, page_block_size: kcache/vcache are
+ *    (pages, page_block_size, Hk, 128), cache_capacity = pages per sequence x page_block_size, row r of sequence b
+ *    is row r % page_block_size of page block_table[b][r / page_block_size] (flash_api.cpp:1593-1611;
+ *    flash_fwd_kernel.h:696-712); the page size must be a multiple of 64 (the reference asks for 256); not
+ *    together with cache_batch_idx or cache_leftpad, as in the reference;
+ *  - rotary_cos, rotary_sin (seqlen_ro >= capacity, rotary_dim / 2) bf16, dense: the appended keys are turned at
+ *    their cache rows and the query at cache_seqlens[b] before use, interleaved pairs (2i, 2i+1) or contiguous
+ *    pairs (i, i + rotary_dim / 2) (flash_api.cpp:1773-1798; flash_fwd_kernel.h:787-929; rotary.h); needs k_new. */
 int infllmv2_fwd_kvcache(void* stream, const void* q, void* kcache, void* vcache, const void* k_new,
                          const void* v_new, const int32_t* cache_seqlens, void* out, float* softmax_lse,
                          const uint64_t* blockmask, void* workspace, size_t workspace_bytes, int batch,
@@ -234,7 +245,10 @@ int infllmv2_fwd_kvcache(void* stream, const void* q, void* kcache, void* vcache
                          int seqlen_new, const int64_t* q_strides, const int64_t* kcache_strides,
                          const int64_t* vcache_strides, const int64_t* knew_strides,
                          const int64_t* vnew_strides, const int64_t* o_strides, int n_uint64_per_row,
-                         int num_splits, float softmax_scale);
+                         int num_splits, float softmax_scale, const int32_t* cache_batch_idx,
+                         const int32_t* cache_leftpad, const int32_t* block_table,
+                         int64_t block_table_batch_stride, int page_block_size, const void* rotary_cos,
+                         const void* rotary_sin, int rotary_dim, int rotary_interleaved);
 
 #ifdef __cplusplus
 }

@@ -220,11 +220,9 @@ def fwd_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_,
     """mha_fwd_kvcache (flash_api.cpp:1549-1843).  Returns ``[out, softmax_lse]``."""
     from .decode import decode_with_kvcache
     _reject_unsupported(0.0, (window_size_left, window_size_right), softcap, alibi_slopes_, is_causal)
-    for name, val in (("rotary_cos", rotary_cos_), ("rotary_sin", rotary_sin_), ("cache_batch_idx", cache_batch_idx_),
-                      ("leftpad_k", leftpad_k_), ("block_table", block_table_)):
-        if val is not None:
-            raise RuntimeError(f"{name} is not supported by this build")
-    out, lse = decode_with_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, softmax_scale, is_causal, num_splits, blockmask_)
+    out, lse = decode_with_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, softmax_scale, is_causal, num_splits, blockmask_,
+                                   cache_batch_idx_, leftpad_k_, block_table_, rotary_cos_, rotary_sin_,
+                                   is_rotary_interleaved)
     if out_ is not None:
         out_.copy_(out)
         out = out_

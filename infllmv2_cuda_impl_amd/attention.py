@@ -259,7 +259,10 @@ def infllmv2_attn_with_kvcache(q, k_cache, v_cache, k=None, v=None, rotary_cos=N
     at ``cache_seqlens`` first (in place) and take part in the attention.  ``topk_idx`` int32
     ``(batch, nheads_k, 1, k)`` selects 64-key blocks of the cache (mask width from the cache capacity).
     Returns ``out (batch, 1, nheads, 128)`` or ``(out, softmax_lse (batch, nheads, 1))``.  No backward.
-    Rotary embedding, paged KV, ``cache_batch_idx`` and ``cache_leftpad`` are not supported.
+    ``rotary_cos``/``rotary_sin`` ``(seqlen_ro, rotary_dim / 2)`` turn the appended keys (at their cache rows) and
+    the query (at ``cache_seqlens``); ``cache_batch_idx`` ``(batch,)`` picks each sequence's cache row;
+    ``cache_leftpad`` ``(batch,)`` is the cache row a sequence's keys start at; ``block_table``
+    ``(batch, pages)`` makes the caches ``(num_pages, page_size, nheads_k, 128)`` (page size a multiple of 64).
     """
     from .decode import decode_with_kvcache
     assert k_cache.stride(-1) == 1, "k_cache must have contiguous last dimension"
@@ -267,16 +270,17 @@ def infllmv2_attn_with_kvcache(q, k_cache, v_cache, k=None, v=None, rotary_cos=N
     if softmax_scale is None:
         softmax_scale = q.shape[-1] ** (-0.5)
     _reject_unsupported(0.0, window_size, softcap, alibi_slopes, causal)
-    for name, val in (("rotary_cos", rotary_cos), ("rotary_sin", rotary_sin), ("cache_batch_idx", cache_batch_idx),
-                      ("cache_leftpad", cache_leftpad), ("block_table", block_table)):
-        if val is not None:
-            raise RuntimeError(f"{name} is not supported by this build")
     q, k, v = [_dense_last_dim(x) for x in (q, k, v)]
     if cache_seqlens is not None and isinstance(cache_seqlens, int):
-        cache_seqlens = torch.full((k_cache.shape[0],), cache_seqlens, dtype=torch.int32, device=k_cache.device)
+        cache_seqlens = torch.full((q.shape[0],), cache_seqlens, dtype=torch.int32, device=k_cache.device)
     mask = None
     if topk_idx is not None:
         assert topk_idx.dtype == torch.int32
-        mask, _ = topk_to_uint64(topk_idx, k_cache.shape[1], BLOCK_N)
-    out, lse = decode_with_kvcache(q, k_cache, v_cache, k, v, cache_seqlens, softmax_scale, causal, num_splits, mask)
+        # the mask spans the sequence's whole key capacity; with a paged cache that is pages x page size (the
+        # reference sizes it from k_cache.shape[1], which for a paged cache is one page)
+        capacity = k_cache.shape[1] if block_table is None else block_table.shape[1] * k_cache.shape[1]
+        mask, _ = topk_to_uint64(topk_idx, capacity, BLOCK_N)
+    out, lse = decode_with_kvcache(q, k_cache, v_cache, k, v, cache_seqlens, softmax_scale, causal, num_splits, mask,
+                                   cache_batch_idx, cache_leftpad, block_table, rotary_cos, rotary_sin,
+                                   rotary_interleaved)
     return (out, lse) if return_softmax_lse else out

@@ -40,7 +40,67 @@ struct DecodeParams {
     int64_t kn_batch, kn_row, kn_head, vn_batch, vn_row, vn_head;
     int batch, num_heads_k, capacity, seqlen_new, n64, splits;
     float scale_log2;
+    // where a sequence's rows lie (flash_api.cpp:1593-1611, 1762-1771, 1800-1808)
+    const int* cache_batch_idx;     // sequence b uses cache row cache_batch_idx[b]; null: b
+    const int* leftpad;             // the sequence's keys start at cache row leftpad[b]; null: 0
+    const int* block_table;         // (batch, pages per sequence): the caches are (pages, page_size, Hk, d)
+    int64_t bt_batch;
+    int page_size;
+    // rotary embedding of the appended keys and of the query (flash_fwd_kernel.h:787-929, rotary.h)
+    const bf16_bits* rot_cos;       // (seqlen_ro, rotary_dim / 2)
+    const bf16_bits* rot_sin;
+    int rotary_dim, rotary_interleaved;
+    bf16_bits* q_rot;               // (batch, Hq, 128): the turned query, in the workspace
 };
+
+// element offset of cache row `row` of sequence b (head 0)
+__device__ __forceinline__ int64_t cache_row_offset(const DecodeParams& p, int b, int row, int64_t batch_stride,
+                                                    int64_t row_stride) {
+    if (p.block_table) {
+        const int page = p.block_table[b * p.bt_batch + row / p.page_size];
+        return page * batch_stride + static_cast<int64_t>(row % p.page_size) * row_stride;
+    }
+    const int cb = p.cache_batch_idx ? p.cache_batch_idx[b] : b;
+    return cb * batch_stride + static_cast<int64_t>(row) * row_stride;
+}
+
+// One 16-byte chunk (8 values, d = 8 chunk ...) of a head vector turned at position pos.  Interleaved: pairs
+// (2i, 2i+1) lie inside the chunk; contiguous: the partner of d is d +- rotary_dim / 2, in another chunk of the
+// same head vector.  (a, b) -> (a cos - b sin, a sin + b cos) in fp32, one rounding (rotary.h:57-62, 131-133).
+__device__ __forceinline__ uint4 rotary_chunk(const DecodeParams& p, const bf16_bits* head_vec, int chunk, int pos) {
+    const uint4 raw = *reinterpret_cast<const uint4*>(head_vec + chunk * 8);
+    const int d0 = chunk * 8, half = p.rotary_dim >> 1;
+    if (d0 >= p.rotary_dim) return raw;
+    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+    float x[8], y[8];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        x[2 * e] = __uint_as_float(w[e] << 16);
+        x[2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
+    }
+    const bf16_bits* cs = p.rot_cos + static_cast<int64_t>(pos) * half;
+    const bf16_bits* sn = p.rot_sin + static_cast<int64_t>(pos) * half;
+    if (p.rotary_interleaved) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float c = bf16_to_f32(cs[(d0 >> 1) + i]), s = bf16_to_f32(sn[(d0 >> 1) + i]);
+            y[2 * i] = x[2 * i] * c - x[2 * i + 1] * s;
+            y[2 * i + 1] = x[2 * i] * s + x[2 * i + 1] * c;
+        }
+    } else {
+        const bool left = d0 < half;
+        const uint4 oraw = *reinterpret_cast<const uint4*>(head_vec + (left ? d0 + half : d0 - half));
+        const uint32_t ow[4] = {oraw.x, oraw.y, oraw.z, oraw.w};
+        const int i0 = left ? d0 : d0 - half;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float o = (e & 1) ? __uint_as_float(ow[e >> 1] & 0xffff0000u) : __uint_as_float(ow[e >> 1] << 16);
+            const float c = bf16_to_f32(cs[i0 + e]), s = bf16_to_f32(sn[i0 + e]);
+            y[e] = left ? x[e] * c - o * s : x[e] * c + o * s;
+        }
+    }
+    return make_uint4(pack_bf16x2(y[0], y[1]), pack_bf16x2(y[2], y[3]), pack_bf16x2(y[4], y[5]), pack_bf16x2(y[6], y[7]));
+}
 
 constexpr int kVtPitch = kHeadDim + 8;                         // LDS row pitch (elements) of the V tile
 
@@ -55,12 +115,27 @@ void decode_append_kernel(const DecodeParams p) {
     const int h = static_cast<int>(r % p.num_heads_k); r /= p.num_heads_k;
     const int t = static_cast<int>(r % p.seqlen_new);
     const int b = static_cast<int>(r / p.seqlen_new);
-    const int pos = (p.cache_seqlens ? p.cache_seqlens[b] : 0) + t;
+    const int pos = (p.cache_seqlens ? p.cache_seqlens[b] : 0) + t;             // cache row, left padding included
     if (pos >= p.capacity) return;
-    const uint4 kv = *reinterpret_cast<const uint4*>(p.knew + b * p.kn_batch + t * p.kn_row + h * p.kn_head + chunk * 8);
+    const bf16_bits* kvec = p.knew + b * p.kn_batch + t * p.kn_row + h * p.kn_head;
+    const uint4 kv = p.rotary_dim > 0 ? rotary_chunk(p, kvec, chunk, pos) : *reinterpret_cast<const uint4*>(kvec + chunk * 8);
     const uint4 vv = *reinterpret_cast<const uint4*>(p.vnew + b * p.vn_batch + t * p.vn_row + h * p.vn_head + chunk * 8);
-    *reinterpret_cast<uint4*>(p.kcache + b * p.kc_batch + static_cast<int64_t>(pos) * p.kc_row + h * p.kc_head + chunk * 8) = kv;
-    *reinterpret_cast<uint4*>(p.vcache + b * p.vc_batch + static_cast<int64_t>(pos) * p.vc_row + h * p.vc_head + chunk * 8) = vv;
+    *reinterpret_cast<uint4*>(p.kcache + cache_row_offset(p, b, pos, p.kc_batch, p.kc_row) + h * p.kc_head + chunk * 8) = kv;
+    *reinterpret_cast<uint4*>(p.vcache + cache_row_offset(p, b, pos, p.vc_batch, p.vc_row) + h * p.vc_head + chunk * 8) = vv;
+}
+
+// the query turned at the position of the first appended key (all 16 grouped heads of the single query token take
+// the same position: the non-causal rule of flash_fwd_kernel.h:899-901)
+__global__ __launch_bounds__(256)
+void decode_rotate_q_kernel(const DecodeParams p) {
+    const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    const int heads = p.num_heads_k * 16;
+    if (idx >= static_cast<int64_t>(p.batch) * heads * 16) return;
+    const int chunk = static_cast<int>(idx & 15);
+    const int head = static_cast<int>((idx >> 4) % heads), b = static_cast<int>((idx >> 4) / heads);
+    const int pos = p.cache_seqlens ? p.cache_seqlens[b] : 0;
+    *reinterpret_cast<uint4*>(p.q_rot + (static_cast<int64_t>(b) * heads + head) * kHeadDim + chunk * 8) =
+        rotary_chunk(p, p.q + b * p.q_batch + head * p.q_head, chunk, pos);
 }
 
 template <bool kDirect>
@@ -70,8 +145,10 @@ void decode_split_kernel(const DecodeParams p) {
     const int lane = threadIdx.x;
     const int n = lane & 15, g = lane >> 4;
     const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const int lp = p.leftpad ? p.leftpad[b] : 0;              // the sequence's key 0 is cache row lp
     int L = (p.cache_seqlens ? p.cache_seqlens[b] : p.capacity - p.seqlen_new) + p.seqlen_new;
     if (L > p.capacity) L = p.capacity;
+    L -= lp;                                                   // keys of the sequence; mask block j = keys 64 j ..
     const int last_blk = L <= 0 ? -1 : ((L - 1) >> 6);
     const uint64_t* row = p.mask ? p.mask + (static_cast<int64_t>(b) * p.num_heads_k + h) * p.n64 : nullptr;
     BlockWalker walk;
@@ -97,7 +174,9 @@ void decode_split_kernel(const DecodeParams p) {
 
     bf16x8 qf[4];
     {
-        const bf16_bits* qp = p.q + b * p.q_batch + (16 * h + n) * p.q_head + 8 * g;
+        const bf16_bits* qp = p.rotary_dim > 0
+            ? p.q_rot + (static_cast<int64_t>(b) * p.num_heads_k * 16 + 16 * h + n) * kHeadDim + 8 * g
+            : p.q + b * p.q_batch + (16 * h + n) * p.q_head + 8 * g;
 #pragma unroll
         for (int c = 0; c < 4; ++c) qf[c] = *reinterpret_cast<const bf16x8*>(qp + 32 * c);
     }
@@ -106,19 +185,20 @@ void decode_split_kernel(const DecodeParams p) {
 #pragma unroll
     for (int dt = 0; dt < 8; ++dt) o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    const bf16_bits* kbase = p.kcache + b * p.kc_batch + h * p.kc_head;
-    const bf16_bits* vbase = p.vcache + b * p.vc_batch + h * p.vc_head;
     int j = -1;
     for (int skip = 0; skip <= begin && count > 0; ++skip) j = walk.next();   // ordinal `begin` of the row
     for (int it = 0; it < count && j >= 0; ++it) {
         const int key0 = j * kBlockN;
+        // a block never straddles two pages (page_size is a multiple of 64 and paged caches have no left padding)
+        const bf16_bits* kbase = p.kcache + cache_row_offset(p, b, lp + key0, p.kc_batch, p.kc_row) + h * p.kc_head;
+        const bf16_bits* vbase = p.vcache + cache_row_offset(p, b, lp + key0, p.vc_batch, p.vc_row) + h * p.vc_head;
         // K rows as A operands; rows past the end are clamped to a valid row and masked below
         bf16x8 kreg[16];
 #pragma unroll
         for (int kt = 0; kt < 4; ++kt) {
             int key = key0 + 16 * kt + n;
             key = key < L ? key : L - 1;
-            const bf16_bits* src = kbase + static_cast<int64_t>(key) * p.kc_row + 8 * g;
+            const bf16_bits* src = kbase + static_cast<int64_t>(key - key0) * p.kc_row + 8 * g;
 #pragma unroll
             for (int c = 0; c < 4; ++c) kreg[kt * 4 + c] = *reinterpret_cast<const bf16x8*>(src + 32 * c);
         }
@@ -129,7 +209,7 @@ void decode_split_kernel(const DecodeParams p) {
             const int unit = lane + 64 * u;
             int key = key0 + (unit >> 4);
             key = key < L ? key : L - 1;
-            vreg[u] = *reinterpret_cast<const uint4*>(vbase + static_cast<int64_t>(key) * p.vc_row + (unit & 15) * 8);
+            vreg[u] = *reinterpret_cast<const uint4*>(vbase + static_cast<int64_t>(key - key0) * p.vc_row + (unit & 15) * 8);
         }
         floatx4 s[4];
 #pragma unroll
@@ -280,9 +360,15 @@ extern "C" int infllmv2_fwd_kvcache_num_splits(int batch, int num_heads_k, int r
     return s;
 }
 
-extern "C" size_t infllmv2_fwd_kvcache_workspace_bytes(int batch, int num_heads_k, int num_splits) {
+static size_t decode_partials_bytes(int batch, int num_heads_k, int num_splits) {
     if (num_splits <= 1) return 0;
     return static_cast<size_t>(batch) * num_heads_k * num_splits * 16 * (kHeadDim + 1) * sizeof(float);
+}
+
+extern "C" size_t infllmv2_fwd_kvcache_workspace_bytes(int batch, int num_heads_k, int num_splits) {
+    // per-split partial results, then room for the query turned by the rotary embedding
+    return decode_partials_bytes(batch, num_heads_k, num_splits) +
+           static_cast<size_t>(batch) * num_heads_k * 16 * kHeadDim * sizeof(bf16_bits);
 }
 
 extern "C" int infllmv2_fwd_kvcache(void* stream, const void* q, void* kcache, void* vcache, const void* k_new,
@@ -292,7 +378,10 @@ extern "C" int infllmv2_fwd_kvcache(void* stream, const void* q, void* kcache, v
                                     int seqlen_new, const int64_t* q_strides, const int64_t* kcache_strides,
                                     const int64_t* vcache_strides, const int64_t* knew_strides,
                                     const int64_t* vnew_strides, const int64_t* o_strides, int n_uint64_per_row,
-                                    int num_splits, float softmax_scale) {
+                                    int num_splits, float softmax_scale, const int32_t* cache_batch_idx,
+                                    const int32_t* cache_leftpad, const int32_t* block_table,
+                                    int64_t block_table_batch_stride, int page_block_size, const void* rotary_cos,
+                                    const void* rotary_sin, int rotary_dim, int rotary_interleaved) {
     IV2_CHECK(head_dim == kHeadDim, "fwd_kvcache: this build only supports head_dim 128 (got %d)", head_dim);
     IV2_CHECK(seqlen_q == 1, "fwd_kvcache: this build only supports one query token per sequence (got %d)", seqlen_q);
     IV2_CHECK(num_heads_k > 0 && num_heads == num_heads_k * kGroup,
@@ -307,7 +396,19 @@ extern "C" int infllmv2_fwd_kvcache(void* stream, const void* q, void* kcache, v
     IV2_CHECK(num_splits >= 1 && num_splits <= 64, "fwd_kvcache: num_splits must be in [1, 64]");
     IV2_CHECK(workspace_bytes >= infllmv2_fwd_kvcache_workspace_bytes(batch, num_heads_k, num_splits),
               "fwd_kvcache: workspace too small");
-    IV2_CHECK(num_splits == 1 || workspace != nullptr, "fwd_kvcache: split decode needs a workspace");
+    IV2_CHECK(workspace != nullptr || (num_splits == 1 && rotary_cos == nullptr), "fwd_kvcache: split decode and rotary need a workspace");
+    IV2_CHECK(block_table == nullptr || cache_batch_idx == nullptr, "Paged KVcache does not support cache_batch_idx");
+    IV2_CHECK(block_table == nullptr || cache_leftpad == nullptr,
+              "We don't support Paged KV and leftpad_k running at the same time yet");
+    IV2_CHECK(block_table == nullptr || (page_block_size > 0 && page_block_size % kBlockN == 0 && block_table_batch_stride > 0),
+              "fwd_kvcache: the page size of a paged KV cache must be a positive multiple of 64 (got %d)", page_block_size);
+    IV2_CHECK((rotary_cos == nullptr) == (rotary_sin == nullptr), "If rotary cos is provided, rotary sin must also be provided");
+    IV2_CHECK(rotary_cos == nullptr || k_new != nullptr,
+              "If rotary cos/sin are provided, new key / value to be appended to KV cache must also be provided");
+    IV2_CHECK(rotary_cos == nullptr || (rotary_dim > 0 && rotary_dim <= head_dim), "rotary_dim must be <= headdim");
+    IV2_CHECK(rotary_cos == nullptr || rotary_dim % 16 == 0, "Only rotary dimensions divisible by 16 are currently supported");
+    IV2_CHECK(rotary_cos == nullptr || (reinterpret_cast<uintptr_t>(rotary_cos) % 2 == 0 && reinterpret_cast<uintptr_t>(rotary_sin) % 2 == 0),
+              "fwd_kvcache: rotary tables must be 2-byte aligned");
     const void* aligned16[] = {q, kcache, vcache, out};
     for (const void* a : aligned16) IV2_CHECK(reinterpret_cast<uintptr_t>(a) % 16 == 0, "fwd_kvcache: tensors must be 16-byte aligned");
     IV2_CHECK(q_strides[0] % 8 == 0 && q_strides[1] % 8 == 0 && o_strides[0] % 8 == 0 && o_strides[1] % 8 == 0,
@@ -333,6 +434,11 @@ extern "C" int infllmv2_fwd_kvcache(void* stream, const void* q, void* kcache, v
     p.seqlen_new = k_new ? seqlen_new : 0;
     p.n64 = n_uint64_per_row; p.splits = num_splits;
     p.scale_log2 = softmax_scale * 1.44269504088896340736f;
+    p.cache_batch_idx = cache_batch_idx; p.leftpad = cache_leftpad;
+    p.block_table = block_table; p.bt_batch = block_table_batch_stride; p.page_size = block_table ? page_block_size : 1;
+    p.rot_cos = static_cast<const bf16_bits*>(rotary_cos); p.rot_sin = static_cast<const bf16_bits*>(rotary_sin);
+    p.rotary_dim = rotary_cos ? rotary_dim : 0; p.rotary_interleaved = rotary_interleaved;
+    p.q_rot = reinterpret_cast<bf16_bits*>(static_cast<unsigned char*>(workspace) + decode_partials_bytes(batch, num_heads_k, num_splits));
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (k_new != nullptr) {
         IV2_CHECK(reinterpret_cast<uintptr_t>(k_new) % 16 == 0 && reinterpret_cast<uintptr_t>(v_new) % 16 == 0,
@@ -344,6 +450,11 @@ extern "C" int infllmv2_fwd_kvcache(void* stream, const void* q, void* kcache, v
         const int64_t total = static_cast<int64_t>(batch) * seqlen_new * num_heads_k * 16;
         hipLaunchKernelGGL(decode_append_kernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, st, p);
         IV2_LAUNCH_CHECK();
+        if (p.rotary_dim > 0) {
+            const int64_t units = static_cast<int64_t>(batch) * num_heads * 16;
+            hipLaunchKernelGGL(decode_rotate_q_kernel, dim3(static_cast<unsigned>((units + 255) / 256)), dim3(256), 0, st, p);
+            IV2_LAUNCH_CHECK();
+        }
     }
     const dim3 grid(num_splits, num_heads_k, batch);
     if (num_splits == 1) {

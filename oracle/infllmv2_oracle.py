@@ -26,7 +26,9 @@ Pinning status (how each function is checked independently of its own formula, s
 * stage-1 compressed LSE: closed form, reduces to exact mode when v is k.
 * stage-2 forward: dense masked softmax; stage-2 backward: central finite
   differences in fp64 on tiny shapes + softmax-Jacobian identities.
-* decode: the stage-2 forward oracle with one query token.
+* decode: the stage-2 forward oracle with one query token; its options (paged cache,
+  cache_batch_idx, left padding) are gathers checked by relabelling invariance, rotary by
+  complex multiplication, norm preservation, angle addition and the identity at angle 0.
 
 Unpinned here (stated in the tests that touch it): the tie order of the *external*
 ``torch.topk`` the reference's callers use (PyTorch leaves it unspecified); this
@@ -431,6 +433,78 @@ def decode_forward(q, k_cache, v_cache, cache_seqlens, fwd_mask_words, softmax_s
         words = None if fwd_mask_words is None else np.asarray(fwd_mask_words)[b]
         o, ls = stage2_forward(np.asarray(q[b], dtype=dtype), np.asarray(k_cache[b, :L], dtype=dtype),
                                np.asarray(v_cache[b, :L], dtype=dtype), cu_q, cu_k, words,
+                               softmax_scale, False, dtype=dtype)
+        out[b] = o
+        lse[b, :, 0] = ls.reshape(Hk, 1, G).reshape(-1)
+    return out, lse
+
+
+def rotary_apply(x: np.ndarray, cos: np.ndarray, sin: np.ndarray, pos: int, interleaved: bool) -> np.ndarray:
+    """Rotary embedding of the rows of ``x`` (..., d) at position ``pos`` (csrc/flash_attn/src/rotary.h:19-82
+    interleaved, :84-150 contiguous): only the first ``rotary_dim = 2 * cos.shape[1]`` columns turn.
+    interleaved: pairs (2i, 2i+1); contiguous: pairs (i, i + rotary_dim/2);
+    (a, b) -> (a cos_i - b sin_i, a sin_i + b cos_i), fp32 arithmetic, result rounded to bf16."""
+    x = np.asarray(x, dtype=np.float32).copy()
+    half = cos.shape[1]
+    c = np.asarray(cos[pos], dtype=np.float32)
+    s_ = np.asarray(sin[pos], dtype=np.float32)
+    if interleaved:
+        a, b = x[..., 0:2 * half:2].copy(), x[..., 1:2 * half:2].copy()
+        x[..., 0:2 * half:2] = a * c - b * s_
+        x[..., 1:2 * half:2] = a * s_ + b * c
+    else:
+        a, b = x[..., :half].copy(), x[..., half:2 * half].copy()
+        x[..., :half] = a * c - b * s_
+        x[..., half:2 * half] = a * s_ + b * c
+    return bf16_round(x)
+
+
+def decode_forward_ext(q, k_cache, v_cache, cache_seqlens, fwd_mask_words, softmax_scale: float, k_new=None,
+                       v_new=None, cache_batch_idx=None, cache_leftpad=None, block_table=None, rotary_cos=None,
+                       rotary_sin=None, rotary_interleaved=True, dtype=np.float64):
+    """mha_fwd_kvcache with its remaining options (flash_api.cpp:1549-1843, flash_fwd_kernel.h:606-1199):
+    * cache_batch_idx (b): sequence b lives in cache row cache_batch_idx[b];
+    * cache_leftpad (b): the sequence's keys are cache rows [leftpad, cache_seqlens) (block_info.h:23-25, 41-43);
+      mask block j covers rows leftpad + 64 j ...;
+    * block_table (b, max_pages): the caches are (num_pages, page_size, Hk, d) and row r of sequence b is row
+      r % page_size of page block_table[b, r // page_size];
+    * rotary_cos/sin (seqlen_ro, rotary_dim/2): the new keys are turned at their cache rows cache_seqlens[b] + t and
+      the query at cache_seqlens[b] (the non-causal rule, flash_fwd_kernel.h:899-901) before anything else.
+    The caches are updated in place.  Returns out (b, 1, Hq, d), lse (b, Hq, 1)."""
+    B, Sq, Hq, d = q.shape
+    assert Sq == 1
+    Hk = k_cache.shape[2]
+    G = Hq // Hk
+    out = np.zeros((B, 1, Hq, d), dtype=dtype)
+    lse = np.full((B, Hq, 1), np.inf, dtype=dtype)
+
+    def rows(b, lo, hi):
+        """(cache index array, row index array) of rows lo..hi-1 of sequence b"""
+        r = np.arange(lo, hi)
+        if block_table is not None:
+            page = k_cache.shape[1]
+            return np.asarray(block_table)[b, r // page], r % page
+        cb = b if cache_batch_idx is None else int(cache_batch_idx[b])
+        return np.full(r.shape, cb), r
+
+    for b in range(B):
+        end = int(cache_seqlens[b])
+        lp = 0 if cache_leftpad is None else int(cache_leftpad[b])
+        qb = np.asarray(q[b], dtype=np.float32)
+        if k_new is not None:
+            n = k_new.shape[1]
+            ci, ri = rows(b, end, end + n)
+            kn = np.asarray(k_new[b], dtype=np.float32)
+            if rotary_cos is not None:
+                kn = np.stack([rotary_apply(kn[t], rotary_cos, rotary_sin, end + t, rotary_interleaved) for t in range(n)])
+                qb = rotary_apply(qb, rotary_cos, rotary_sin, end, rotary_interleaved)
+            k_cache[ci, ri] = kn
+            v_cache[ci, ri] = v_new[b]
+            end += n
+        ci, ri = rows(b, lp, end)
+        words = None if fwd_mask_words is None else np.asarray(fwd_mask_words)[b]
+        o, ls = stage2_forward(np.asarray(qb, dtype=dtype), np.asarray(k_cache[ci, ri], dtype=dtype),
+                               np.asarray(v_cache[ci, ri], dtype=dtype), [0, 1], [0, end - lp], words,
                                softmax_scale, False, dtype=dtype)
         out[b] = o
         lse[b, :, 0] = ls.reshape(Hk, 1, G).reshape(-1)

@@ -404,3 +404,121 @@ def test_decode_is_stage2_with_one_query():
         ref = _torch_stage2(q[b], kc2[b, :L], vc2[b, :L], [0, 1], [0, L], bits, 128 ** -0.5, False)
         assert np.abs(out[b] - ref).max() < 1e-9
     assert lse.shape == (B, 32, 1)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# decode options (rotary, paged cache, cache_batch_idx, left padding)
+# ---------------------------------------------------------------------------------------------------------------
+def _angles(n_pos, half, seed=0):
+    rng = np.random.default_rng(seed)
+    theta = rng.uniform(-np.pi, np.pi, size=(n_pos, half))
+    return O.bf16_round(np.cos(theta).astype(np.float32)), O.bf16_round(np.sin(theta).astype(np.float32)), theta
+
+
+@pytest.mark.parametrize("interleaved", [True, False])
+@pytest.mark.parametrize("half", [8, 32, 64])
+def test_rotary_is_complex_multiplication(interleaved, half):
+    """Each pair (a, b) becomes (a + ib)(cos + i sin) (rotary.h:57-62, 131-133); columns beyond rotary_dim stay."""
+    rng = np.random.default_rng(1)
+    cos, sin, _ = _angles(5, half)
+    x = O.bf16_round(rng.standard_normal((3, 128)).astype(np.float32))
+    y = O.rotary_apply(x, cos, sin, 3, interleaved)
+    if interleaved:
+        za = x[:, 0:2 * half:2] + 1j * x[:, 1:2 * half:2]
+        zb = y[:, 0:2 * half:2] + 1j * y[:, 1:2 * half:2]
+    else:
+        za = x[:, :half] + 1j * x[:, half:2 * half]
+        zb = y[:, :half] + 1j * y[:, half:2 * half]
+    want = za * (cos[3].astype(np.float64) + 1j * sin[3].astype(np.float64))
+    assert np.allclose(zb, want, rtol=2 ** -7, atol=1e-6)                 # one bf16 rounding
+    assert np.array_equal(y[:, 2 * half:], x[:, 2 * half:])
+
+
+def test_rotary_identity_norm_and_angle_addition():
+    half = 64
+    x = np.random.default_rng(2).standard_normal((4, 128)).astype(np.float32)
+    one, zero = np.ones((1, half), np.float32), np.zeros((1, half), np.float32)
+    for inter in (True, False):
+        assert np.array_equal(O.rotary_apply(O.bf16_round(x), one, zero, 0, inter), O.bf16_round(x))
+        # a quarter turn maps (a, b) to (-b, a)
+        y = O.rotary_apply(O.bf16_round(x), zero, one, 0, inter)
+        xb = O.bf16_round(x)
+        if inter:
+            assert np.array_equal(y[:, 0::2], -xb[:, 1::2]) and np.array_equal(y[:, 1::2], xb[:, 0::2])
+        else:
+            assert np.array_equal(y[:, :half], -xb[:, half:]) and np.array_equal(y[:, half:], xb[:, :half])
+    # exact (unrounded) angles: norms are preserved and two turns add up, within bf16 rounding of the result
+    theta = np.random.default_rng(3).uniform(-3, 3, size=(2, half))
+    c, s_ = np.cos(theta).astype(np.float32), np.sin(theta).astype(np.float32)
+    y = O.rotary_apply(O.bf16_round(x), c, s_, 0, True)
+    assert np.allclose(np.linalg.norm(y, axis=1), np.linalg.norm(O.bf16_round(x), axis=1), rtol=2e-3)
+    c2, s2 = np.cos(theta[:1] + theta[1:]).astype(np.float32), np.sin(theta[:1] + theta[1:]).astype(np.float32)
+    twice = O.rotary_apply(O.rotary_apply(O.bf16_round(x), c, s_, 0, True), c, s_, 1, True)
+    assert np.allclose(twice, O.rotary_apply(O.bf16_round(x), c2, s2, 0, True), atol=0.05)
+
+
+def _decode_case(seed, B=3, cap=512, Hk=2):
+    rng = np.random.default_rng(seed)
+    q = O.bf16_round(rng.standard_normal((B, 1, 16 * Hk, 128)).astype(np.float32))
+    kc = O.bf16_round(rng.standard_normal((B, cap, Hk, 128)).astype(np.float32))
+    vc = O.bf16_round(rng.standard_normal((B, cap, Hk, 128)).astype(np.float32))
+    lens = np.array([200, 333, 448][:B], dtype=np.int32)
+    idx = np.stack([np.stack([np.sort(rng.choice(cap // 64, size=4, replace=False)) for _ in range(Hk)]) for _ in range(B)])
+    words = O.topk_to_uint64(idx.reshape(B, Hk, 1, 4).astype(np.int32), cap, 64)[0]
+    return q, kc, vc, lens, words
+
+
+def test_decode_ext_reduces_to_plain_decode():
+    q, kc, vc, lens, words = _decode_case(4)
+    a = O.decode_forward(q, kc.copy(), vc.copy(), lens, words, 128 ** -0.5)
+    b = O.decode_forward_ext(q, kc.copy(), vc.copy(), lens, words, 128 ** -0.5)
+    assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1])
+
+
+def test_decode_ext_relabelling_invariance():
+    """Paging, cache_batch_idx and left padding only say where a sequence's rows lie: moving the rows and telling
+    the oracle where they went must not change the result."""
+    q, kc, vc, lens, words = _decode_case(5)
+    base = O.decode_forward_ext(q, kc.copy(), vc.copy(), lens, words, 128 ** -0.5)
+    B, cap = kc.shape[:2]
+    # cache_batch_idx: shuffle the sequences inside a larger cache
+    perm = np.array([4, 0, 2])
+    big_k, big_v = np.zeros((6,) + kc.shape[1:], np.float32), np.zeros((6,) + vc.shape[1:], np.float32)
+    big_k[perm], big_v[perm] = kc, vc
+    got = O.decode_forward_ext(q, big_k, big_v, lens, words, 128 ** -0.5, cache_batch_idx=perm)
+    assert np.array_equal(got[0], base[0]) and np.array_equal(got[1], base[1])
+    # paged: cut every sequence into pages of 128 rows and scatter them
+    page = 128
+    n_pages = B * cap // page
+    order = np.random.default_rng(6).permutation(n_pages)
+    table = order.reshape(B, cap // page).astype(np.int32)
+    pk, pv = np.zeros((n_pages, page) + kc.shape[2:], np.float32), np.zeros((n_pages, page) + kc.shape[2:], np.float32)
+    pk[table.reshape(-1)] = kc.reshape(n_pages, page, *kc.shape[2:])
+    pv[table.reshape(-1)] = vc.reshape(n_pages, page, *vc.shape[2:])
+    got = O.decode_forward_ext(q, pk, pv, lens, words, 128 ** -0.5, block_table=table)
+    assert np.array_equal(got[0], base[0]) and np.array_equal(got[1], base[1])
+    # left padding: shift every sequence right by its pad
+    pad = np.array([7, 64, 30], dtype=np.int32)
+    sk, sv = np.zeros_like(kc), np.zeros_like(vc)
+    for b in range(B):
+        sk[b, pad[b]:pad[b] + lens[b]] = kc[b, :lens[b]]
+        sv[b, pad[b]:pad[b] + lens[b]] = vc[b, :lens[b]]
+    got = O.decode_forward_ext(q, sk, sv, lens + pad, words, 128 ** -0.5, cache_leftpad=pad)
+    assert np.array_equal(got[0], base[0]) and np.array_equal(got[1], base[1])
+
+
+def test_decode_ext_rotary_equals_rotating_by_hand():
+    q, kc, vc, lens, words = _decode_case(7)
+    rng = np.random.default_rng(8)
+    kn = O.bf16_round(rng.standard_normal((3, 2, 2, 128)).astype(np.float32))
+    vn = O.bf16_round(rng.standard_normal((3, 2, 2, 128)).astype(np.float32))
+    cos, sin, _ = _angles(600, 32, seed=9)
+    got = O.decode_forward_ext(q, kc.copy(), vc.copy(), lens, words, 128 ** -0.5, k_new=kn, v_new=vn,
+                               rotary_cos=cos, rotary_sin=sin, rotary_interleaved=False)
+    q2, kn2 = q.copy(), kn.copy()
+    for b in range(3):
+        q2[b] = O.rotary_apply(q[b], cos, sin, int(lens[b]), False)
+        for t in range(2):
+            kn2[b, t] = O.rotary_apply(kn[b, t], cos, sin, int(lens[b]) + t, False)
+    want = O.decode_forward(q2, kc.copy(), vc.copy(), lens, words, 128 ** -0.5, k_new=kn2, v_new=vn)
+    assert np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1])
