@@ -16,7 +16,10 @@ from .attention import (
     infllmv2_attn_with_kvcache,
 )
 
+from .layer import InfLLMv2Attention, SequenceCache
+
 __all__ = [
+    "InfLLMv2Attention", "SequenceCache",
     "blockmask_to_uint64", "topk_to_uint64", "uint64_to_bool", "transpose_blockmask",
     "max_pooling_1d", "max_pooling_1d_varlen", "topk_blocks", "compress_keys", "select_blocks",
     "infllmv2_attn_varlen_func", "infllmv2_attn_stage1", "infllmv2_attn_stage1_pooled",
