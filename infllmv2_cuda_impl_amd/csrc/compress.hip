@@ -41,37 +41,41 @@ struct CompressParams {
     int first_row;                   // rows before this one are left alone (appending to a cache of compressed keys)
 };
 
+constexpr int kCompressRowsPerWg = 8;
+
 __global__ __launch_bounds__(256)
 void compress_keys_kernel(const CompressParams p) {
     const int b = blockIdx.y;
     const int k0 = p.cu_k[b];
     const int rows = compressed_rows(p.cu_k[b + 1] - k0, p.kernel_size, p.stride);
-    const int rows_per_wg = 256 / p.units_per_row;             // units_per_row divides 256 (checked by the launcher)
-    const int j = p.first_row + blockIdx.x * rows_per_wg + threadIdx.x / p.units_per_row;
-    if (j >= rows) return;
-    const int u = threadIdx.x % p.units_per_row;
-    const int head = u / p.units_per_head, piece = u % p.units_per_head;
-    const bf16_bits* src = p.k + (static_cast<int64_t>(k0) + static_cast<int64_t>(j) * p.stride) * p.k_row_stride +
-                           head * p.k_head_stride + piece * 8;
-    float acc[8];
+    const int j0 = p.first_row + blockIdx.x * kCompressRowsPerWg;
+    for (int item = threadIdx.x; item < kCompressRowsPerWg * p.units_per_row; item += 256) {
+        const int j = j0 + item / p.units_per_row;
+        if (j >= rows) break;                                  // items are ordered by row
+        const int u = item % p.units_per_row;
+        const int head = u / p.units_per_head, piece = u % p.units_per_head;
+        const bf16_bits* src = p.k + (static_cast<int64_t>(k0) + static_cast<int64_t>(j) * p.stride) * p.k_row_stride +
+                               head * p.k_head_stride + piece * 8;
+        float acc[8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) acc[e] = 0.f;
-    for (int i = 0; i < p.kernel_size; ++i) {
-        const uint4 raw = *reinterpret_cast<const uint4*>(src + i * p.k_row_stride);
-        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+        for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+        for (int i = 0; i < p.kernel_size; ++i) {
+            const uint4 raw = *reinterpret_cast<const uint4*>(src + i * p.k_row_stride);
+            const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            acc[2 * e] += __uint_as_float(w[e] << 16);
-            acc[2 * e + 1] += __uint_as_float(w[e] & 0xffff0000u);
+            for (int e = 0; e < 4; ++e) {
+                acc[2 * e] += __uint_as_float(w[e] << 16);
+                acc[2 * e + 1] += __uint_as_float(w[e] & 0xffff0000u);
+            }
         }
+        const float n = static_cast<float>(p.kernel_size);
+        uint4 o;
+        o.x = pack_bf16x2(acc[0] / n, acc[1] / n);
+        o.y = pack_bf16x2(acc[2] / n, acc[3] / n);
+        o.z = pack_bf16x2(acc[4] / n, acc[5] / n);
+        o.w = pack_bf16x2(acc[6] / n, acc[7] / n);
+        *reinterpret_cast<uint4*>(p.out + (static_cast<int64_t>(p.cu_out[b]) + j) * p.units_per_row * 8 + u * 8) = o;
     }
-    const float n = static_cast<float>(p.kernel_size);
-    uint4 o;
-    o.x = pack_bf16x2(acc[0] / n, acc[1] / n);
-    o.y = pack_bf16x2(acc[2] / n, acc[3] / n);
-    o.z = pack_bf16x2(acc[4] / n, acc[5] / n);
-    o.w = pack_bf16x2(acc[6] / n, acc[7] / n);
-    *reinterpret_cast<uint4*>(p.out + (static_cast<int64_t>(p.cu_out[b]) + j) * p.units_per_row * 8 + u * 8) = o;
 }
 
 }  // namespace infllmv2
@@ -87,7 +91,6 @@ extern "C" int infllmv2_compress_keys(void* stream, const void* k, void* out, co
     IV2_CHECK(k && out && cu_seqlens_k && cu_seqlens_out, "compress_keys: null pointer");
     IV2_CHECK(head_dim > 0 && head_dim % 8 == 0 && num_heads_k > 0, "compress_keys: head_dim must be a multiple of 8");
     const int units = num_heads_k * head_dim / 8;
-    IV2_CHECK(units <= 256 && 256 % units == 0, "compress_keys: num_heads_k * head_dim / 8 = %d must divide 256", units);
     IV2_CHECK(reinterpret_cast<uintptr_t>(k) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 &&
               k_row_stride % 8 == 0 && k_head_stride % 8 == 0, "compress_keys: k and out must be 16-byte aligned, strides multiples of 8");
     hipStream_t st = static_cast<hipStream_t>(stream);
@@ -103,8 +106,7 @@ extern "C" int infllmv2_compress_keys(void* stream, const void* k, void* out, co
     p.k_row_stride = k_row_stride; p.k_head_stride = k_head_stride;
     p.units_per_row = units; p.units_per_head = head_dim / 8;
     p.kernel_size = kernel_size; p.stride = stride; p.first_row = first_row;
-    const int rows_per_wg = 256 / units;
-    const dim3 grid((max_rows - first_row + rows_per_wg - 1) / rows_per_wg, batch);
+    const dim3 grid((max_rows - first_row + kCompressRowsPerWg - 1) / kCompressRowsPerWg, batch);
     hipLaunchKernelGGL(compress_keys_kernel, grid, dim3(256), 0, st, p);
     IV2_LAUNCH_CHECK();
     return 0;

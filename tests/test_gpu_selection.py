@@ -38,6 +38,15 @@ def test_compress_keys_bit_exact(ops, seqs, kernel, stride):
     assert got.shape[0] >= n and np.array_equal(bf16_np(got[:n]), ref)
 
 
+@pytest.mark.parametrize("Hk", [1, 4, 40])
+def test_compress_keys_other_head_counts(ops, Hk):
+    k = rand_k(5, 300, Hk)
+    cu = np.array([0, 300], np.int32)
+    ref, _ = O.compress_keys(bf16_np(k), cu, 32, 16)
+    got, _ = ops.compress_keys(k.cuda(), torch.from_numpy(cu).cuda(), 300, 32, 16)
+    assert np.array_equal(bf16_np(got), ref)
+
+
 def test_compress_keys_strided_input(ops):
     """k as a slice of a fused qkv projection output: row stride larger than heads * d."""
     g = torch.Generator(device="cpu").manual_seed(2)
