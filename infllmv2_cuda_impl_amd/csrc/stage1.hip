@@ -14,10 +14,10 @@
 // Design: S = Q.K^T with the 16 heads of one token as the 16 MFMA rows and 16 compressed keys as
 // the columns, so a lane owns four heads of one key column; the per-head running max/sum of
 // pass 1 stay lane-local until one 16-lane butterfly at the end, and the sum over the 16 heads
-// in pass 2 is an in-lane add of four values plus two cross-lane adds.  A workgroup is 4
-// wavefronts x 4 consecutive tokens; each 64-key tile of compressed keys is staged once in LDS
+// in pass 2 is an in-lane add of four values plus two cross-lane adds.  A workgroup is 8
+// wavefronts x 2 consecutive tokens; each 64-key tile of compressed keys is staged once in LDS
 // (LDS-DMA, straight into MFMA-operand order, read back with conflict-free ds_read_b128) and reused
-// by all 16 tokens, and inside a wavefront one operand read feeds four MFMAs.
+// by all 16 tokens, and inside a wavefront one operand read feeds two MFMAs.
 #include "common.h"
 #include "block_walker.h"
 #include "../../include/infllmv2_hip.h"
@@ -46,8 +46,11 @@ struct Stage1Params {
     int local_blocks, init_blocks;
 };
 
-constexpr int kTokPerWave = 4;
-constexpr int kWavesS1 = 4;
+// 8 wavefronts x 2 tokens: 112 registers, so four wavefronts share a SIMD and the exp-heavy VALU work of one hides
+// behind the MFMAs of another (4 x 4 at two wavefronts per SIMD measures 6 % slower, 8 x 1 15 % slower)
+constexpr int kTokPerWave = 2;
+constexpr int kWavesS1 = 8;
+constexpr int kWavesPerSimdS1 = 4;
 constexpr int kTokPerBlock = kTokPerWave * kWavesS1;   // 16
 constexpr int kKeysPerBlock = 4;                       // compressed keys (stride 16) per 64-token key block
 
@@ -62,9 +65,8 @@ __device__ __forceinline__ int stage1_visible(int i, int s, int L, int Sq, bool 
 }
 
 // A (64 keys x 128 d) tile goes from global memory to LDS by LDS-DMA, in MFMA-operand order: 16-byte unit
-// u = (kt*4 + c)*64 + 16*g + n holds K[16*kt + n][32*c + 8*g ..].  Thread tid of 256 moves units tid + 256*it, i.e.
-// wavefront w moves, for key tile kt = it, the chunk c = w of its 16 keys: lane l's unit lands at
-// lds_base + 16 l, which is exactly operand order, so the operand reads are linear and free of bank conflicts.
+// u = (kt*4 + c)*64 + 16*g + n holds K[16*kt + n][32*c + 8*g ..].  Wavefront w of the workgroup moves the 64-unit groups
+// grp = w, w + 8 (key tile grp / 4, chunk grp % 4 of its 16 keys): lane l's unit lands at lds_base + 16 l, which is exactly operand order, so the operand reads are linear and free of bank conflicts.
 // Keys beyond the last one are read from the last row (finite values that every consumer masks).
 // The compiler's wait counts do not see these loads: the code waits for them by hand before the barrier that
 // publishes the tile.
@@ -78,11 +80,12 @@ __device__ __forceinline__ void s1_dma16(const void* base, uint32_t lane_off, ui
 __device__ __forceinline__ void issue_tile(const bf16_bits* base, int row_stride, int key0, int L, uint32_t lds_tile,
                                            int wave, int n, int g) {
 #pragma unroll
-    for (int it = 0; it < 4; ++it) {
-        int row = key0 + 16 * it + n;
+    for (int it = 0; it < 16 / kWavesS1; ++it) {
+        const int grp = it * kWavesS1 + wave;                  // (kt, c) = (grp / 4, grp % 4)
+        int row = key0 + 16 * (grp >> 2) + n;
         row = row < L ? row : L - 1;
-        const uint32_t off = static_cast<uint32_t>(row * row_stride + 32 * wave + 8 * g) * 2u;
-        s1_dma16(base, off, lds_tile + (it * 4 + wave) * 1024);
+        const uint32_t off = static_cast<uint32_t>(row * row_stride + 32 * (grp & 3) + 8 * g) * 2u;
+        s1_dma16(base, off, lds_tile + grp * 1024);
     }
 }
 
@@ -110,7 +113,7 @@ __device__ __forceinline__ float dpp_quad_xor2(float x) {
 // keys, stride 4, padding 1, forced blocks +inf, empty windows -inf: the rule of csrc/max_pooling_1d.cuh:12-160
 // applied to the scores this kernel would have written, which never reach memory).
 template <bool kCausal, bool kPool>
-__global__ __launch_bounds__(256)
+__global__ __launch_bounds__(64 * kWavesS1) __attribute__((amdgpu_waves_per_eu(kWavesPerSimdS1, kWavesPerSimdS1)))
 void stage1_kernel(const Stage1Params p) {
     __shared__ uint4 tile[2][1024];                            // two 16 KiB operand-ordered key tiles
     const int tid = threadIdx.x;
@@ -385,11 +388,11 @@ int launch_stage1(const char* who, void* stream, const void* q, const void* k, c
     const dim3 grid((max_seqlen_q + kTokPerBlock - 1) / kTokPerBlock, batch, num_heads_k);
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (pool) {
-        if (is_causal) hipLaunchKernelGGL((stage1_kernel<true, true>), grid, dim3(256), 0, st, p);
-        else hipLaunchKernelGGL((stage1_kernel<false, true>), grid, dim3(256), 0, st, p);
+        if (is_causal) hipLaunchKernelGGL((stage1_kernel<true, true>), grid, dim3(64 * kWavesS1), 0, st, p);
+        else hipLaunchKernelGGL((stage1_kernel<false, true>), grid, dim3(64 * kWavesS1), 0, st, p);
     } else {
-        if (is_causal) hipLaunchKernelGGL((stage1_kernel<true, false>), grid, dim3(256), 0, st, p);
-        else hipLaunchKernelGGL((stage1_kernel<false, false>), grid, dim3(256), 0, st, p);
+        if (is_causal) hipLaunchKernelGGL((stage1_kernel<true, false>), grid, dim3(64 * kWavesS1), 0, st, p);
+        else hipLaunchKernelGGL((stage1_kernel<false, false>), grid, dim3(64 * kWavesS1), 0, st, p);
     }
     IV2_LAUNCH_CHECK();
     return 0;
