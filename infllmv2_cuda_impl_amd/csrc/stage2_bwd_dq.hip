@@ -21,7 +21,7 @@
 namespace infllmv2 {
 
 constexpr int kDqTokens = 8;
-constexpr int kDqChunk = 64;                                   // token groups per XCD chunk
+constexpr int kDqChunk = 16;                                   // token groups per XCD chunk
 constexpr int kDqTileBytes = 32768;
 constexpr int kDqMaskWords = 256;                              // LDS copies of the mask rows: up to 16384 key blocks
 constexpr int kDqLdsTiles = 2 * kDqTileBytes + 8 * 8192;       // 2-tile ring + 8 private half K tiles

@@ -30,7 +30,7 @@
 namespace infllmv2 {
 
 constexpr int kHybTokens = 8;                                  // tokens (= wavefronts) per workgroup
-constexpr int kHybChunk = 64;                                  // token groups per XCD chunk
+constexpr int kHybChunk = 16;                                  // token groups per XCD chunk
 constexpr int kRingTiles = 3;
 constexpr int kTileBytes = 32768;                              // K image | V image of one block
 constexpr int kMaxMaskWords = 256;                             // LDS copies of the mask rows: up to 16384 key blocks
