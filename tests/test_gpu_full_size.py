@@ -1,7 +1,8 @@
 """BASELINE-size runs checked through sampled rows and size-independent properties.
 
 Config 2 (prefill, 32768 tokens) end to end; config 3 (four packed sequences, ~64K tokens, forward +
-backward); config 5 (decode, batch 64, cache lengths up to 131072).  Oracle parity on sampled rows; for
+backward); config 4 (prefill, 131072 tokens, fused front end); config 5 (decode, batch 64, cache lengths up to
+131072).  Oracle parity on sampled rows; for
 the rest: forced blocks always selected, popcount == k, sum_keys dV = sum_tokens dO and sum_keys dK = 0
 (rows of P sum to one, rows of dS sum to zero)."""
 import numpy as np
@@ -180,3 +181,50 @@ def test_config5_decode_batch64(ops):
     # split-count independence at full size
     out1 = ops.infllmv2_attn_with_kvcache(q, kc, vc, cache_seqlens=L, topk_idx=idx.to(dev), num_splits=1)
     assert float((out.float() - out1.float()).abs().max()) <= 8e-3
+
+
+def test_config4_prefill_128k_fused_front_end(ops):
+    """BASELINE config 4 (131072 tokens): the one-call selection, which never writes the 4.3 GB score tensor, against
+    the separate calls (bit-exact pooled scores and identical top-k), selection invariants over all rows, and the
+    Stage-2 forward on sampled tokens against the oracle."""
+    dev = torch.device("cuda:0")
+    S, topk = 131072, 64
+    g = torch.Generator(device="cpu").manual_seed(4)
+    q = torch.randn(S, 32, 128, generator=g).to(torch.bfloat16).to(dev)
+    k = torch.randn(S, 2, 128, generator=g).to(torch.bfloat16).to(dev)
+    v = torch.randn(S, 2, 128, generator=g).to(torch.bfloat16).to(dev)
+    mk = lambda n: torch.tensor([0, n], dtype=torch.int32, device=dev)
+    idx = ops.select_blocks(q, k, mk(S), mk(S), S, S, topk, 31, 1)
+    # the separate calls on separately built compressed keys
+    kf, kc = compress(k, 32, 16), compress(k, 128, 64)
+    kf2, cu_f = ops.compress_keys(k, mk(S), S, 32, 16)
+    assert torch.equal(kf2, kf) or float((kf2.float() - kf.float()).abs().max()) <= 2.0 ** -8 * float(kf.float().abs().max())
+    Lk = kf2.shape[0]
+    kc2, cu_c = ops.compress_keys(k, mk(S), S, 128, 64)
+    score = ops.infllmv2_attn_stage1(q, kf2, kc2, mk(S), cu_f, cu_c, S, Lk, causal=True)
+    pooled = ops.max_pooling_1d(score, 0, 31, 1)
+    del score
+    fused = ops.infllmv2_attn_stage1_pooled(q, kf2, kc2, mk(S), cu_f, cu_c, S, Lk, 31, 1, causal=True)
+    assert torch.equal(fused.view(torch.int16), pooled.view(torch.int16))
+    assert torch.equal(idx, ops.topk_blocks(pooled, topk))
+    del pooled, fused
+    words, kb = ops.topk_to_uint64(idx, S, 64)
+    assert kb == 2048 and words.shape[-1] == 32
+    bits = ops.uint64_to_bool(words, kb)
+    tok = torch.arange(S, device=dev)
+    bq = tok // 64
+    assert bool(bits[:, :, 0].all()) and bool((bits.sum(-1) == topk).all())
+    for d in (0, 1, 31):
+        assert bool(bits[:, tok, torch.clamp(bq - d, min=0)].all())
+    # a token with at least topk causal blocks selects nothing from the future (earlier tokens must pad with such blocks,
+    # which the Stage-2 kernels never visit)
+    late = bq >= topk
+    future = torch.arange(kb, device=dev)[None, None, :] > bq[None, late, None]
+    assert not bool((bits[:, late] & future).any())
+    del bits
+    out = ops.infllmv2_attn_varlen_func(q, k, v, mk(S), mk(S), S, S, causal=True, topk_idx=idx)
+    wnp = words_np(words)
+    for r in [0, 63, 4096, 50001, 100000, 131071]:
+        o_ref, _ = token_oracle(q, k, v, wnp[:, r], r, S, S, r)
+        err = np.abs(bf16_np(out[r]) - o_ref)
+        assert err.max() <= 2e-2 and err.mean() <= 1e-3, (r, err.max(), err.mean())
