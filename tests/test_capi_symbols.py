@@ -36,6 +36,55 @@ def test_argument_errors_are_reported_without_gpu():
     assert rc != 0 and b"exceeds" in _lib.lib.infllmv2_last_error()
 
 
+def _err(lib):
+    return lib.infllmv2_last_error().decode()
+
+
+def test_new_entry_points_validate_before_launch():
+    """Argument checks of the fused front end, the compressed-key kernel and the decode options run on the host."""
+    import ctypes as C
+    from infllmv2_cuda_impl_amd import _lib
+    lib = _lib.lib
+    i64 = _lib.i64_array
+    fake = 0x1000                                           # a non-null, 16-byte aligned "pointer"; nothing is launched
+    # fused Stage-1/pool: only the 5/4/1 window on 64-token blocks
+    rc = lib.infllmv2_varlen_fwd_stage1_pooled(None, fake, fake, fake, fake, fake, fake, fake, None, 0, 1, 128, 32, 2, 128,
+                                               128, 7, i64([4096, 128, 2048]), i64([256, 128]), i64([256, 128]), 2,
+                                               0.088, 1, 9, 8, 1, 128, 1, 1)
+    assert rc != 0 and "only the 5/4/1 window" in _err(lib)
+    # Stage 1: head_dim, group size, alignment
+    rc = lib.infllmv2_varlen_fwd_stage1(None, fake, fake, fake, fake, fake, fake, fake, 1, 128, 32, 2, 64, 128, 7,
+                                        i64([4096, 128, 2048]), i64([256, 128]), i64([256, 128]), 896, 7, 0.088, 1)
+    assert rc != 0 and "head_dim 128" in _err(lib)
+    rc = lib.infllmv2_varlen_fwd_stage1(None, fake, fake, fake, fake, fake, fake, fake, 1, 128, 24, 2, 128, 128, 7,
+                                        i64([4096, 128, 2048]), i64([256, 128]), i64([256, 128]), 896, 7, 0.088, 1)
+    assert rc != 0 and "16 * num_heads_k" in _err(lib)
+    rc = lib.infllmv2_varlen_fwd_stage1(None, fake + 2, fake, fake, fake, fake, fake, fake, 1, 128, 32, 2, 128, 128, 7,
+                                        i64([4096, 128, 2048]), i64([256, 128]), i64([256, 128]), 896, 7, 0.088, 1)
+    assert rc != 0 and "16-byte aligned" in _err(lib)
+    # compressed keys
+    rc = lib.infllmv2_compress_keys(None, fake, fake, fake, fake, 1, 128, 2, 128, 256, 128, 0, 16, 0)
+    assert rc != 0 and "must be positive" in _err(lib)
+    rc = lib.infllmv2_compress_keys(None, None, fake, fake, fake, 1, 128, 2, 128, 256, 128, 32, 16, 0)
+    assert rc != 0 and "null pointer" in _err(lib)
+    # decode: option conflicts carry the reference's messages (flash_api.cpp:1596, 1763, 1774)
+    def kv(**o):
+        a = dict(knew=None, cbi=None, lp=None, bt=None, page=0, cos=None, sin=None, rd=0)
+        a.update(o)
+        return lib.infllmv2_fwd_kvcache(None, fake, fake, fake, a["knew"], a["knew"], fake, fake, fake, None, fake, 1 << 20,
+                                        1, 1, 32, 2, 128, 512, 1 if a["knew"] else 0, i64([4096, 128]),
+                                        i64([131072, 256, 128]), i64([131072, 256, 128]), i64([256, 256, 128]),
+                                        i64([256, 256, 128]), i64([4096, 128]), 0, 1, 0.088, a["cbi"], a["lp"], a["bt"],
+                                        8 if a["bt"] else 0, a["page"], a["cos"], a["sin"], a["rd"], 1)
+    assert kv(bt=fake, page=256, cbi=fake) != 0 and "does not support cache_batch_idx" in _err(lib)
+    assert kv(bt=fake, page=256, lp=fake) != 0 and "leftpad_k running at the same time" in _err(lib)
+    assert kv(bt=fake, page=100) != 0 and "multiple of 64" in _err(lib)
+    assert kv(cos=fake, sin=fake, rd=64) != 0 and "new key / value to be appended" in _err(lib)
+    assert kv(cos=fake, sin=None, rd=64, knew=fake) != 0 and "rotary sin must also be provided" in _err(lib)
+    assert kv(cos=fake, sin=fake, rd=24, knew=fake) != 0 and "divisible by 16" in _err(lib)
+    assert kv(cos=fake, sin=fake, rd=256, knew=fake) != 0 and "rotary_dim must be <= headdim" in _err(lib)
+
+
 def test_product_package_does_not_import_oracle():
     pkg = os.path.join(ROOT, "infllmv2_cuda_impl_amd")
     for dirpath, _, files in os.walk(pkg):
