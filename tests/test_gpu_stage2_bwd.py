@@ -83,3 +83,22 @@ def test_unselected_blocks_get_zero_gradient(ops):
     ops.infllmv2_attn_varlen_func(qg, kg, vg, cu_q, cu_k, 256, 256, causal=True, topk_idx=idx).sum().backward()
     assert float(kg.grad[64:].abs().max()) == 0.0 and float(vg.grad[64:].abs().max()) == 0.0
     assert float(vg.grad[:64].abs().max()) > 0.0
+
+
+def test_forward_and_dq_are_bit_reproducible(ops):
+    """The reference offers deterministic=True for a reproducible dQ (flash_api.cpp:1448-1453: its default dQ goes
+    through fp32 atomics).  Here out, LSE and dQ never pass through atomics: two runs agree bit for bit, with and
+    without the flag; dK/dV are accumulated with fp32 atomics and agree to rounding."""
+    dev = torch.device("cuda:0")
+    q, k, v, cu_q, cu_k, idx = make_case(7, [1500, 700], [1500, 700], 2, 6, dev)
+    dout = torch.randn(q.shape, generator=torch.Generator(device="cpu").manual_seed(8)).to(torch.bfloat16).to(dev)
+    runs = []
+    for det in (False, True, False):
+        qg, kg, vg = [t.clone().requires_grad_(True) for t in (q, k, v)]
+        out = ops.infllmv2_attn_varlen_func(qg, kg, vg, cu_q, cu_k, 1500, 1500, causal=True, topk_idx=idx, deterministic=det)
+        out.backward(dout)
+        runs.append((out.detach(), qg.grad, kg.grad, vg.grad))
+    for other in runs[1:]:
+        assert torch.equal(runs[0][0], other[0]) and torch.equal(runs[0][1], other[1])
+        for a, b in ((runs[0][2], other[2]), (runs[0][3], other[3])):
+            assert float((a.float() - b.float()).abs().max()) <= 2.0 ** -7 * float(a.float().abs().max())
