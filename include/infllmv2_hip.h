@@ -23,7 +23,7 @@
 extern "C" {
 #endif
 
-#define INFLLMV2_ABI_VERSION 2
+#define INFLLMV2_ABI_VERSION 3
 
 /* ---- library ------------------------------------------------------------------------------ */
 
@@ -190,6 +190,10 @@ int infllmv2_pack_kv(void* stream, const void* k, const void* v, const int32_t* 
  * transposed per-token images of q and dout, fp32 dK/dV accumulators. */
 size_t infllmv2_varlen_bwd_workspace_bytes(int batch, int64_t total_q, int64_t total_k, int num_heads_k,
                                            int max_seqlen_k);
+/* The same plus the slots of the deterministic mode of infllmv2_varlen_bwd (one 64 KiB slot per KV head, key block
+ * and 512-token slice of the packed query axis: 4.4 GB at 32768 tokens, growing with the square of the length). */
+size_t infllmv2_varlen_bwd_deterministic_workspace_bytes(int batch, int64_t total_q, int64_t total_k, int num_heads_k,
+                                                         int max_seqlen_k);
 
 /* csrc/entry.cu:17,213 `varlen_bwd` = mha_varlen_bwd (csrc/flash_attn/flash_api.cpp:1278-1547; kernels
  * flash_bwd_kernel.h:80-856, flash_bwd_preprocess_kernel.h:56-137,181-263) together with the mask
@@ -197,9 +201,11 @@ size_t infllmv2_varlen_bwd_workspace_bytes(int batch, int64_t total_q, int64_t t
  * FORWARD mask (Hk, total_q, n_uint64_per_row), or null for dense attention.
  * dout, q, out, dq: strides {token, head-in-group, kv-head} as in infllmv2_varlen_fwd; k, v, dk, dv:
  * {row, head}; softmax_lse: the forward's output with its strides.  dq, dk, dv are fully written
- * (bf16).  workspace: infllmv2_varlen_bwd_workspace_bytes() bytes, 256-byte aligned.  dK/dV are
- * accumulated with fp32 atomics (one flush per 64-key block and 2048-token slice), so their last bits
- * can differ between runs, as the reference's dQ does; dQ is bit-reproducible. */
+ * (bf16).  workspace: infllmv2_varlen_bwd_workspace_bytes() bytes, 256-byte aligned.  dQ is always
+ * bit-reproducible.  dK/dV are accumulated with fp32 atomics (one flush per 64-key block and 512-token slice),
+ * so their last bits can differ between runs, unless `deterministic` is set (the flag of flash_api.cpp:1448-1453,
+ * which there concerns dQ): then every work item stores its tiles in a slot of its own and a second kernel adds them
+ * in a fixed order; the workspace must then hold infllmv2_varlen_bwd_deterministic_workspace_bytes() bytes. */
 int infllmv2_varlen_bwd(void* stream, const void* dout, const void* q, const void* k, const void* v,
                         const void* out, const float* softmax_lse, void* dq, void* dk, void* dv,
                         const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
@@ -209,7 +215,7 @@ int infllmv2_varlen_bwd(void* stream, const void* dout, const void* q, const voi
                         const int64_t* k_strides, const int64_t* v_strides, const int64_t* o_strides,
                         const int64_t* do_strides, const int64_t* dq_strides, const int64_t* dk_strides,
                         const int64_t* dv_strides, const int64_t* lse_strides, int n_uint64_per_row,
-                        float softmax_scale, int is_causal);
+                        float softmax_scale, int is_causal, int deterministic);
 
 /* ---- Stage 2: decode against a KV cache -------------------------------------------------------- */
 

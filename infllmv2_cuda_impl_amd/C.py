@@ -202,7 +202,9 @@ def varlen_bwd(dout, q, k, v, out, softmax_lse, dq_, dk_, dv_, cu_seqlens_q, cu_
         fwd_mask = transpose_blockmask(col_blockmask_[:, :k_blocks].contiguous(), total_q)   # rows <-> columns
         n64 = fwd_mask.shape[-1]
     total_k = k.shape[0]
-    ws_bytes = _lib.lib.infllmv2_varlen_bwd_workspace_bytes(batch, total_q, total_k, Hk, max_seqlen_k)
+    size_query = (_lib.lib.infllmv2_varlen_bwd_deterministic_workspace_bytes if deterministic
+                  else _lib.lib.infllmv2_varlen_bwd_workspace_bytes)
+    ws_bytes = size_query(batch, total_q, total_k, Hk, max_seqlen_k)
     ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=q.device)
     with torch.cuda.device(q.device):
         _lib.call("infllmv2_varlen_bwd", stream_ptr(q.device), dout.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
@@ -210,7 +212,7 @@ def varlen_bwd(dout, q, k, v, out, softmax_lse, dq_, dk_, dv_, cu_seqlens_q, cu_
                   cu_seqlens_k.data_ptr(), ptr(fwd_mask), ws.data_ptr(), ws.numel(), batch, total_q, total_k, Hq, Hk,
                   q.shape[-1], max_q, max_seqlen_k, _layout(q, expanded), _kv(k), _kv(v), _layout(out, expanded),
                   _layout(dout, expanded), _layout(dq, expanded), _kv(dk), _kv(dv), lse_strides, n64,
-                  float(softmax_scale), int(bool(is_causal)))
+                  float(softmax_scale), int(bool(is_causal)), int(bool(deterministic)))
     return [dq, dk, dv, torch.empty((0,), dtype=torch.float32, device=q.device)]
 
 

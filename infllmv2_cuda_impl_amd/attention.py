@@ -161,7 +161,8 @@ class Infllmv2AttnVarlenFunc(torch.autograd.Function):
         from .backward import sparse_backward
         q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, fwd_mask = ctx.saved_tensors
         dq, dk, dv = sparse_backward(dout, q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, ctx.max_seqlen_q,
-                                     ctx.max_seqlen_k, ctx.softmax_scale, ctx.causal, fwd_mask, ctx.sparse)
+                                     ctx.max_seqlen_k, ctx.softmax_scale, ctx.causal, fwd_mask, ctx.sparse,
+                                     ctx.deterministic)
         return (dq, dk, dv) + (None,) * 14
 
 

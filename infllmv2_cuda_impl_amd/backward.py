@@ -22,8 +22,9 @@ def _nat(t):
 
 
 def sparse_backward(dout, q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, softmax_scale,
-                    causal, fwd_mask, lse_expanded: bool):
-    """Returns (dq, dk, dv) with the shapes and dtype of (q, k, v)."""
+                    causal, fwd_mask, lse_expanded: bool, deterministic: bool = False):
+    """Returns (dq, dk, dv) with the shapes and dtype of (q, k, v).  dq is always bit-reproducible; with
+    ``deterministic`` dk and dv are too (slots + ordered sum instead of fp32 atomics, at the price of a large workspace)."""
     if dout.stride(-1) != 1:
         dout = dout.contiguous()
     if dout.dtype != q.dtype or tuple(dout.shape) != tuple(q.shape):
@@ -36,7 +37,9 @@ def sparse_backward(dout, q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, max_seq
         lse_strides = _lib.i64_array([GROUP, 1, total_q * GROUP])
     else:
         lse_strides = _lib.i64_array([1, total_q, GROUP * total_q])
-    ws_bytes = _lib.lib.infllmv2_varlen_bwd_workspace_bytes(batch, total_q, total_k, Hk, max_seqlen_k)
+    size_query = (_lib.lib.infllmv2_varlen_bwd_deterministic_workspace_bytes if deterministic
+                  else _lib.lib.infllmv2_varlen_bwd_workspace_bytes)
+    ws_bytes = size_query(batch, total_q, total_k, Hk, max_seqlen_k)
     workspace = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=q.device)
     n64 = 0 if fwd_mask is None else fwd_mask.shape[-1]
     kv = lambda t: _lib.i64_array([t.stride(0), t.stride(1)])
@@ -46,5 +49,5 @@ def sparse_backward(dout, q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, max_seq
                   cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), ptr(fwd_mask), workspace.data_ptr(),
                   workspace.numel(), batch, total_q, total_k, Hq, Hk, d, max_seqlen_q, max_seqlen_k,
                   _nat(q), kv(k), kv(v), _nat(out), _nat(dout), _nat(dq), kv(dk), kv(dv), lse_strides, n64,
-                  float(softmax_scale), int(bool(causal)))
+                  float(softmax_scale), int(bool(causal)), int(bool(deterministic)))
     return dq, dk, dv

@@ -33,11 +33,20 @@ struct BwdParams {
     int64_t n_slots, total_q, total_k;
     int n64_fwd, n64_bwd, k_blocks, num_heads_k;
     float scale_log2, scale;
+    // deterministic dK/dV: every (block, 512-token slice) work item stores its two tiles in a slot of its own and a
+    // second kernel adds the slots of a block in slice order (no atomics); null: fp32 atomics into dk_acc / dv_acc
+    float* det_slots;               // (Hk, n_slots, det_slices, 2, 64, 128) fp32
+    uint32_t* det_flags;            // (Hk, n_slots, det_slices): 1 where a slot was written
+    int det_slices;
 };
 
 // dQ, 8 consecutive tokens per workgroup sharing their common blocks through LDS: stage2_bwd_dq.hip
 int launch_bwd_dq_hybrid(hipStream_t st, const BwdParams& p, int batch, int max_seqlen_q, bool causal);
 // dK/dV, one wavefront per (64-key block, 512-token slice): stage2_bwd_dkdv.hip
 int launch_bwd_dkdv_wave(hipStream_t st, const BwdParams& p, int batch, int max_seqlen_q, bool causal);
+
+// deterministic mode only: adds the slots of every key block in slice order into dk_acc / dv_acc
+int launch_bwd_dkdv_reduce(hipStream_t st, const BwdParams& p, int batch);
+constexpr int kDkdvSlice = 512;     // query tokens per dK/dV work item (slices are cut on the packed token axis)
 
 }  // namespace infllmv2

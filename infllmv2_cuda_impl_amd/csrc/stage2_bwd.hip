@@ -87,6 +87,8 @@ static size_t align256(size_t x) { return (x + 255) & ~static_cast<size_t>(255);
 
 struct BwdLayout {
     size_t images, mask, dsum, rowstat, dk_acc, dv_acc, total;
+    size_t det_flags, det_slots, det_total;                    // deterministic mode only, after everything else
+    int det_slices;
 };
 
 static BwdLayout bwd_layout(int batch, int64_t total_q, int64_t total_k, int num_heads_k, int max_seqlen_k) {
@@ -100,6 +102,11 @@ static BwdLayout bwd_layout(int batch, int64_t total_q, int64_t total_k, int num
     L.dk_acc = off; off += align256(static_cast<size_t>(total_k) * num_heads_k * kHeadDim * 4);
     L.dv_acc = off; off += align256(static_cast<size_t>(total_k) * num_heads_k * kHeadDim * 4);
     L.total = off;
+    L.det_slices = static_cast<int>((total_q + kDkdvSlice - 1) / kDkdvSlice) + 1;
+    const size_t items = static_cast<size_t>(num_heads_k) * image_slots(total_k, batch) * L.det_slices;
+    L.det_flags = off; off += align256(items * 4);
+    L.det_slots = off; off += align256(items * 2 * kBlockN * kHeadDim * 4);
+    L.det_total = off;
     return L;
 }
 
@@ -112,6 +119,11 @@ extern "C" size_t infllmv2_varlen_bwd_workspace_bytes(int batch, int64_t total_q
     return bwd_layout(batch, total_q, total_k, num_heads_k, max_seqlen_k).total;
 }
 
+extern "C" size_t infllmv2_varlen_bwd_deterministic_workspace_bytes(int batch, int64_t total_q, int64_t total_k,
+                                                                    int num_heads_k, int max_seqlen_k) {
+    return bwd_layout(batch, total_q, total_k, num_heads_k, max_seqlen_k).det_total;
+}
+
 extern "C" int infllmv2_varlen_bwd(void* stream, const void* dout, const void* q, const void* k, const void* v,
                                    const void* out, const float* softmax_lse, void* dq, void* dk, void* dv,
                                    const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
@@ -121,7 +133,7 @@ extern "C" int infllmv2_varlen_bwd(void* stream, const void* dout, const void* q
                                    const int64_t* k_strides, const int64_t* v_strides, const int64_t* o_strides,
                                    const int64_t* do_strides, const int64_t* dq_strides, const int64_t* dk_strides,
                                    const int64_t* dv_strides, const int64_t* lse_strides, int n_uint64_per_row,
-                                   float softmax_scale, int is_causal) {
+                                   float softmax_scale, int is_causal, int deterministic) {
     IV2_CHECK(head_dim == kHeadDim, "varlen_bwd: this build only supports head_dim 128 (got %d)", head_dim);
     IV2_CHECK(num_heads_k > 0 && num_heads == num_heads_k * kGroup,
               "varlen_bwd: requires num_heads == 16 * num_heads_k (got %d and %d)", num_heads, num_heads_k);
@@ -130,7 +142,8 @@ extern "C" int infllmv2_varlen_bwd(void* stream, const void* dout, const void* q
               "varlen_bwd: null pointer");
     IV2_CHECK(num_heads_k <= 65535 && batch <= 65535, "varlen_bwd: batch and num_heads_k must not exceed 65535");
     const BwdLayout L = bwd_layout(batch, total_q, total_k, num_heads_k, max_seqlen_k);
-    IV2_CHECK(workspace_bytes >= L.total, "varlen_bwd: workspace too small (%zu < %zu)", workspace_bytes, L.total);
+    const size_t ws_needed = deterministic ? L.det_total : L.total;
+    IV2_CHECK(workspace_bytes >= ws_needed, "varlen_bwd: workspace too small (%zu < %zu)", workspace_bytes, ws_needed);
     IV2_CHECK(reinterpret_cast<uintptr_t>(workspace) % 256 == 0, "varlen_bwd: workspace must be 256-byte aligned");
     const void* ptrs16[] = {dout, q, k, v, out};
     for (const void* ptr16 : ptrs16) IV2_CHECK(reinterpret_cast<uintptr_t>(ptr16) % 16 == 0, "varlen_bwd: inputs must be 16-byte aligned");
@@ -178,6 +191,14 @@ extern "C" int infllmv2_varlen_bwd(void* stream, const void* dout, const void* q
     p.scale = softmax_scale;
     p.scale_log2 = softmax_scale * kLog2e;
 
+    if (deterministic) {
+        p.det_flags = reinterpret_cast<uint32_t*>(ws + L.det_flags);
+        p.det_slots = reinterpret_cast<float*>(ws + L.det_slots);
+        p.det_slices = L.det_slices;
+        hipLaunchKernelGGL(zero_f32_kernel, dim3(256), dim3(256), 0, st, reinterpret_cast<float4*>(p.det_flags),
+                           static_cast<int64_t>((L.det_slots - L.det_flags) / 16));
+        IV2_LAUNCH_CHECK();
+    }
     // dK/dV accumulators start at zero (fill kernel, no memset node)
     if (total_k > 0) {
         const int64_t n4 = static_cast<int64_t>((L.dv_acc - L.dk_acc) / 16) * 2;
@@ -203,6 +224,10 @@ extern "C" int infllmv2_varlen_bwd(void* stream, const void* dout, const void* q
         if (rc != 0) return rc;
         rc = launch_bwd_dkdv_wave(st, p, batch, max_seqlen_q, is_causal != 0);
         if (rc != 0) return rc;
+        if (deterministic) {
+            rc = launch_bwd_dkdv_reduce(st, p, batch);
+            if (rc != 0) return rc;
+        }
     } else if (total_q > 0) {
         // no keys at all: dq = 0
         IV2_CHECK(false, "varlen_bwd: empty key set is not supported");

@@ -28,7 +28,7 @@
 
 namespace infllmv2 {
 
-constexpr int kColSlice = 512;                                 // query tokens per work item
+constexpr int kColSlice = kDkdvSlice;                          // query tokens per work item
 constexpr int kGroupSlices = 4;                                // slices that pool their light members
 constexpr int kGroupWords = kGroupSlices * kColSlice / 64;     // = 32: one mask word per lane of the lower half
 constexpr int kHeavyPairs = 128;                               // a slice with fewer selected tokens is "light"
@@ -425,14 +425,70 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
                 *reinterpret_cast<float4*>(tile + (16 * kt + n) * kFlushPitch + 16 * dt + 4 * g) = make_float4(v[0], v[1], v[2], v[3]);
             }
         __syncthreads();
-        float* acc = (which == 0 ? p.dk_acc : p.dv_acc) + (row0 * p.num_heads_k + h) * kHeadDim + lane;
         const float mul = which == 0 ? p.scale : 1.f;
+        if (p.det_slots != nullptr) {
+            // deterministic mode: the tile goes to this work item's own slot (all 64 rows: rows past the sequence
+            // end hold zeros), to be added in slice order by bwd_dkdv_reduce_kernel
+            const int64_t item = (static_cast<int64_t>(h) * p.n_slots + image_slot0(p.cu_seqlens_k, b) + j) * p.det_slices + slice;
+            float* dst = p.det_slots + (item * 2 + which) * (kBlockN * kHeadDim) + lane;
+            for (int key = 0; key < kBlockN; ++key) {
+                dst[key * kHeadDim] = tile[key * kFlushPitch + lane] * mul;
+                dst[key * kHeadDim + 64] = tile[key * kFlushPitch + 64 + lane] * mul;
+            }
+            if (which == 1 && lane == 0) p.det_flags[item] = 1u;
+            continue;
+        }
+        float* acc = (which == 0 ? p.dk_acc : p.dv_acc) + (row0 * p.num_heads_k + h) * kHeadDim + lane;
         for (int key = 0; key < valid_keys; ++key) {
             float* dst = acc + static_cast<int64_t>(key) * p.num_heads_k * kHeadDim;
             unsafeAtomicAdd(dst, tile[key * kFlushPitch + lane] * mul);
             unsafeAtomicAdd(dst + 64, tile[key * kFlushPitch + 64 + lane] * mul);
         }
     }
+}
+
+// Deterministic mode: one workgroup per (key block, sequence, KV head) adds the slots its work items wrote, in
+// ascending slice order, and stores the sums where the atomic mode accumulates.
+__global__ __launch_bounds__(256)
+void bwd_dkdv_reduce_kernel(const BwdParams p) {
+    const int j = blockIdx.x, b = blockIdx.y, h = blockIdx.z;
+    const int k0 = p.cu_seqlens_k[b];
+    const int Sk = p.cu_seqlens_k[b + 1] - k0;
+    if (j * kBlockN >= Sk) return;
+    const int64_t item0 = (static_cast<int64_t>(h) * p.n_slots + image_slot0(p.cu_seqlens_k, b) + j) * p.det_slices;
+    const int valid_keys = (Sk - j * kBlockN) < kBlockN ? (Sk - j * kBlockN) : kBlockN;
+    float4 acc[2][8];                                          // [dK | dV][8 x (256 threads x 4 floats)] = 64 x 128 each
+#pragma unroll
+    for (int w = 0; w < 2; ++w)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[w][i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int s = 0; s < p.det_slices; ++s) {
+        if (p.det_flags[item0 + s] == 0u) continue;            // uniform per workgroup
+        const float4* src = reinterpret_cast<const float4*>(p.det_slots + (item0 + s) * 2 * (kBlockN * kHeadDim)) + threadIdx.x;
+#pragma unroll
+        for (int w = 0; w < 2; ++w)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float4 v = src[w * 2048 + i * 256];
+                acc[w][i].x += v.x; acc[w][i].y += v.y; acc[w][i].z += v.z; acc[w][i].w += v.w;
+            }
+    }
+    const int64_t row0 = static_cast<int64_t>(k0) + static_cast<int64_t>(j) * kBlockN;
+#pragma unroll
+    for (int w = 0; w < 2; ++w)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int e = (i * 256 + threadIdx.x) * 4;         // element of the 64 x 128 tile
+            const int key = e >> 7, d = e & 127;
+            if (key < valid_keys)
+                *reinterpret_cast<float4*>((w == 0 ? p.dk_acc : p.dv_acc) + ((row0 + key) * p.num_heads_k + h) * kHeadDim + d) = acc[w][i];
+        }
+}
+
+int launch_bwd_dkdv_reduce(hipStream_t st, const BwdParams& p, int batch) {
+    hipLaunchKernelGGL(bwd_dkdv_reduce_kernel, dim3(p.k_blocks, batch, p.num_heads_k), dim3(256), 0, st, p);
+    IV2_LAUNCH_CHECK();
+    return 0;
 }
 
 int launch_bwd_dkdv_wave(hipStream_t st, const BwdParams& p, int batch, int max_seqlen_q, bool causal) {

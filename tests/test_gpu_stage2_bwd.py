@@ -102,3 +102,29 @@ def test_forward_and_dq_are_bit_reproducible(ops):
         assert torch.equal(runs[0][0], other[0]) and torch.equal(runs[0][1], other[1])
         for a, b in ((runs[0][2], other[2]), (runs[0][3], other[3])):
             assert float((a.float() - b.float()).abs().max()) <= 2.0 ** -7 * float(a.float().abs().max())
+
+
+@pytest.mark.parametrize("sq,sk,k_sel,causal,sparse", [([1500, 700], [1500, 700], 6, True, True),
+                                                        ([300], [300], 2, True, False), ([2100], [2100], 40, True, True)])
+def test_deterministic_mode(ops, sq, sk, k_sel, causal, sparse):
+    """deterministic=True: dK and dV come from per-work-item slots added in a fixed order instead of fp32 atomics:
+    bitwise equal between runs, and equal to the oracle to the usual tolerance."""
+    dev = torch.device("cuda:0")
+    q, k, v, cu_q, cu_k, idx = make_case(9, sq, sk, 2, k_sel, dev)
+    dout = torch.randn(q.shape, generator=torch.Generator(device="cpu").manual_seed(10)).to(torch.bfloat16).to(dev)
+    grads = []
+    for _ in range(3):
+        qg, kg, vg = [t.clone().requires_grad_(True) for t in (q, k, v)]
+        out = ops.infllmv2_attn_varlen_func(qg, kg, vg, cu_q, cu_k, max(sq), max(sk), causal=causal,
+                                            topk_idx=idx if sparse else None, deterministic=True)
+        out.backward(dout)
+        grads.append((qg.grad, kg.grad, vg.grad))
+    for other in grads[1:]:
+        for a, b in zip(grads[0], other):
+            assert torch.equal(a, b)
+    words = O.topk_to_uint64(idx.cpu().numpy(), max(sk), 64)[0] if sparse else None
+    dq, dk, dv = O.stage2_backward(bf16_np(q), bf16_np(k), bf16_np(v), bf16_np(dout), cu_q.cpu().numpy(),
+                                   cu_k.cpu().numpy(), words, 128 ** -0.5, causal)
+    check_grad("dq", grads[0][0], dq)
+    check_grad("dk", grads[0][1], dk)
+    check_grad("dv", grads[0][2], dv)
