@@ -148,6 +148,7 @@ class Infllmv2AttnVarlenFunc(torch.autograd.Function):
         ctx.causal = causal
         ctx.deterministic = deterministic
         ctx.sparse = topk_idx is not None
+        ctx.max_selected = topk_idx.shape[-1] if topk_idx is not None else 0     # a mask row has at most k set bits
         if not return_softmax:
             return out
         # S_dmask is only materialised with dropout, which this build rejects
@@ -162,7 +163,7 @@ class Infllmv2AttnVarlenFunc(torch.autograd.Function):
         q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, fwd_mask = ctx.saved_tensors
         dq, dk, dv = sparse_backward(dout, q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, ctx.max_seqlen_q,
                                      ctx.max_seqlen_k, ctx.softmax_scale, ctx.causal, fwd_mask, ctx.sparse,
-                                     ctx.deterministic)
+                                     ctx.deterministic, ctx.max_selected)
         return (dq, dk, dv) + (None,) * 14
 
 

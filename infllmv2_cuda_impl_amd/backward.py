@@ -8,6 +8,8 @@ transposed by a single kernel inside it.
 """
 from __future__ import annotations
 
+import os
+
 import torch
 
 from . import _lib
@@ -15,6 +17,7 @@ from ._util import ptr, stream_ptr
 
 GROUP = 16
 HAVE_BACKWARD = True
+HANDOFF_MAX_BYTES = 64 << 30          # above this much dS scratch the backward recomputes S and dP in the dQ kernel
 
 
 def _nat(t):
@@ -22,9 +25,11 @@ def _nat(t):
 
 
 def sparse_backward(dout, q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, softmax_scale,
-                    causal, fwd_mask, lse_expanded: bool, deterministic: bool = False):
+                    causal, fwd_mask, lse_expanded: bool, deterministic: bool = False, max_selected: int = 0):
     """Returns (dq, dk, dv) with the shapes and dtype of (q, k, v).  dq is always bit-reproducible; with
-    ``deterministic`` dk and dv are too (slots + ordered sum instead of fp32 atomics, at the price of a large workspace)."""
+    ``deterministic`` dk and dv are too (slots + ordered sum instead of fp32 atomics, at the price of a large workspace).
+    ``max_selected`` > 0 (an upper bound of the set bits per mask row) lets the dK/dV kernel hand its dS tiles to the dQ
+    kernel (2 KiB of workspace per token, KV head and selectable block); INFLLMV2_BWD_HANDOFF=0 switches that off."""
     if dout.stride(-1) != 1:
         dout = dout.contiguous()
     if dout.dtype != q.dtype or tuple(dout.shape) != tuple(q.shape):
@@ -37,11 +42,13 @@ def sparse_backward(dout, q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, max_seq
         lse_strides = _lib.i64_array([GROUP, 1, total_q * GROUP])
     else:
         lse_strides = _lib.i64_array([1, total_q, GROUP * total_q])
-    size_query = (_lib.lib.infllmv2_varlen_bwd_deterministic_workspace_bytes if deterministic
-                  else _lib.lib.infllmv2_varlen_bwd_workspace_bytes)
-    ws_bytes = size_query(batch, total_q, total_k, Hk, max_seqlen_k)
-    workspace = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=q.device)
     n64 = 0 if fwd_mask is None else fwd_mask.shape[-1]
+    if fwd_mask is None or os.environ.get("INFLLMV2_BWD_HANDOFF", "1") == "0" or \
+            Hk * total_q * (max_selected + 1) * 2048 > HANDOFF_MAX_BYTES:
+        max_selected = 0
+    ws_bytes = _lib.lib.infllmv2_varlen_bwd_workspace_bytes_ex(batch, total_q, total_k, Hk, max_seqlen_k,
+                                                              int(bool(deterministic)), int(max_selected), n64)
+    workspace = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=q.device)
     kv = lambda t: _lib.i64_array([t.stride(0), t.stride(1)])
     with torch.cuda.device(q.device):
         _lib.call("infllmv2_varlen_bwd", stream_ptr(q.device), dout.data_ptr(), q.data_ptr(), k.data_ptr(),
@@ -49,5 +56,5 @@ def sparse_backward(dout, q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, max_seq
                   cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), ptr(fwd_mask), workspace.data_ptr(),
                   workspace.numel(), batch, total_q, total_k, Hq, Hk, d, max_seqlen_q, max_seqlen_k,
                   _nat(q), kv(k), kv(v), _nat(out), _nat(dout), _nat(dq), kv(dk), kv(dv), lse_strides, n64,
-                  float(softmax_scale), int(bool(causal)), int(bool(deterministic)))
+                  float(softmax_scale), int(bool(causal)), int(bool(deterministic)), int(max_selected))
     return dq, dk, dv

@@ -32,7 +32,7 @@ constexpr int kColSlice = kDkdvSlice;                          // query tokens p
 constexpr int kGroupSlices = 4;                                // slices that pool their light members
 constexpr int kGroupWords = kGroupSlices * kColSlice / 64;     // = 32: one mask word per lane of the lower half
 constexpr int kHeavyPairs = 128;                               // a slice with fewer selected tokens is "light"
-constexpr int kStage = 16384 + 512;                            // q a|b, dout a|b (4 KiB each) + the pair's 64 row scalars
+constexpr int kStage = 16384 + 512 + 512;                      // q a|b, dout a|b (4 KiB each), the pair's 64 row scalars, its two rank records
 constexpr int kWaveLds = 2 * kStage;                           // = 64 rows x 132 floats: also the flush tile
 constexpr int kFlushPitch = 132;                               // floats per key row of the flush tile
 
@@ -213,6 +213,10 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
     const bf16_bits* q_head = p.q + static_cast<int64_t>(h) * p.q_kvh;
     const bf16_bits* do_head = p.dout + static_cast<int64_t>(h) * p.do_kvh;
     const float* stat_head = p.rowstat + static_cast<int64_t>(h) * p.total_q * 32;
+    const bool handoff = p.ds_buf != nullptr;                  // uniform over the launch
+    const uint32_t rank_lane = static_cast<uint32_t>((lane & 3) * 4);
+    const uint4* rank_head = handoff ? p.rankinfo + static_cast<int64_t>(h) * p.total_q * p.n64_fwd + (j >> 6) : nullptr;
+    const uint64_t below_j = (1ull << (j & 63)) - 1ull;        // the mask bits of the blocks before j in its word
     auto issue = [&](int64_t ta, int64_t tb, int stage) {
         const uint32_t st = ring_lds + stage * kStage;
         const bf16_bits* qa = q_head + ta * p.q_tok;
@@ -230,6 +234,11 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
         // token a's [lse * log2e (16) | D (16)] (both half-wavefronts fetch the same 128 bytes), then token b's
         dma4(stat_head + ta * 32, stat_lane, st + 16384);
         dma4(stat_head + tb * 32, stat_lane, st + 16384 + 256);
+        if (handoff) {
+            // the 16-byte rank record of (token, mask word of block j), replicated over the 256-byte region
+            dma4(rank_head + ta * p.n64_fwd, rank_lane, st + 16896);
+            dma4(rank_head + tb * p.n64_fwd, rank_lane, st + 16896 + 256);
+        }
     };
 
     // Every ordinary load issued so far must have landed before the first LDS-DMA goes out: the compiler would
@@ -255,16 +264,22 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
     bool more = next_pair(ta, tb, has_b);
     if (more) issue(ta, tb, 0);
     int stage = 0;
+    bool first_turn = true;
     while (more) {
         int64_t na, nb2;
         bool nhb;
         const bool have_next = next_pair(na, nb2, nhb);
         if (have_next) {
             issue(na, nb2, stage ^ 1);                         // the other stage was consumed by the previous turn
-            __builtin_amdgcn_s_waitcnt(0x4F72);                // vmcnt(18): this turn's 18 loads have landed
+            // this turn's loads have landed when only the younger operations are still in flight: the next pair's 18
+            // loads, or with the hand-off its 20 loads and the previous turn's 8 tile stores
+            if (!handoff) __builtin_amdgcn_s_waitcnt(0x4F72);                  // vmcnt(18)
+            else if (first_turn) __builtin_amdgcn_s_waitcnt(0x4F74);           // vmcnt(20)
+            else __builtin_amdgcn_s_waitcnt(0x4F7C);                           // vmcnt(28)
         } else {
             __builtin_amdgcn_s_waitcnt(0x0F70);
         }
+        first_turn = false;
         const unsigned char* st = ring + stage * kStage;
 
         int lim_a, lim_b;                                      // in-block key index limit (inclusive)
@@ -288,6 +303,25 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
         const float lse_a[4] = {la.x, la.y, la.z, la.w};
         const float lse_b[4] = {lb.x, lb.y, lb.z, lb.w};
         const bool edge = (lim_a < kBlockN - 1) || (lim_b < kBlockN - 1);
+        // hand-off: where the dS^T tiles of this pair go (rank of block j among the set bits of each token's mask row)
+        bf16_bits* ds_a = nullptr;
+        bf16_bits* ds_b = nullptr;
+        if (handoff) {
+            const uint4 ra = *reinterpret_cast<const uint4*>(st + 16896);
+            const uint4 rb = *reinterpret_cast<const uint4*>(st + 16896 + 256);
+            const uint32_t alo = __builtin_amdgcn_readfirstlane(ra.x), ahi = __builtin_amdgcn_readfirstlane(ra.y);
+            const uint32_t blo = __builtin_amdgcn_readfirstlane(rb.x), bhi = __builtin_amdgcn_readfirstlane(rb.y);
+            int rank_a = static_cast<int>(__builtin_amdgcn_readfirstlane(ra.z)) +
+                         __builtin_popcountll(((static_cast<uint64_t>(ahi) << 32) | alo) & below_j);
+            int rank_b = static_cast<int>(__builtin_amdgcn_readfirstlane(rb.z)) +
+                         __builtin_popcountll(((static_cast<uint64_t>(bhi) << 32) | blo) & below_j);
+            // a row with more set bits than announced, or the absent second token, writes to the row's spare slot
+            if (rank_a > p.max_sel) rank_a = p.max_sel;
+            if (rank_b > p.max_sel || !has_b) rank_b = p.max_sel;
+            const int64_t row_tiles = p.max_sel + 1;
+            ds_a = p.ds_buf + ((static_cast<int64_t>(h) * p.total_q + ta) * row_tiles + rank_a) * (kBlockN * 16);
+            ds_b = p.ds_buf + ((static_cast<int64_t>(h) * p.total_q + tb) * row_tiles + rank_b) * (kBlockN * 16);
+        }
 
         // Four phases, each 32 MFMAs, with the VALU work of the softmax backward hidden behind the matrix pipeline:
         //   A  S = Q K^T                       (both tokens, all 64 keys; every fragment read from LDS feeds 4 MFMAs)
@@ -387,6 +421,19 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        if (handoff) {
+            // dS^T tiles [key][head]: lane (key n of tile kt, heads 4g..4g+3) holds 8 bytes per token; always 8 stores
+#pragma unroll
+            for (int kt = 0; kt < 4; ++kt) {
+                uint4 raw;
+                __builtin_memcpy(&raw, &dsfr[kt], 16);
+                const int at = kt * 256 + n * 16 + 4 * g;         // the tile bases are wave-uniform: scalar base + lane offset
+                // streaming stores: the tiles are read much later, by another kernel, and should not push q / dout out of L2
+                typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+                __builtin_nontemporal_store(u32x2{raw.x, raw.y}, reinterpret_cast<u32x2*>(ds_a + at));
+                __builtin_nontemporal_store(u32x2{raw.z, raw.w}, reinterpret_cast<u32x2*>(ds_b + at));
             }
         }
         {   // D: transposed reads of the q tiles

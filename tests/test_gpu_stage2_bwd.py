@@ -128,3 +128,30 @@ def test_deterministic_mode(ops, sq, sk, k_sel, causal, sparse):
     check_grad("dq", grads[0][0], dq)
     check_grad("dk", grads[0][1], dk)
     check_grad("dv", grads[0][2], dv)
+
+
+@pytest.mark.parametrize("handoff", ["1", "0"])
+@pytest.mark.parametrize("sq,sk,k_sel", [([300], [4500], 12), ([1500, 700], [1500, 700], 6), ([130], [130], 3)])
+def test_ds_handoff_and_recompute_agree_with_oracle(ops, monkeypatch, handoff, sq, sk, k_sel):
+    """With a top-k mask the dK/dV kernel hands its dS tiles to the dQ kernel (slot = rank of the block in the token's
+    mask row; [300] x [4500] has rows of two 64-bit words, so ranks continue across a word boundary);
+    INFLLMV2_BWD_HANDOFF=0 keeps the dQ kernel that recomputes S and dP.  Both must meet the oracle."""
+    monkeypatch.setenv("INFLLMV2_BWD_HANDOFF", handoff)
+    run_case(ops, sq, sk, 2, k_sel, True, seed=21)
+
+
+def test_ds_handoff_with_duplicate_and_missing_indices(ops):
+    """Rows with fewer set bits than the announced bound (-1 entries and repeated blocks) leave slots unused."""
+    dev = torch.device("cuda:0")
+    q, k, v, cu_q, cu_k, idx = make_case(23, [700], [700], 2, 5, dev)
+    idx[:, ::3, 1] = idx[:, ::3, 0]
+    idx[:, 1::3, 3:] = -1
+    dout = torch.randn(q.shape, generator=torch.Generator(device="cpu").manual_seed(24)).to(torch.bfloat16).to(dev)
+    qg, kg, vg = [t.clone().requires_grad_(True) for t in (q, k, v)]
+    ops.infllmv2_attn_varlen_func(qg, kg, vg, cu_q, cu_k, 700, 700, causal=True, topk_idx=idx).backward(dout)
+    words = O.topk_to_uint64(idx.cpu().numpy(), 700, 64)[0]
+    dq, dk, dv = O.stage2_backward(bf16_np(q), bf16_np(k), bf16_np(v), bf16_np(dout), cu_q.cpu().numpy(),
+                                   cu_k.cpu().numpy(), words, 128 ** -0.5, True)
+    check_grad("dq", qg.grad, dq)
+    check_grad("dk", kg.grad, dk)
+    check_grad("dv", vg.grad, dv)
