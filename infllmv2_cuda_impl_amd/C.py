@@ -55,14 +55,6 @@ def get_probs(*args, **kwargs):
     raise NotImplementedError("get_probs is bound by the reference but unused by its package; not built here")
 
 
-def fwd(*args, **kwargs):
-    raise NotImplementedError("fixed-length dense attention (mha_fwd) is not reachable from the infllm_v2 API; not built")
-
-
-def bwd(*args, **kwargs):
-    raise NotImplementedError("fixed-length dense attention (mha_bwd) is not reachable from the infllm_v2 API; not built")
-
-
 # ---- tensor group ---------------------------------------------------------------------------------
 def _layout(t, expanded: bool):
     """{token, head-in-group, kv-head} strides and (total_q, Hq, Hk) of a q-like tensor."""
@@ -229,3 +221,80 @@ def fwd_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_,
         out_.copy_(out)
         out = out_
     return [out, lse]
+
+
+# ---- fixed-length batches: the packed entries with equal sequence lengths -----------------------------
+def _packed(t, name):
+    """(b, s, h, d) -> (b * s, h, d) sharing memory when the batch rows follow one another, else a copy."""
+    if t.dim() != 4:
+        raise RuntimeError(f"{name} must have shape (batch_size, seqlen, num_heads, head_size)")
+    return t.reshape(t.shape[0] * t.shape[1], t.shape[2], t.shape[3])
+
+
+def _cu(batch, seqlen, device):
+    return torch.arange(batch + 1, dtype=torch.int32, device=device) * seqlen
+
+
+def fwd(q, k, v, out_, alibi_slopes_, p_dropout, softmax_scale, is_causal, window_size_left, window_size_right,
+        softcap, return_softmax, gen_=None):
+    """mha_fwd (flash_api.cpp:349-517): dense attention over a fixed-length batch, q ``(b, sq, Hq, d)``, k/v
+    ``(b, sk, Hk, d)``.  Runs the packed kernels with equal sequence lengths.  Returns
+    ``[out, softmax_lse (b, Hq, sq) fp32, p, rng_state]``."""
+    b, sq, Hq, d = q.shape
+    sk = k.shape[1]
+    if k.shape[0] != b or v.shape != k.shape:
+        raise RuntimeError("k and v must have shape (batch_size, seqlen_k, num_heads_k, head_size)")
+    if out_ is not None and tuple(out_.shape) != tuple(q.shape):
+        raise RuntimeError("out must have the shape of q")
+    out2 = None
+    if out_ is not None:
+        out2 = _packed(out_, "out")
+        if out2.data_ptr() != out_.data_ptr() or out_.stride(0) != sq * out_.stride(1):
+            out2 = None                                     # not viewable as packed rows: copy at the end
+    res = varlen_fwd(_packed(q, "q"), _packed(k, "k"), _packed(v, "v"), out2, _cu(b, sq, q.device), _cu(b, sk, q.device),
+                     None, None, None, alibi_slopes_, sq, sk, p_dropout, softmax_scale, False, is_causal,
+                     window_size_left, window_size_right, softcap, return_softmax, gen_)
+    out = res[0].view(b, sq, Hq, d)
+    if out_ is not None:
+        if out2 is None:
+            out_.copy_(out)
+        out = out_
+    lse = res[1].view(Hq, b, sq).permute(1, 0, 2).contiguous()
+    return [out, lse, res[2], res[3]]
+
+
+def bwd(dout, q, k, v, out, softmax_lse, dq_, dk_, dv_, alibi_slopes_, p_dropout, softmax_scale, is_causal,
+        window_size_left, window_size_right, softcap, deterministic, gen_=None, rng_state=None):
+    """mha_bwd (flash_api.cpp:1062-1276): gradients of ``fwd``; softmax_lse ``(b, Hq, sq)``.  dq_, dk_, dv_ are
+    filled in place when given.  Returns ``[dq, dk, dv, softmax_d]`` (softmax_d empty: D never leaves the
+    workspace)."""
+    b, sq, Hq, d = q.shape
+    sk = k.shape[1]
+    if tuple(softmax_lse.shape) != (b, Hq, sq):
+        raise RuntimeError("softmax_lse must have shape (batch_size, num_heads, seqlen_q)")
+    lse = softmax_lse.permute(1, 0, 2).reshape(Hq, b * sq).contiguous()
+    given = (dq_, dk_, dv_)
+    like = (q, k, v)
+    packed = []
+    for g, l in zip(given, like):
+        if g is not None and tuple(g.shape) != tuple(l.shape):
+            raise RuntimeError("dq, dk, dv must have the shapes of q, k, v")
+        p2 = None
+        if g is not None and g.stride(-1) == 1:
+            p2 = _packed(g, "gradient")
+            if p2.data_ptr() != g.data_ptr() or g.stride(0) != g.shape[1] * g.stride(1):
+                p2 = None
+        packed.append(p2)
+    res = varlen_bwd(_packed(dout, "dout"), _packed(q, "q"), _packed(k, "k"), _packed(v, "v"), _packed(out, "out"), lse,
+                     packed[0], packed[1], packed[2], _cu(b, sq, q.device), _cu(b, sk, q.device), alibi_slopes_, sq, sk,
+                     p_dropout, softmax_scale, False, is_causal, window_size_left, window_size_right, softcap,
+                     deterministic, None, gen_, rng_state)
+    grads = []
+    for r, g, l, p2 in zip(res[:3], given, like, packed):
+        r = r.view(l.shape)
+        if g is not None:
+            if p2 is None:
+                g.copy_(r)
+            r = g
+        grads.append(r)
+    return grads + [res[3]]

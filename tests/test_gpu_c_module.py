@@ -93,4 +93,41 @@ def test_reference_style_stage1_and_pooling_through_C():
     assert torch.equal(pos[:, :10], ref_idx)
     assert torch.equal(val[:, :10], torch.gather(pooled.reshape(2 * S, out_len), 1, ref_idx.long()))
     with pytest.raises(NotImplementedError):
-        C.fwd()
+        C.get_probs()
+
+
+@pytest.mark.parametrize("causal", [True, False])
+def test_fixed_length_fwd_bwd_through_C(causal):
+    """`C.fwd` / `C.bwd` (mha_fwd / mha_bwd, flash_api.cpp:349-517, 1062-1276): dense attention over a
+    (batch, seqlen, heads, d) batch.  Checked against the fp64 oracle per sequence; gradients land in the
+    caller's tensors, also when those are not viewable as packed rows."""
+    from infllm_v2 import C
+    from oracle import infllmv2_oracle as O
+    from conftest import bf16_np
+    dev = torch.device("cuda:0")
+    b, sq, sk, Hk = 3, 70, 130, 2
+    g = torch.Generator(device="cpu").manual_seed(31)
+    mk = lambda *shape: torch.randn(*shape, generator=g).to(torch.bfloat16).to(dev)
+    q, k, v, dout = mk(b, sq, 16 * Hk, 128), mk(b, sk, Hk, 128), mk(b, sk, Hk, 128), mk(b, sq, 16 * Hk, 128)
+    out, lse, _, _ = C.fwd(q, k, v, None, None, 0.0, 128 ** -0.5, causal, -1, -1, 0.0, False, None)
+    assert out.shape == q.shape and lse.shape == (b, 16 * Hk, sq) and lse.dtype == torch.float32
+    dq = torch.empty_like(q)
+    dk_wide = torch.zeros(b, sk, Hk, 256, dtype=torch.bfloat16, device=dev)
+    dk = dk_wide[..., :128]                                     # last-dim contiguous, rows twice as far apart
+    dv_t = torch.empty(sk, b, Hk, 128, dtype=torch.bfloat16, device=dev).transpose(0, 1)    # not packable: copied back
+    r = C.bwd(dout, q, k, v, out, lse, dq, dk, dv_t, None, 0.0, 128 ** -0.5, causal, -1, -1, 0.0, False, None, None)
+    assert r[0] is dq and r[1] is dk and r[2] is dv_t
+    cu_q = np.arange(b + 1, dtype=np.int32) * sq
+    cu_k = np.arange(b + 1, dtype=np.int32) * sk
+    flat = lambda t: bf16_np(t.reshape(-1, t.shape[2], t.shape[3]))
+    ref_o, ref_lse = O.stage2_forward(flat(q), flat(k), flat(v), cu_q, cu_k, None, 128 ** -0.5, causal)
+    assert np.abs(bf16_np(out).reshape(ref_o.shape).astype(np.float64) - ref_o).max() <= 2e-2
+    got_lse = lse.permute(1, 0, 2).reshape(16 * Hk, b * sq).cpu().numpy()
+    ref_heads = ref_lse.reshape(Hk, b * sq, 16).transpose(0, 2, 1).reshape(16 * Hk, b * sq)     # column t*16+g -> row 16h+g
+    assert np.abs(got_lse - ref_heads).max() <= 1e-3
+    rq, rk, rv = O.stage2_backward(flat(q), flat(k), flat(v), flat(dout), cu_q, cu_k, None, 128 ** -0.5, causal)
+    for name, got, ref in (("dq", dq, rq), ("dk", dk, rk), ("dv", dv_t, rv)):
+        gnp = bf16_np(got.contiguous()).reshape(ref.shape).astype(np.float64)
+        s = max(1.0, float(np.abs(ref).max()))
+        err = np.abs(gnp - ref)
+        assert err.max() <= 2e-2 * s and err.mean() <= 1e-3 * s, (name, err.max(), err.mean())
