@@ -45,13 +45,16 @@ __device__ __forceinline__ uint32_t lds_addr(const void* ptr) {
 // LDS-DMA: lane l's 16 (4) bytes at base (scalar) + its own byte offset land at lds_base + 16 l (4 l).  The
 // compiler's wait-count tracking does not see these loads; they are ordered by hand with s_waitcnt vmcnt(n).
 // The instruction's immediate offset moves the global source AND the LDS destination, hence the subtraction.
-template <int kOffset>
+// kLds is added to the scalar LDS base inside the asm (one SALU instruction writes M0).
+template <int kOffset, int kLds>
 __device__ __forceinline__ void dma16(const void* base, uint32_t lane_off, uint32_t lds_base) {
-    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1 offset:%3"
-                 : : "v"(lane_off), "s"(base), "s"(lds_base - kOffset), "n"(kOffset) : "memory", "m0");
+    asm volatile("s_add_i32 m0, %2, %4\n\tglobal_load_lds_dwordx4 %0, %1 offset:%3"
+                 : : "v"(lane_off), "s"(base), "s"(lds_base), "n"(kOffset), "n"(kLds - kOffset) : "memory", "m0", "scc");
 }
+template <int kLds>
 __device__ __forceinline__ void dma4(const void* base, uint32_t lane_off, uint32_t lds_base) {
-    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %0, %1" : : "v"(lane_off), "s"(base), "s"(lds_base) : "memory", "m0");
+    asm volatile("s_add_i32 m0, %2, %3\n\tglobal_load_lds_dword %0, %1"
+                 : : "v"(lane_off), "s"(base), "s"(lds_base), "n"(kLds) : "memory", "m0", "scc");
 }
 // One d tile of one of the second GEMMs: acc[kt] += a * b[kt] for the four key tiles, accumulators in AGPRs.
 // Written as one asm block because the compiler cannot see that these are MFMAs: an MFMA must not read a VGPR in
@@ -217,27 +220,36 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
     const uint32_t rank_lane = static_cast<uint32_t>((lane & 3) * 4);
     const uint4* rank_head = handoff ? p.rankinfo + static_cast<int64_t>(h) * p.total_q * p.n64_fwd + (j >> 6) : nullptr;
     const uint64_t below_j = (1ull << (j & 63)) - 1ull;        // the mask bits of the blocks before j in its word
+    // byte strides per token as 32-bit scalars (checked by the launcher): a token's address is one 32 x 32 -> 64 bit
+    // multiplication away
+    const uint32_t q_tok_bytes = static_cast<uint32_t>(p.q_tok * 2), do_tok_bytes = static_cast<uint32_t>(p.do_tok * 2);
+    const uint32_t rank_tok_bytes = static_cast<uint32_t>(p.n64_fwd) * 16u;
+    const unsigned char* q_bytes = reinterpret_cast<const unsigned char*>(q_head);
+    const unsigned char* do_bytes = reinterpret_cast<const unsigned char*>(do_head);
+    const unsigned char* stat_bytes = reinterpret_cast<const unsigned char*>(stat_head);
+    const unsigned char* rank_bytes = reinterpret_cast<const unsigned char*>(rank_head);
     auto issue = [&](int64_t ta, int64_t tb, int stage) {
         const uint32_t st = ring_lds + stage * kStage;
-        const bf16_bits* qa = q_head + ta * p.q_tok;
-        const bf16_bits* qb = q_head + tb * p.q_tok;
-        const bf16_bits* da = do_head + ta * p.do_tok;
-        const bf16_bits* db = do_head + tb * p.do_tok;
-        dma16<0>(qa, q_lane, st);           dma16<64>(qa, q_lane, st + 1024);
-        dma16<128>(qa, q_lane, st + 2048);  dma16<192>(qa, q_lane, st + 3072);
-        dma16<0>(qb, q_lane, st + 4096);    dma16<64>(qb, q_lane, st + 5120);
-        dma16<128>(qb, q_lane, st + 6144);  dma16<192>(qb, q_lane, st + 7168);
-        dma16<0>(da, do_lane, st + 8192);   dma16<64>(da, do_lane, st + 9216);
-        dma16<128>(da, do_lane, st + 10240); dma16<192>(da, do_lane, st + 11264);
-        dma16<0>(db, do_lane, st + 12288);  dma16<64>(db, do_lane, st + 13312);
-        dma16<128>(db, do_lane, st + 14336); dma16<192>(db, do_lane, st + 15360);
+        const uint64_t ua = static_cast<uint32_t>(ta), ub = static_cast<uint32_t>(tb);     // packed token indices fit 31 bits
+        const unsigned char* qa = q_bytes + ua * q_tok_bytes;
+        const unsigned char* qb = q_bytes + ub * q_tok_bytes;
+        const unsigned char* da = do_bytes + ua * do_tok_bytes;
+        const unsigned char* db = do_bytes + ub * do_tok_bytes;
+        dma16<0, 0>(qa, q_lane, st);        dma16<64, 1024>(qa, q_lane, st);
+        dma16<128, 2048>(qa, q_lane, st);   dma16<192, 3072>(qa, q_lane, st);
+        dma16<0, 4096>(qb, q_lane, st);     dma16<64, 5120>(qb, q_lane, st);
+        dma16<128, 6144>(qb, q_lane, st);   dma16<192, 7168>(qb, q_lane, st);
+        dma16<0, 8192>(da, do_lane, st);    dma16<64, 9216>(da, do_lane, st);
+        dma16<128, 10240>(da, do_lane, st); dma16<192, 11264>(da, do_lane, st);
+        dma16<0, 12288>(db, do_lane, st);   dma16<64, 13312>(db, do_lane, st);
+        dma16<128, 14336>(db, do_lane, st); dma16<192, 15360>(db, do_lane, st);
         // token a's [lse * log2e (16) | D (16)] (both half-wavefronts fetch the same 128 bytes), then token b's
-        dma4(stat_head + ta * 32, stat_lane, st + 16384);
-        dma4(stat_head + tb * 32, stat_lane, st + 16384 + 256);
+        dma4<16384>(stat_bytes + (ua << 7), stat_lane, st);
+        dma4<16384 + 256>(stat_bytes + (ub << 7), stat_lane, st);
         if (handoff) {
             // the 16-byte rank record of (token, mask word of block j), replicated over the 256-byte region
-            dma4(rank_head + ta * p.n64_fwd, rank_lane, st + 16896);
-            dma4(rank_head + tb * p.n64_fwd, rank_lane, st + 16896 + 256);
+            dma4<16896>(rank_bytes + ua * rank_tok_bytes, rank_lane, st);
+            dma4<16896 + 256>(rank_bytes + ub * rank_tok_bytes, rank_lane, st);
         }
     };
 
@@ -543,6 +555,8 @@ int launch_bwd_dkdv_wave(hipStream_t st, const BwdParams& p, int batch, int max_
     const int n_slices8 = (n_slices + 8 * kGroupSlices - 1) / (8 * kGroupSlices) * (8 * kGroupSlices);
     const int64_t items = static_cast<int64_t>(n_slices8) * p.k_blocks;
     IV2_CHECK(items <= 0x7fffffffll, "varlen_bwd: too many (slice, block) work items");
+    IV2_CHECK(p.q_tok >= 0 && p.q_tok < (1ll << 31) && p.do_tok >= 0 && p.do_tok < (1ll << 31) && p.total_q < (1ll << 31),
+              "varlen_bwd: token strides of q and dout must lie in [0, 2^31) elements");
     const dim3 grid(static_cast<unsigned>(items), batch, p.num_heads_k);
     const size_t lds = kWaveLds + kGroupWords * 8;
     if (causal) hipLaunchKernelGGL(bwd_dkdv_wave_kernel<true>, grid, dim3(64), lds, st, p);
