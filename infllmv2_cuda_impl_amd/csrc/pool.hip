@@ -8,9 +8,11 @@
 // The maximum is taken with the reference's sequential ">" scan so NaN and signed-zero inputs
 // pick the same element.  Values are copied, never re-rounded, so the result is bit-exact.
 //
-// The kernel is HBM-bound: one workgroup per (query row, head) streams the row once.  When the
-// pooling window is the shipped 5/4/1 and rows are 8-byte aligned a lane fetches its four
-// in-window scores with one 8-byte load.
+// The kernel is HBM-bound.  Score rows are rarely aligned (2047 columns at 32768 tokens), so a
+// wavefront copies a whole row into its own LDS slice with 16-byte loads from the aligned address
+// below the row (a 16-byte unit that holds one valid byte lies in the same page, so the few bytes
+// read before and after the row cannot fault), and every window is then read from LDS.  Rows too
+// long for LDS take the direct kernel, one workgroup per (query row, head).
 #include "common.h"
 #include "../../include/infllmv2_hip.h"
 
@@ -95,17 +97,100 @@ void max_pooling_1d_kernel(const PoolParams p) {
     }
 }
 
+// One wavefront per row at a time, kWaves wavefronts per workgroup, each with an LDS slice of `units` 16-byte units.
+template <int kWaves>
+__global__ __launch_bounds__(kWaves * 64)
+void max_pooling_1d_rows_kernel(const PoolParams p, int units, int rows_per_wave) {
+    extern __shared__ uint4 pool_lds[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    uint4* slice = pool_lds + wave * units;
+    const uint16_t* elems = reinterpret_cast<const uint16_t*>(slice);
+    const int64_t total_rows = static_cast<int64_t>(p.num_heads) * p.total_q;
+    const uint16_t pos_inf = p.is_bf16 ? 0x7f80 : 0x7c00;
+    const uint16_t neg_inf = p.is_bf16 ? 0xff80 : 0xfc00;
+    const int64_t first_row = (static_cast<int64_t>(blockIdx.x) * kWaves + wave) * rows_per_wave;
+    for (int r = 0; r < rows_per_wave; ++r) {
+        const int64_t row = first_row + r;
+        if (row >= total_rows) break;                           // uniform per wavefront; no workgroup barriers in this kernel
+        const int h = static_cast<int>(row / p.total_q);
+        const int q_global = static_cast<int>(row - static_cast<int64_t>(h) * p.total_q);
+        int q_local = q_global, seqlen_k = p.k_len, cache_len = p.cache_len;
+        if (p.cu_seqlens_q != nullptr) {
+            int lo = 0, hi = p.batch;                           // invariant: cu[lo] <= q_global < cu[hi]
+            while (hi - lo > 1) {
+                const int mid = (lo + hi) >> 1;
+                if (p.cu_seqlens_q[mid] <= q_global) lo = mid; else hi = mid;
+            }
+            q_local = q_global - p.cu_seqlens_q[lo];
+            seqlen_k = p.cu_seqlens_k[lo + 1] - p.cu_seqlens_k[lo];
+            seqlen_k = seqlen_k < p.k_len ? seqlen_k : p.k_len;
+            cache_len = p.cache_lens[lo];
+        }
+        const uint16_t* in = p.in + static_cast<int64_t>(h) * p.in_head_stride + static_cast<int64_t>(q_global) * p.in_row_stride;
+        const uintptr_t addr = reinterpret_cast<uintptr_t>(in);
+        const uint4* aligned = reinterpret_cast<const uint4*>(addr & ~static_cast<uintptr_t>(15));
+        const int shift = static_cast<int>(addr & 15) >> 1;     // the row starts at element `shift` of the slice
+        const int n_units = seqlen_k > 0 ? ((shift + seqlen_k) * 2 + 15) >> 4 : 0;
+        for (int u = lane; u < n_units; u += 64) slice[u] = aligned[u];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        uint16_t* out = p.out + (static_cast<int64_t>(h) * p.total_q + q_global) * p.out_len;
+        const int bq = (q_local + cache_len) / p.block_size;
+        for (int kb = lane; kb < p.out_len; kb += 64) {
+            const bool forced = (kb < p.init_blocks) || (bq >= kb && bq <= kb + p.local_blocks);
+            uint16_t best = neg_inf;
+            if (forced) {
+                best = pos_inf;
+            } else {
+                int start = kb * p.stride - p.padding;
+                int end = start + p.kernel_size;
+                start = start < 0 ? 0 : start;
+                end = end < seqlen_k ? end : seqlen_k;
+                if (end > start) {
+                    best = elems[shift + start];
+                    float best_f = elem_to_f32(best, p.is_bf16);
+                    for (int i = start + 1; i < end; ++i) {
+                        const uint16_t v = elems[shift + i];
+                        const float f = elem_to_f32(v, p.is_bf16);
+                        if (f > best_f) { best_f = f; best = v; }
+                    }
+                }
+            }
+            out[kb] = best;
+        }
+        // the slice is overwritten by the next row only after every lane has read this one
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    }
+}
+
 static int launch_pool(void* stream, PoolParams& p) {
     IV2_CHECK(p.num_heads >= 0 && p.total_q >= 0 && p.k_len >= 0 && p.out_len >= 0, "max_pooling_1d: negative size");
     IV2_CHECK(p.block_size > 0 && p.stride > 0 && p.kernel_size > 0, "max_pooling_1d: block_size, stride and kernel_size must be positive");
     IV2_CHECK(p.num_heads <= 65535, "max_pooling_1d: num_heads %d exceeds 65535", p.num_heads);
     if (p.num_heads == 0 || p.total_q == 0 || p.out_len == 0) return 0;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int units = (p.k_len * 2 + 14) / 16 + 2;              // a row plus the bytes before its first element
+    const size_t slice_bytes = static_cast<size_t>(units) * 16;
+    const int64_t total_rows = static_cast<int64_t>(p.num_heads) * p.total_q;
+    if (slice_bytes <= 36 * 1024) {
+        constexpr int kWaves = 4;
+        const int rows_per_wave = total_rows >= 64 * 1024 ? 4 : 1;
+        const int64_t blocks = (total_rows + kWaves * rows_per_wave - 1) / (kWaves * rows_per_wave);
+        IV2_CHECK(blocks <= 0x7fffffffll, "max_pooling_1d: too many rows");
+        hipLaunchKernelGGL(max_pooling_1d_rows_kernel<kWaves>, dim3(static_cast<unsigned>(blocks)), dim3(kWaves * 64),
+                           kWaves * slice_bytes, st, p, units, rows_per_wave);
+        IV2_LAUNCH_CHECK();
+        return 0;
+    }
     p.vec4 = p.kernel_size == 5 && p.stride == 4 && p.padding == 1 &&
              (p.in_row_stride % 4 == 0) && (p.in_head_stride % 4 == 0) &&
              (reinterpret_cast<uintptr_t>(p.in) % 8 == 0);
     const int threads = p.out_len >= 256 ? 256 : (p.out_len > 64 ? 128 : 64);
-    hipLaunchKernelGGL(max_pooling_1d_kernel, dim3(p.total_q, p.num_heads), dim3(threads), 0,
-                       static_cast<hipStream_t>(stream), p);
+    hipLaunchKernelGGL(max_pooling_1d_kernel, dim3(p.total_q, p.num_heads), dim3(threads), 0, st, p);
     IV2_LAUNCH_CHECK();
     return 0;
 }
