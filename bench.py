@@ -28,7 +28,7 @@ if ROOT not in sys.path:
 # HBM bytes per launch of the dominant kernel at the default workload: 2.00 x FETCH_SIZE + 1.00 x WRITE_SIZE of the two
 # rocprofv3 --pmc runs summarised in profiles/stage2_fwd_config2_hbm_traffic.md (counters cannot be read from inside
 # this process); null for any other workload
-MEASURED_FWD_TRAFFIC_BYTES = 5.68e9
+MEASURED_FWD_TRAFFIC_BYTES = 5.66e9
 PEAK_BF16_TFLOPS = 2500.0      # MI355X dense bf16 MFMA peak (vendor figure, no sparsity)
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E peak
 
