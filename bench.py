@@ -255,6 +255,17 @@ def main():
             peak_l1 = 256 * 64 * 2.4e9 / 1e12
             result["roofline"]["gather"] = {"bound": "l1", "bytes": gather_bytes, "achieved": gather_bytes / k_ms / 1e9,
                                             "peak": peak_l1, "unit": "TB/s", "frac": gather_bytes / k_ms / 1e9 / peak_l1}
+        if S % 64 == 0:
+            # the same operator when neighbouring tokens agree on their blocks (every token of a 64-token query block
+            # takes the selection of the block's first token): the i.i.d. scores of the synthetic input are the worst
+            # case for the row-parallel kernels, whose shared-block walk this leg shows
+            idx_shared = idx.view(2, S // 64, 64, topk)[:, :, :1].expand(2, S // 64, 64, topk).reshape(2, S, topk).contiguous()
+            sh_ms = event_ms(torch, lambda: ops.infllmv2_attn_varlen_func(q, k, v, cu_q, cu_q, S, S, causal=True,
+                                                                         topk_idx=idx_shared), 10)
+            sh_bits = ops.uint64_to_bool(ops.topk_to_uint64(idx_shared, S, 64)[0], nblk) & causal_blk[None]
+            sh_flops = 4 * 16 * 64 * 128 * int(sh_bits.sum())
+            result["stage2_fwd_block_shared_selection"] = {"ms": sh_ms, "tflops": sh_flops / sh_ms / 1e9,
+                                                           "frac_peak": sh_flops / sh_ms / 1e9 / PEAK_BF16_TFLOPS}
         try:
             from infllmv2_cuda_impl_amd.backward import HAVE_BACKWARD  # noqa: F401
             qg, kg, vg = [t.clone().requires_grad_(True) for t in (q, k, v)]
