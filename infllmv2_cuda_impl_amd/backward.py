@@ -46,9 +46,17 @@ def sparse_backward(dout, q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, max_seq
     if fwd_mask is None or os.environ.get("INFLLMV2_BWD_HANDOFF", "1") == "0" or \
             Hk * total_q * (max_selected + 1) * 2048 > HANDOFF_MAX_BYTES:
         max_selected = 0
-    ws_bytes = _lib.lib.infllmv2_varlen_bwd_workspace_bytes_ex(batch, total_q, total_k, Hk, max_seqlen_k,
-                                                              int(bool(deterministic)), int(max_selected), n64)
-    workspace = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=q.device)
+    def allocate(selected):
+        ws_bytes = _lib.lib.infllmv2_varlen_bwd_workspace_bytes_ex(batch, total_q, total_k, Hk, max_seqlen_k,
+                                                                  int(bool(deterministic)), int(selected), n64)
+        return torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=q.device)
+    try:
+        workspace = allocate(max_selected)
+    except torch.cuda.OutOfMemoryError:
+        if max_selected == 0:
+            raise
+        max_selected = 0                                      # no room for the dS tiles: recompute S and dP in the dQ kernel
+        workspace = allocate(0)
     kv = lambda t: _lib.i64_array([t.stride(0), t.stride(1)])
     with torch.cuda.device(q.device):
         _lib.call("infllmv2_varlen_bwd", stream_ptr(q.device), dout.data_ptr(), q.data_ptr(), k.data_ptr(),

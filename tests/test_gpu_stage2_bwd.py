@@ -155,3 +155,32 @@ def test_ds_handoff_with_duplicate_and_missing_indices(ops):
     check_grad("dq", qg.grad, dq)
     check_grad("dk", kg.grad, dk)
     check_grad("dv", vg.grad, dv)
+
+
+def test_ds_handoff_falls_back_when_its_workspace_does_not_fit(ops, monkeypatch):
+    """The dS tiles need (k + 1) * 2 KiB per token and KV head; when that allocation fails the backward takes the
+    dQ kernel that recomputes S and dP.  The failure is simulated on the host: the first workspace request of the
+    backward raises torch's out-of-memory error."""
+    dev = torch.device("cuda:0")
+    q, k, v, cu_q, cu_k, idx = make_case(31, [700], [700], 2, 5, dev)
+    dout = torch.randn(q.shape, generator=torch.Generator(device="cpu").manual_seed(32)).to(torch.bfloat16).to(dev)
+    qg, kg, vg = [t.clone().requires_grad_(True) for t in (q, k, v)]
+    out = ops.infllmv2_attn_varlen_func(qg, kg, vg, cu_q, cu_k, 700, 700, causal=True, topk_idx=idx)
+    real_empty, state = torch.empty, {"armed": True, "raised": 0}
+
+    def empty(*args, **kwargs):
+        if state["armed"] and kwargs.get("dtype") == torch.uint8:
+            state["armed"] = False
+            state["raised"] += 1
+            raise torch.cuda.OutOfMemoryError("simulated")
+        return real_empty(*args, **kwargs)
+    monkeypatch.setattr(torch, "empty", empty)
+    out.backward(dout)
+    monkeypatch.setattr(torch, "empty", real_empty)
+    assert state["raised"] == 1
+    words = O.topk_to_uint64(idx.cpu().numpy(), 700, 64)[0]
+    dq, dk, dv = O.stage2_backward(bf16_np(q), bf16_np(k), bf16_np(v), bf16_np(dout), cu_q.cpu().numpy(),
+                                   cu_k.cpu().numpy(), words, 128 ** -0.5, True)
+    check_grad("dq", qg.grad, dq)
+    check_grad("dk", kg.grad, dk)
+    check_grad("dv", vg.grad, dv)
