@@ -30,7 +30,7 @@ Pinning status (how each function is checked independently of its own formula, s
   cache_batch_idx, left padding) are gathers checked by relabelling invariance, rotary by
   complex multiplication, norm preservation, angle addition and the identity at angle 0.
 
-Unpinned here (stated in the tests that touch it): the tie order of the *external*
+Parity unpinned (stated in the tests that touch it): the tie order of the *external*
 ``torch.topk`` the reference's callers use (PyTorch leaves it unspecified); this
 build defines value-descending / index-ascending as csrc/topk.cuh:17,26,37 does.
 """
