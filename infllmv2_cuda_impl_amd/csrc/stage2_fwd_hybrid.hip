@@ -7,11 +7,12 @@
 //
 //   * the blocks that ALL 8 rows select (for InfLLM-V2 masks: the initial block and the local
 //     window, which neighbouring tokens share) are walked in lock step: every such block is
-//     copied once, by LDS-DMA, from its fragment-major image into a 3-deep LDS ring two blocks
-//     ahead, and each wavefront reads its MFMA operands with conflict-free ds_read_b128;
+//     copied once, by LDS-DMA, from its fragment-major image into a 4-tile LDS ring (two blocks in
+//     use, the next two in flight: one workgroup barrier per two blocks), and each wavefront
+//     reads its MFMA operands with conflict-free ds_read_b128;
 //   * the remaining blocks of a row are walked by its wavefront alone, operands straight from
 //     global memory into registers, as in stage2_fwd_kernel;
-//   * the two walks are interleaved, one common and one own block per turn: the first is bound by
+//   * the two walks are interleaved, common, own, common, own per turn: the first is bound by
 //     the matrix pipeline and the VALU, the second by the vector memory path.
 //
 // A per-token kernel is bound by what the vector memory path can deliver (32 KiB of operands per
@@ -31,7 +32,7 @@ namespace infllmv2 {
 
 constexpr int kHybTokens = 8;                                  // tokens (= wavefronts) per workgroup
 constexpr int kHybChunk = 16;                                  // token groups per XCD chunk
-constexpr int kRingTiles = 3;
+constexpr int kRingTiles = 4;
 constexpr int kTileBytes = 32768;                              // K image | V image of one block
 constexpr int kMaxMaskWords = 256;                             // LDS copies of the mask rows: up to 16384 key blocks
 
@@ -184,9 +185,9 @@ void stage2_fwd_hybrid_kernel(const FwdParams p, const HybridExtra x) {
 
     const int64_t slot0 = static_cast<int64_t>(h) * p.n_slots + image_slot0(p.cu_seqlens_k, b);
 
-    // ---- the walk: one turn = one common block (lock step, operands from the LDS ring) + one own block (operands
-    //      from global memory into registers).  The own blocks' loads keep the vector memory path busy while the
-    //      matrix pipeline works on the common block, and the other way round. ----
+    // ---- the walk: one turn = two common blocks (lock step, operands from the LDS ring) alternating with two own
+    //      blocks (operands from global memory into registers).  The own blocks' loads keep the vector memory path
+    //      busy while the matrix pipeline works on a common block, and the other way round. ----
     const uint4* src_lane = (wave < 4 ? reinterpret_cast<const uint4*>(p.kimg) + slot0 * 1024 + wave * 256
                                       : reinterpret_cast<const uint4*>(p.vimg) + slot0 * 1024 + (wave - 4) * 256) + lane;
     const uint32_t ring_base = __builtin_amdgcn_readfirstlane(lds_address_of(ring) + wave * 4096);
@@ -229,90 +230,96 @@ void stage2_fwd_hybrid_kernel(const FwdParams p, const HybridExtra x) {
     for (int c = 0; c < 4; ++c) asm volatile("" : "+v"(qf[c]));
 #pragma unroll
     for (int f = 0; f < 16; ++f) asm volatile("" : "+v"(kreg[f]));
-    int j0 = next_common();
-    int j1 = j0 >= 0 ? next_common() : -1;
-    if (j0 >= 0) issue(j0, 0);
-    if (j1 >= 0) issue(j1, 1);
-    int tile = 0;
-    bool k_ahead = false;                                      // the coming own block's 16 K-fragment loads were issued last turn
-    while (j0 >= 0 || jp >= 0) {
-        if (j0 >= 0) {                                         // uniform over the workgroup
-            // younger than this wavefront's 4 DMA loads of block j0: the 4 of j1 and last turn's 16 K loads
-            const int young = (j1 >= 0 ? 4 : 0) + (k_ahead ? 16 : 0);
-            switch (young) {
-                case 20: asm volatile("s_waitcnt vmcnt(20)" ::: "memory"); break;
-                case 16: asm volatile("s_waitcnt vmcnt(16)" ::: "memory"); break;
-                case 4:  asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
-                default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
-            }
-            __syncthreads();                                   // block j0 is in LDS for everyone; tile (tile + 2) % 3 is free
-            const int j2 = j1 >= 0 ? next_common() : -1;
-            if (j2 >= 0) issue(j2, tile >= 1 ? tile - 1 : 2);
-            if (live) {
-                // all 16 fragments of a tile are fetched before the MFMAs that use them (vreg is free between own
-                // blocks), and the MFMAs run over independent accumulators first
-                const uint4* kb = ring + tile * 2048 + lane;
-                const uint4* vb = kb + 1024;
+    // The common blocks go through the ring in pairs: tiles {0, 1} and {2, 3} alternate, the pair after the current
+    // one is in flight, and one workgroup barrier serves two blocks.
+    int c0 = next_common();
+    int c1 = c0 >= 0 ? next_common() : -1;
+    if (c0 >= 0) issue(c0, 0);
+    if (c1 >= 0) issue(c1, 1);
+    int half = 0;
+    bool k_ahead = false;                                      // the coming own block's 16 K-fragment loads were issued already
+    auto common_part = [&](int j0, int tile) {
+        // all 16 fragments of a tile are fetched before the MFMAs that use them (vreg is free between own
+        // blocks), and the MFMAs run over independent accumulators first
+        const uint4* kb = ring + tile * 2048 + lane;
+        const uint4* vb = kb + 1024;
 #pragma unroll
-                for (int f = 0; f < 16; ++f) {
-                    const uint4 raw = kb[f * 64];
-                    __builtin_memcpy(&vreg[f], &raw, 16);
-                }
-                floatx4 s[4];
-#pragma unroll
-                for (int kt = 0; kt < 4; ++kt) s[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int c = 0; c < 4; ++c)
-#pragma unroll
-                    for (int kt = 0; kt < 4; ++kt)
-                        s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg[kt * 4 + c], qf[c], s[kt], 0, 0, 0);
-#pragma unroll
-                for (int f = 0; f < 16; ++f) {
-                    const uint4 raw = vb[f * 64];
-                    __builtin_memcpy(&vreg[f], &raw, 16);
-                }
-                bf16x8 pf[2];
-                softmax_step(s, m, l, o, pf, (j0 == last_blk) ? last_key - j0 * kBlockN : kBlockN, g, p.scale_log2);
-#pragma unroll
-                for (int cc = 0; cc < 2; ++cc)
-#pragma unroll
-                    for (int dt = 0; dt < 8; ++dt)
-                        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg[dt * 2 + cc], pf[cc], o[dt], 0, 0, 0);
-            }
-            j0 = j1;
-            j1 = j2;
-            tile = tile == 2 ? 0 : tile + 1;
+        for (int f = 0; f < 16; ++f) {
+            const uint4 raw = kb[f * 64];
+            __builtin_memcpy(&vreg[f], &raw, 16);
         }
+        floatx4 s[4];
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt) s[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+#pragma unroll
+            for (int kt = 0; kt < 4; ++kt)
+                s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg[kt * 4 + c], qf[c], s[kt], 0, 0, 0);
+#pragma unroll
+        for (int f = 0; f < 16; ++f) {
+            const uint4 raw = vb[f * 64];
+            __builtin_memcpy(&vreg[f], &raw, 16);
+        }
+        bf16x8 pf[2];
+        softmax_step(s, m, l, o, pf, (j0 == last_blk) ? last_key - j0 * kBlockN : kBlockN, g, p.scale_log2);
+#pragma unroll
+        for (int cc = 0; cc < 2; ++cc)
+#pragma unroll
+            for (int dt = 0; dt < 8; ++dt)
+                o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg[dt * 2 + cc], pf[cc], o[dt], 0, 0, 0);
+    };
+    auto own_part = [&]() {
+        {
+            const bf16_bits* src = vimg + static_cast<int64_t>(jp) * kImageElems;
+#pragma unroll
+            for (int f = 0; f < 16; ++f) vreg[f] = *reinterpret_cast<const bf16x8*>(src + f * 512);
+        }
+        floatx4 s[4];
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt) s[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+#pragma unroll
+            for (int kt = 0; kt < 4; ++kt)
+                s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[kt * 4 + c], qf[c], s[kt], 0, 0, 0);
+        bf16x8 pf[2];
+        softmax_step(s, m, l, o, pf, (jp == last_blk) ? last_key - jp * kBlockN : kBlockN, g, p.scale_log2);
+#pragma unroll
+        for (int cc = 0; cc < 2; ++cc)
+#pragma unroll
+            for (int dt = 0; dt < 8; ++dt)
+                o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg[dt * 2 + cc], pf[cc], o[dt], 0, 0, 0);
+        const int jn = next_own();
         k_ahead = false;
-        if (jp >= 0) {                                         // per wavefront
-            {
-                const bf16_bits* src = vimg + static_cast<int64_t>(jp) * kImageElems;
+        if (jn >= 0) {                                         // K fragments of the next own block
+            const bf16_bits* src = kimg + static_cast<int64_t>(jn) * kImageElems;
 #pragma unroll
-                for (int f = 0; f < 16; ++f) vreg[f] = *reinterpret_cast<const bf16x8*>(src + f * 512);
-            }
-            floatx4 s[4];
-#pragma unroll
-            for (int kt = 0; kt < 4; ++kt) s[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int c = 0; c < 4; ++c)
-#pragma unroll
-                for (int kt = 0; kt < 4; ++kt)
-                    s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[kt * 4 + c], qf[c], s[kt], 0, 0, 0);
-            bf16x8 pf[2];
-            softmax_step(s, m, l, o, pf, (jp == last_blk) ? last_key - jp * kBlockN : kBlockN, g, p.scale_log2);
-#pragma unroll
-            for (int cc = 0; cc < 2; ++cc)
-#pragma unroll
-                for (int dt = 0; dt < 8; ++dt)
-                    o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg[dt * 2 + cc], pf[cc], o[dt], 0, 0, 0);
-            const int jn = next_own();
-            if (jn >= 0) {                                     // K fragments of the next own block
-                const bf16_bits* src = kimg + static_cast<int64_t>(jn) * kImageElems;
-#pragma unroll
-                for (int f = 0; f < 16; ++f) kreg[f] = *reinterpret_cast<const bf16x8*>(src + f * 512);
-                k_ahead = true;
-            }
-            jp = jn;
+            for (int f = 0; f < 16; ++f) kreg[f] = *reinterpret_cast<const bf16x8*>(src + f * 512);
+            k_ahead = true;
+        }
+        jp = jn;
+    };
+    while (c0 >= 0 || jp >= 0) {
+        int n0 = -1, n1 = -1;
+        if (c0 >= 0) {                                         // uniform over the workgroup
+            // younger than this wavefront's DMA loads of the pair: the 16 K loads of the coming own block
+            if (k_ahead) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();                                   // the pair is in LDS for everyone; the other two tiles are free
+            n0 = c1 >= 0 ? next_common() : -1;
+            n1 = n0 >= 0 ? next_common() : -1;
+            if (n0 >= 0) issue(n0, 2 - 2 * half);
+            if (n1 >= 0) issue(n1, 3 - 2 * half);
+            if (live) common_part(c0, 2 * half);
+        }
+        if (jp >= 0) own_part();                               // per wavefront
+        if (c1 >= 0 && live) common_part(c1, 2 * half + 1);
+        if (jp >= 0 && c1 >= 0) own_part();
+        if (c0 >= 0) {
+            c0 = n0;
+            c1 = n1;
+            half ^= 1;
         }
     }
     if (!live) return;
