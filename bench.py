@@ -28,7 +28,7 @@ if ROOT not in sys.path:
 # HBM bytes per launch of the dominant kernel at the default workload: 2.00 x FETCH_SIZE + 1.00 x WRITE_SIZE of the two
 # rocprofv3 --pmc runs summarised in profiles/stage2_fwd_config2_hbm_traffic.md (counters cannot be read from inside
 # this process); null for any other workload
-MEASURED_FWD_TRAFFIC_BYTES = 5.66e9
+MEASURED_FWD_TRAFFIC_BYTES = 5.86e9
 PEAK_BF16_TFLOPS = 2500.0      # MI355X dense bf16 MFMA peak (vendor figure, no sparsity)
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E peak
 
@@ -44,6 +44,9 @@ def parse_args():
     ap.add_argument("--unfused-front-end", action="store_true",
                     help="time the reference's call sequence (Stage-1 scores, then max_pooling_1d) instead of the fused launch")
     ap.add_argument("--no-stages", action="store_true", help="skip the per-stage and kernel-only timings")
+    ap.add_argument("--no-shared-selection", action="store_true",
+                    help="skip the extra leg with selections shared inside each query block (keeps a profile of the "
+                         "Stage-2 kernel to one workload)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three plain 1 GiB device copies (a kernel of known traffic for scaling rocprofv3 --pmc counters)")
     return ap.parse_args()
@@ -255,7 +258,7 @@ def main():
             peak_l1 = 256 * 64 * 2.4e9 / 1e12
             result["roofline"]["gather"] = {"bound": "l1", "bytes": gather_bytes, "achieved": gather_bytes / k_ms / 1e9,
                                             "peak": peak_l1, "unit": "TB/s", "frac": gather_bytes / k_ms / 1e9 / peak_l1}
-        if S % 64 == 0:
+        if S % 64 == 0 and not args.no_shared_selection:
             # the same operator when neighbouring tokens agree on their blocks (every token of a 64-token query block
             # takes the selection of the block's first token): the i.i.d. scores of the synthetic input are the worst
             # case for the row-parallel kernels, whose shared-block walk this leg shows
