@@ -183,3 +183,54 @@ def test_random_case_decode_options(seed):
     print(f"seed {seed}: B {B} Hk {Hk} cap {cap} page {page} new {new} layout {layout} pad {pad} lens {lens} "
           f"k {k_sel} splits {num_splits} rotary {'rotary_cos' in opts}", flush=True)
     D.check_ext(ops, q, kc, vc, L, idx, cap, new=(kn, vn) if new else None, num_splits=num_splits, **opts)
+
+
+def test_empty_sequence_inside_a_packed_batch():
+    """cu_seqlens with a zero-length sequence in the middle and at the end: every kernel skips it."""
+    import infllmv2_cuda_impl_amd as ops
+    r = np.random.default_rng(77)
+    seqs = [150, 0, 200, 0]
+    Hk, k_sel, T = 2, 3, 350
+    cu = np.cumsum([0] + seqs).astype(np.int32)
+    mk = lambda *shape: O.bf16_round(r.standard_normal(shape).astype(np.float32))
+    q, k, v, dout = mk(T, 32, 128), mk(T, Hk, 128), mk(T, Hk, 128), mk(T, 32, 128)
+    idx = np.full((Hk, T, k_sel), -1, np.int32)
+    for b, s in enumerate(seqs):
+        for i in range(s):
+            nb = (s + 63) // 64
+            for h in range(Hk):
+                idx[h, cu[b] + i, :min(k_sel, nb)] = np.sort(r.permutation(nb)[:k_sel])
+    dev = torch.device("cuda:0")
+    t = lambda x: torch.from_numpy(x).to(torch.bfloat16).to(dev)
+    tcu = torch.from_numpy(cu).to(dev)
+    qg, kg, vg = [t(x).requires_grad_(True) for x in (q, k, v)]
+    out, lse, _ = ops.infllmv2_attn_varlen_func(qg, kg, vg, tcu, tcu, max(seqs), max(seqs), causal=True,
+                                                topk_idx=torch.from_numpy(idx).to(dev), return_attn_probs=True)
+    out.backward(t(dout))
+    words, _ = O.topk_to_uint64(idx, max(seqs), 64)
+    ref_o, ref_lse = O.stage2_forward(q, k, v, cu, cu, words, 128 ** -0.5, True)
+    assert np.abs(bf16_np(out) - ref_o).max() <= 2e-2
+    dq, dk, dv = O.stage2_backward(q, k, v, dout, cu, cu, words, 128 ** -0.5, True)
+    for got, ref in ((qg.grad, dq), (kg.grad, dk), (vg.grad, dv)):
+        s = max(1.0, float(np.abs(ref).max()))
+        e = np.abs(bf16_np(got).astype(np.float64) - ref)
+        assert e.max() <= 2e-2 * s and e.mean() <= 1e-3 * s
+    # selection front end on the same batch
+    tk = t(k)
+    kf, cu_f = ops.compress_keys(tk, tcu, max(seqs), 32, 16)
+    kc, cu_c = ops.compress_keys(tk, tcu, max(seqs), 128, 64)
+    rkf, rcu_f = O.compress_keys(k, cu, 32, 16)
+    rkc, rcu_c = O.compress_keys(k, cu, 128, 64)
+    assert np.array_equal(cu_f.cpu().numpy(), rcu_f) and np.array_equal(cu_c.cpu().numpy(), rcu_c)
+    max_lk = int(np.diff(rcu_f).max())
+    score = ops.infllmv2_attn_stage1(t(q), kf, kc, tcu, cu_f, cu_c, max(seqs), max_lk, causal=True)
+    ref = O.stage1_scores(q, O.bf16_round(rkf), O.bf16_round(rkc), cu, rcu_f, rcu_c, max_lk, 128 ** -0.5, True,
+                          round_output=False).astype(np.float64)
+    assert np.all(np.abs(bf16_np(score) - ref) <= 2.0 ** -7 * np.abs(ref) + 2e-3)
+    cache_lens = torch.zeros(len(seqs), dtype=torch.int32, device=dev)
+    pooled = ops.max_pooling_1d_varlen(score, tcu, cu_f, cache_lens, max(seqs), max_lk, 1, 1)
+    fused = ops.infllmv2_attn_stage1_pooled(t(q), kf, kc, tcu, cu_f, cu_c, max(seqs), max_lk, 1, 1, cache_lens=cache_lens,
+                                            causal=True)
+    assert torch.equal(fused.view(torch.int16), pooled.view(torch.int16))
+    assert np.array_equal(bf16_np(pooled), O.max_pooling_1d_varlen(bf16_np(score), cu, rcu_f, np.zeros(4, np.int32),
+                                                                   max(seqs), max_lk, 1, 1))
