@@ -234,3 +234,30 @@ def test_empty_sequence_inside_a_packed_batch():
     assert torch.equal(fused.view(torch.int16), pooled.view(torch.int16))
     assert np.array_equal(bf16_np(pooled), O.max_pooling_1d_varlen(bf16_np(score), cu, rcu_f, np.zeros(4, np.int32),
                                                                    max(seqs), max_lk, 1, 1))
+
+
+def test_operators_follow_the_current_stream():
+    """Everything is launched on torch's current stream (flash_api.cpp:764; topk_to_uint64.py:54-55): the same calls
+    on a side stream (default priority) give the same bits, forward and backward."""
+    import infllmv2_cuda_impl_amd as ops
+    from test_gpu_stage2_fwd import make_case
+    dev = torch.device("cuda:0")
+    q, k, v, cu_q, cu_k, idx = make_case(55, [700, 300], [700, 300], 2, 5, dev)
+    dout = torch.randn(q.shape, generator=torch.Generator(device="cpu").manual_seed(56)).to(torch.bfloat16).to(dev)
+
+    def run():
+        qg, kg, vg = [t.clone().requires_grad_(True) for t in (q, k, v)]
+        out = ops.infllmv2_attn_varlen_func(qg, kg, vg, cu_q, cu_k, 700, 700, causal=True, topk_idx=idx, deterministic=True)
+        out.backward(dout)
+        sel = ops.select_blocks(q, k, cu_q, cu_k, 700, 700, 4, 1, 1,
+                                cache_lens=torch.zeros(2, dtype=torch.int32, device=dev), max_cache_len=0)
+        return out.detach(), qg.grad, kg.grad, vg.grad, sel
+    ref = run()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream(device=dev)
+    side.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(side):
+        got = run()
+    side.synchronize()
+    for a, b in zip(ref, got):
+        assert torch.equal(a, b)
