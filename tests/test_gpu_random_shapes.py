@@ -261,3 +261,42 @@ def test_operators_follow_the_current_stream():
     side.synchronize()
     for a, b in zip(ref, got):
         assert torch.equal(a, b)
+
+
+def test_forward_and_decode_replay_from_a_hip_graph():
+    """The library launches kernels only (no allocation, memset, copy or synchronisation of its own), so a forward
+    step and a decode step can be captured in a HIP graph.  Replayed three times, with eager work and
+    synchronisations in between and new input values each time, every replay equals the eager result."""
+    import infllmv2_cuda_impl_amd as ops
+    from test_gpu_stage2_fwd import make_case
+    import test_gpu_decode as D
+    dev = torch.device("cuda:0")
+    q, k, v, cu_q, cu_k, idx = make_case(61, [600, 424], [600, 424], 2, 5, dev)
+    dq_, dkc, dvc, _, _, L, didx = D.make(62, 3, 512, [200, 333, 448], 4)
+    dq_, dkc, dvc, L, didx = [t.to(dev) for t in (dq_, dkc, dvc, L, didx)]
+
+    def step():
+        sel = ops.select_blocks(q, k, cu_q, cu_k, 600, 600, 5, 1, 1,
+                                cache_lens=torch.zeros(2, dtype=torch.int32, device=dev), max_cache_len=0)
+        out = ops.infllmv2_attn_varlen_func(q, k, v, cu_q, cu_k, 600, 600, causal=True, topk_idx=sel)
+        dec = ops.infllmv2_attn_with_kvcache(dq_, dkc, dvc, cache_seqlens=L, topk_idx=didx)
+        return sel, out, dec
+    step()                                                     # warm-up outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream(device=dev)
+    side.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            captured = step()
+    torch.cuda.synchronize()
+    gen = torch.Generator(device="cpu").manual_seed(63)
+    for _ in range(3):
+        q.copy_(torch.randn(q.shape, generator=gen).to(torch.bfloat16))       # new values in the captured tensors
+        dq_.copy_(torch.randn(dq_.shape, generator=gen).to(torch.bfloat16))
+        eager = step()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for a, b in zip(eager, captured):
+            assert torch.equal(a, b)
