@@ -92,3 +92,44 @@ def test_product_package_does_not_import_oracle():
             if f.endswith((".py", ".hip", ".h")):
                 src = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in src, f"{f} mentions the oracle"
+
+
+def test_ctypes_signatures_have_the_headers_parameter_counts():
+    """Every declaration of include/infllmv2_hip.h is parsed for its parameter list; the ctypes argtypes of the
+    binding must have the same length and pointer / integer / float kinds in the same places (an argument added on
+    one side only would shift every later one silently)."""
+    import ctypes as C
+    import re
+    from infllmv2_cuda_impl_amd import _lib
+    text = open(os.path.join(ROOT, "include", "infllmv2_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", " ", text, flags=re.S)
+    text = re.sub(r"//[^\n]*", " ", text)
+    decls = dict(re.findall(r"\b(infllmv2_\w+)\s*\(([^)]*)\)\s*;", text))
+    assert len(decls) >= 10
+
+    def kind_of_c(param):
+        p = param.strip()
+        if p in ("void", ""):
+            return None
+        if "*" in p:
+            return "p"
+        if re.search(r"\b(float|double)\b", p):
+            return "f"
+        return "i"
+
+    def kind_of_ctype(t):
+        if t in (C.c_void_p, C.c_char_p) or isinstance(t, type) and issubclass(t, C._Pointer):
+            return "p"
+        if t in (C.c_float, C.c_double):
+            return "f"
+        return "i"
+    checked = 0
+    for name, params in decls.items():
+        want = [k for k in (kind_of_c(x) for x in params.split(",")) if k is not None]
+        fn = getattr(_lib.lib, name)
+        if fn.argtypes is None:
+            continue
+        got = [kind_of_ctype(t) for t in fn.argtypes]
+        assert got == want, (name, "".join(got), "".join(want))
+        checked += 1
+    assert checked >= 10
