@@ -300,3 +300,26 @@ def test_forward_and_decode_replay_from_a_hip_graph():
         torch.cuda.synchronize()
         for a, b in zip(eager, captured):
             assert torch.equal(a, b)
+
+
+def test_kv_heads_can_be_computed_separately():
+    """Sharding by KV head (the reference's tests/test_tp.py:25-33 reassembles such shards): each KV head with its 16
+    query heads, given as strided slices of the full tensors, yields exactly the slice of the full result, forward
+    and backward (deterministic mode, so that dK/dV compare bit for bit)."""
+    import infllmv2_cuda_impl_amd as ops
+    from test_gpu_stage2_fwd import make_case
+    dev = torch.device("cuda:0")
+    q, k, v, cu_q, cu_k, idx = make_case(71, [500, 260], [500, 260], 2, 4, dev)
+    dout = torch.randn(q.shape, generator=torch.Generator(device="cpu").manual_seed(72)).to(torch.bfloat16).to(dev)
+
+    def run(qs, ks, vs, ds, sel):
+        qg, kg, vg = [t.clone().requires_grad_(True) for t in (qs, ks, vs)]     # clones keep the slices' strides
+        out = ops.infllmv2_attn_varlen_func(qg, kg, vg, cu_q, cu_k, 500, 500, causal=True, topk_idx=sel, deterministic=True)
+        out.backward(ds)
+        return out.detach(), qg.grad, kg.grad, vg.grad
+    full = run(q, k, v, dout, idx)
+    for h in range(2):
+        hs = slice(16 * h, 16 * h + 16)
+        part = run(q[:, hs], k[:, h:h + 1], v[:, h:h + 1], dout[:, hs], idx[h:h + 1].contiguous())
+        assert torch.equal(part[0], full[0][:, hs]) and torch.equal(part[1], full[1][:, hs])
+        assert torch.equal(part[2], full[2][:, h:h + 1]) and torch.equal(part[3], full[3][:, h:h + 1])
