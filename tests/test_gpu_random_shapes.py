@@ -323,3 +323,29 @@ def test_kv_heads_can_be_computed_separately():
         part = run(q[:, hs], k[:, h:h + 1], v[:, h:h + 1], dout[:, hs], idx[h:h + 1].contiguous())
         assert torch.equal(part[0], full[0][:, hs]) and torch.equal(part[1], full[1][:, hs])
         assert torch.equal(part[2], full[2][:, h:h + 1]) and torch.equal(part[3], full[3][:, h:h + 1])
+
+
+def test_query_chunk_against_the_full_prefix_equals_rows_of_the_full_run():
+    """Sharding by query range (the reference's tests/test_stage1_cp_load.py scores a chunk of queries against the
+    whole key history): the last 256 tokens of a 1024-token sequence as queries, all 1024 tokens as keys, give the
+    same Stage-1 scores and the same attention output as those rows of the full computation (bit for bit: the chunk
+    starts on a workgroup boundary, so every reduction runs in the same order)."""
+    import infllmv2_cuda_impl_amd as ops
+    from test_gpu_stage2_fwd import make_case
+    dev = torch.device("cuda:0")
+    S, C = 1024, 256
+    q, k, v, cu, _, idx = make_case(81, [S], [S], 2, 6, dev)
+    one = lambda n: torch.tensor([0, n], dtype=torch.int32, device=dev)
+    kf, cu_f = ops.compress_keys(k, cu, S, 32, 16)
+    kc, cu_c = ops.compress_keys(k, cu, S, 128, 64)
+    lf = int(cu_f[-1])
+    full_score = ops.infllmv2_attn_stage1(q, kf, kc, cu, cu_f, cu_c, S, lf, causal=True)
+    part_score = ops.infllmv2_attn_stage1(q[S - C:], kf, kc, one(C), cu_f, cu_c, C, lf, causal=True)
+    assert torch.equal(part_score.view(torch.int16), full_score[:, S - C:].contiguous().view(torch.int16))
+    full_pool = ops.max_pooling_1d(full_score, 0, 1, 1)
+    part_pool = ops.max_pooling_1d(part_score, S - C, 1, 1)     # cache_len = tokens before the chunk
+    assert torch.equal(part_pool.view(torch.int16), full_pool[:, S - C:].contiguous().view(torch.int16))
+    full_out = ops.infllmv2_attn_varlen_func(q, k, v, cu, cu, S, S, causal=True, topk_idx=idx)
+    part_out = ops.infllmv2_attn_varlen_func(q[S - C:], k, v, one(C), cu, C, S, causal=True,
+                                             topk_idx=idx[:, S - C:].contiguous())
+    assert torch.equal(part_out, full_out[S - C:])
