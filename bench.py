@@ -280,6 +280,7 @@ def main():
                 qg.grad = kg.grad = vg.grad = None
             fb_ms = event_ms(torch, fwd_bwd, 5)
             result["stage2_fwd_bwd_ms"] = fb_ms
+            result["stage2_bwd_ms"] = fb_ms - stages["stage2_fwd_op"]          # the backward alone (incl. its packing and mask transpose)
             result["stage2_fwd_bwd_tflops"] = 3.5 * fwd_flops / fb_ms / 1e9
             result["stage2_fwd_bwd_frac_peak"] = 3.5 * fwd_flops / fb_ms / 1e9 / PEAK_BF16_TFLOPS
         except ImportError:
