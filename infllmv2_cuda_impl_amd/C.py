@@ -6,8 +6,9 @@ what the library checks, returns nothing and is asynchronous on the given stream
 tensor group (entry.cu:13-18, 209-214) takes torch tensors in the layouts the reference's Python wrappers
 produce — for the sparse path q / out / dout re-laid-out as ``(total_q * 16, Hk, d)`` with
 ``cu_seqlens_q`` and ``max_seqlen_q`` multiplied by 16 — and is served by the same kernels through
-strides, without copying.  ``fwd``, ``bwd`` (fixed-length dense attention) and ``get_probs`` are bound
-by the reference but never reached from its Python package; they raise NotImplementedError here.
+strides, without copying.  ``fwd`` and ``bwd`` (fixed-length dense attention, never reached from the
+reference's Python package) run the packed kernels with equal sequence lengths; ``get_probs`` (bound by
+the reference, called by nothing) raises NotImplementedError.
 """
 from __future__ import annotations
 
@@ -94,7 +95,8 @@ def varlen_fwd(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftpad_k_,
                window_size_right, softcap, return_softmax, gen_, blockmask_=None):
     """mha_varlen_fwd (flash_api.cpp:519-782).  Returns ``[out, softmax_lse, p, rng_state]``."""
     _common_checks(q, k, v, cu_seqlens_q, cu_seqlens_k)
-    _reject_unsupported(p_dropout, (window_size_left, window_size_right), softcap, alibi_slopes_, is_causal)
+    is_causal = _reject_unsupported(p_dropout, (window_size_left, window_size_right), softcap, alibi_slopes_, is_causal,
+                                    max_seqlen_k)
     for name, val in (("seqused_k", seqused_k), ("leftpad_k", leftpad_k_), ("block_table", block_table_)):
         if val is not None:
             raise RuntimeError(f"{name} is not supported by this build")
@@ -143,7 +145,8 @@ def varlen_fwd_stage1(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, cu_seqlens_v, s
     Returns ``[p]`` with p bf16 ``(Hk, T, round128(max_seqlen_k))`` like the reference's buffer
     (flash_api.cpp:941); columns >= max_seqlen_k are zero."""
     _common_checks(q, k, v, cu_seqlens_q, cu_seqlens_k)
-    _reject_unsupported(p_dropout, (window_size_left, window_size_right), softcap, alibi_slopes_, is_causal)
+    is_causal = _reject_unsupported(p_dropout, (window_size_left, window_size_right), softcap, alibi_slopes_, is_causal,
+                                    max_seqlen_k)
     Hk = k.shape[1]
     if q.shape[1] != Hk or q.shape[0] % GROUP != 0:
         raise RuntimeError("stage 1 expects the query re-laid-out as (total_q * 16, num_heads_k, head_size)")
@@ -169,7 +172,8 @@ def varlen_bwd(dout, q, k, v, out, softmax_lse, dq_, dk_, dv_, cu_seqlens_q, cu_
     mask (the dQ kernel walks rows, the dK/dV kernel re-derives the columns).  dq, dk, dv are written in
     place and returned with an empty softmax_d."""
     _common_checks(q, k, v, cu_seqlens_q, cu_seqlens_k)
-    _reject_unsupported(p_dropout, (window_size_left, window_size_right), softcap, alibi_slopes_, is_causal)
+    is_causal = _reject_unsupported(p_dropout, (window_size_left, window_size_right), softcap, alibi_slopes_, is_causal,
+                                    max_seqlen_k)
     Hk = k.shape[1]
     expanded = col_blockmask_ is not None and q.shape[1] == Hk
     batch = cu_seqlens_q.numel() - 1

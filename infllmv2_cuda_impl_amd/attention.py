@@ -23,23 +23,43 @@ def _dense_last_dim(x):
     return x.contiguous() if x is not None and x.stride(-1) != 1 else x
 
 
-def _reject_unsupported(dropout_p, window_size, softcap, alibi_slopes, causal):
+def _reject_unsupported(dropout_p, window_size, softcap, alibi_slopes, causal, max_seqlen_k=None):
     """Options the reference build compiles out (setup.py:235-239) fail with its messages
-    (flash_api.cpp:107-109, 131-133, 144-147, 330-332)."""
+    (flash_api.cpp:107-109, 131-133, 144-147, 330-332).  Returns the causal flag the kernels must run with, derived
+    from the window the way the reference derives it: a window side that reaches ``max_seqlen_k`` is unbounded
+    (flash_api.cpp:621-622), ``causal`` closes the right side (flash_api.cpp:600), and the launch is causal iff the
+    left side is unbounded and the right side is 0 (flash_api.cpp:137) -- so ``window_size=(-1, 0)`` with
+    ``causal=False`` runs causal."""
     if softcap > 0.0:
         raise RuntimeError("This flash attention build does not support softcap.")
     if not dropout_p < 1.0:
         raise RuntimeError("Expected p_dropout < 1.f to be true, but got false.")
     if dropout_p != 0.0:
         raise RuntimeError("This flash attention build does not support dropout.")
-    wl, wr = window_size
-    if causal:
-        wr = 0
-    is_causal = wl < 0 and wr == 0
-    if not (is_causal or (wl < 0 and wr < 0)):
+    is_causal = normalise_causal(causal, window_size, max_seqlen_k)
+    if is_causal is None:
         raise RuntimeError("This flash attention build does not support local attention.")
     if alibi_slopes is not None:
         raise RuntimeError("This flash attention build does not support alibi.")
+    return is_causal
+
+
+def normalise_causal(causal, window_size, max_seqlen_k=None):
+    """True / False: the causal flag of the launch; None: a sliding window that this build (like the reference's,
+    FLASHATTENTION_DISABLE_LOCAL) does not have."""
+    wl, wr = int(window_size[0]), int(window_size[1])
+    if max_seqlen_k is not None:
+        if wl >= max_seqlen_k:
+            wl = -1
+        if wr >= max_seqlen_k:
+            wr = -1
+    if causal:
+        wr = 0
+    if wl < 0 and wr == 0:
+        return True
+    if wl < 0 and wr < 0:
+        return False
+    return None
 
 
 def _check_qkv(q, k, v, cu_seqlens_q, cu_seqlens_k, same_kv_len=True):
@@ -128,7 +148,7 @@ class Infllmv2AttnVarlenFunc(torch.autograd.Function):
                 causal, window_size, softcap, alibi_slopes, deterministic, return_softmax, block_table, topk_idx):
         if softmax_scale is None:
             softmax_scale = q.shape[-1] ** (-0.5)
-        _reject_unsupported(dropout_p, window_size, softcap, alibi_slopes, causal)
+        causal = _reject_unsupported(dropout_p, window_size, softcap, alibi_slopes, causal, max_seqlen_k)
         if block_table is not None:
             raise RuntimeError("paged KV (block_table) is not supported by this build")
         q, k, v = [_dense_last_dim(x) for x in (q, k, v)]
@@ -203,7 +223,7 @@ def infllmv2_attn_stage1(q, k, v, cu_seqlens_q, cu_seqlens_k, cu_seqlens_v, max_
     from .stage1 import stage1_scores
     if softmax_scale is None:
         softmax_scale = q.shape[-1] ** (-0.5)
-    _reject_unsupported(dropout_p, window_size, softcap, alibi_slopes, causal)
+    causal = _reject_unsupported(dropout_p, window_size, softcap, alibi_slopes, causal, max_seqlen_k)
     if block_table is not None:
         raise RuntimeError("paged KV (block_table) is not supported by this build")
     q, k, v = [_dense_last_dim(x) for x in (q, k, v)]

@@ -17,7 +17,18 @@ from ._util import ptr, stream_ptr
 
 GROUP = 16
 HAVE_BACKWARD = True
-HANDOFF_MAX_BYTES = 64 << 30          # above this much dS scratch the backward recomputes S and dP in the dQ kernel
+# The dS hand-off (the dK/dV kernel stores its dS tiles, the dQ kernel reads them instead of recomputing S and dP) is
+# opt-in: it buys a few per cent of backward time for (k + 1) * 2 KiB of transient workspace per token and KV head
+# (8.7 GB at 32768 tokens with k = 64).  INFLLMV2_BWD_HANDOFF=1 switches it on for workspaces up to
+# INFLLMV2_BWD_HANDOFF_MAX_BYTES (default 16 GiB); anything larger, or an allocation failure, recomputes.
+HANDOFF_MAX_BYTES = 16 << 30
+
+
+def _handoff_limit() -> int:
+    """Bytes of dS scratch the caller allows; 0 = recompute (the default)."""
+    if os.environ.get("INFLLMV2_BWD_HANDOFF", "0") != "1":
+        return 0
+    return int(os.environ.get("INFLLMV2_BWD_HANDOFF_MAX_BYTES", HANDOFF_MAX_BYTES))
 
 
 def _nat(t):
@@ -29,7 +40,8 @@ def sparse_backward(dout, q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, max_seq
     """Returns (dq, dk, dv) with the shapes and dtype of (q, k, v).  dq is always bit-reproducible; with
     ``deterministic`` dk and dv are too (slots + ordered sum instead of fp32 atomics, at the price of a large workspace).
     ``max_selected`` > 0 (an upper bound of the set bits per mask row) lets the dK/dV kernel hand its dS tiles to the dQ
-    kernel (2 KiB of workspace per token, KV head and selectable block); INFLLMV2_BWD_HANDOFF=0 switches that off."""
+    kernel (2 KiB of workspace per token, KV head and selectable block) when INFLLMV2_BWD_HANDOFF=1 is set; the default
+    recomputes S and dP in the dQ kernel and needs no such workspace."""
     if dout.stride(-1) != 1:
         dout = dout.contiguous()
     if dout.dtype != q.dtype or tuple(dout.shape) != tuple(q.shape):
@@ -43,8 +55,7 @@ def sparse_backward(dout, q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, max_seq
     else:
         lse_strides = _lib.i64_array([1, total_q, GROUP * total_q])
     n64 = 0 if fwd_mask is None else fwd_mask.shape[-1]
-    if fwd_mask is None or os.environ.get("INFLLMV2_BWD_HANDOFF", "1") == "0" or \
-            Hk * total_q * (max_selected + 1) * 2048 > HANDOFF_MAX_BYTES:
+    if fwd_mask is None or Hk * total_q * (max_selected + 1) * 2048 > _handoff_limit():
         max_selected = 0
     def allocate(selected):
         ws_bytes = _lib.lib.infllmv2_varlen_bwd_workspace_bytes_ex(batch, total_q, total_k, Hk, max_seqlen_k,

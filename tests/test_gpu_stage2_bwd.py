@@ -133,15 +133,16 @@ def test_deterministic_mode(ops, sq, sk, k_sel, causal, sparse):
 @pytest.mark.parametrize("handoff", ["1", "0"])
 @pytest.mark.parametrize("sq,sk,k_sel", [([300], [4500], 12), ([1500, 700], [1500, 700], 6), ([130], [130], 3)])
 def test_ds_handoff_and_recompute_agree_with_oracle(ops, monkeypatch, handoff, sq, sk, k_sel):
-    """With a top-k mask the dK/dV kernel hands its dS tiles to the dQ kernel (slot = rank of the block in the token's
+    """With a top-k mask and INFLLMV2_BWD_HANDOFF=1 the dK/dV kernel hands its dS tiles to the dQ kernel (slot = rank of the block in the token's
     mask row; [300] x [4500] has rows of two 64-bit words, so ranks continue across a word boundary);
-    INFLLMV2_BWD_HANDOFF=0 keeps the dQ kernel that recomputes S and dP.  Both must meet the oracle."""
+    without INFLLMV2_BWD_HANDOFF=1 (the default) the dQ kernel recomputes S and dP.  Both must meet the oracle."""
     monkeypatch.setenv("INFLLMV2_BWD_HANDOFF", handoff)
     run_case(ops, sq, sk, 2, k_sel, True, seed=21)
 
 
-def test_ds_handoff_with_duplicate_and_missing_indices(ops):
+def test_ds_handoff_with_duplicate_and_missing_indices(ops, monkeypatch):
     """Rows with fewer set bits than the announced bound (-1 entries and repeated blocks) leave slots unused."""
+    monkeypatch.setenv("INFLLMV2_BWD_HANDOFF", "1")
     dev = torch.device("cuda:0")
     q, k, v, cu_q, cu_k, idx = make_case(23, [700], [700], 2, 5, dev)
     idx[:, ::3, 1] = idx[:, ::3, 0]
@@ -161,6 +162,7 @@ def test_ds_handoff_falls_back_when_its_workspace_does_not_fit(ops, monkeypatch)
     """The dS tiles need (k + 1) * 2 KiB per token and KV head; when that allocation fails the backward takes the
     dQ kernel that recomputes S and dP.  The failure is simulated on the host: the first workspace request of the
     backward raises torch's out-of-memory error."""
+    monkeypatch.setenv("INFLLMV2_BWD_HANDOFF", "1")
     dev = torch.device("cuda:0")
     q, k, v, cu_q, cu_k, idx = make_case(31, [700], [700], 2, 5, dev)
     dout = torch.randn(q.shape, generator=torch.Generator(device="cpu").manual_seed(32)).to(torch.bfloat16).to(dev)

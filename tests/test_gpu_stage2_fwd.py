@@ -128,3 +128,20 @@ def test_rejected_options_raise_like_the_reference(ops):
         f(q, k, v, cu_q.long(), cu_k, 64, 64, topk_idx=idx)
     with pytest.raises(AssertionError):
         f(q, k, v, cu_q, cu_k, 64, 64, topk_idx=idx.long())
+
+
+def test_causal_flag_follows_the_window_like_the_reference(ops):
+    """flash_api.cpp:137, 600, 621-622: window (-1, 0) IS causal whatever the `causal` argument says, and a left window
+    that reaches max_seqlen_k counts as unbounded."""
+    dev = torch.device("cuda:0")
+    q, k, v, cu_q, cu_k, idx = make_case(3, [200], [200], 2, 2, dev)
+    f = ops.infllmv2_attn_varlen_func
+    want = f(q, k, v, cu_q, cu_k, 200, 200, causal=True, topk_idx=idx)
+    assert torch.equal(f(q, k, v, cu_q, cu_k, 200, 200, causal=False, window_size=(-1, 0), topk_idx=idx), want)
+    assert torch.equal(f(q, k, v, cu_q, cu_k, 200, 200, causal=False, window_size=(200, 0), topk_idx=idx), want)
+    assert torch.equal(f(q, k, v, cu_q, cu_k, 200, 200, causal=True, window_size=(4096, 4096), topk_idx=idx), want)
+    non_causal = f(q, k, v, cu_q, cu_k, 200, 200, causal=False, topk_idx=idx)
+    assert not torch.equal(non_causal, want)
+    assert torch.equal(f(q, k, v, cu_q, cu_k, 200, 200, causal=False, window_size=(300, 200), topk_idx=idx), non_causal)
+    with pytest.raises(RuntimeError, match="does not support local attention"):
+        f(q, k, v, cu_q, cu_k, 200, 200, causal=False, window_size=(199, 0), topk_idx=idx)
