@@ -23,7 +23,7 @@
 extern "C" {
 #endif
 
-#define INFLLMV2_ABI_VERSION 4
+#define INFLLMV2_ABI_VERSION 5
 
 /* ---- library ------------------------------------------------------------------------------ */
 
@@ -265,6 +265,26 @@ int infllmv2_fwd_kvcache(void* stream, const void* q, void* kcache, void* vcache
                          const int32_t* cache_leftpad, const int32_t* block_table,
                          int64_t block_table_batch_stride, int page_block_size, const void* rotary_cos,
                          const void* rotary_sin, int rotary_dim, int rotary_interleaved);
+
+/* No counterpart in the reference.  infllmv2_fwd_kvcache for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): the same kernels and arguments, without
+ * the workspace pair.  The split partials and the turned query go to a buffer of INFLLMV2_STATIC_SCRATCH_BYTES that is
+ * part of the library's device code (one copy per GPU, held until the process ends); the call allocates and frees
+ * nothing.  Sizes with infllmv2_fwd_kvcache_workspace_bytes(batch, num_heads_k, num_splits) above that limit are
+ * rejected.  All calls on one GPU share the buffer: calls that overlap on one GPU (different streams or threads) race;
+ * the buffer needs no clearing between calls (every element read has been written by the same call). */
+#define INFLLMV2_STATIC_SCRATCH_BYTES (32u << 20)
+int infllmv2_fwd_kvcache_static(void* stream, const void* q, void* kcache, void* vcache, const void* k_new,
+                                const void* v_new, const int32_t* cache_seqlens, void* out, float* softmax_lse,
+                                const uint64_t* blockmask, int batch, int seqlen_q, int num_heads, int num_heads_k,
+                                int head_dim, int cache_capacity, int seqlen_new, const int64_t* q_strides,
+                                const int64_t* kcache_strides, const int64_t* vcache_strides,
+                                const int64_t* knew_strides, const int64_t* vnew_strides, const int64_t* o_strides,
+                                int n_uint64_per_row, int num_splits, float softmax_scale,
+                                const int32_t* cache_batch_idx, const int32_t* cache_leftpad,
+                                const int32_t* block_table, int64_t block_table_batch_stride, int page_block_size,
+                                const void* rotary_cos, const void* rotary_sin, int rotary_dim,
+                                int rotary_interleaved);
 
 #ifdef __cplusplus
 }

@@ -11,7 +11,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libinfllmv2_hip.so")
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 _p, _i, _i64, _sz, _f = C.c_void_p, C.c_int, C.c_int64, C.c_size_t, C.c_float
 
@@ -35,6 +35,7 @@ SIGNATURES = {
                             _p, _p, _p, _p, _p, _i, _f, _i],
     "infllmv2_varlen_bwd": [_p] * 14 + [_sz, _i, _i64, _i64, _i, _i, _i, _i, _i] + [_p] * 9 + [_i, _f, _i, _i, _i],
     "infllmv2_fwd_kvcache": [_p] * 11 + [_sz] + [_i] * 7 + [_p] * 6 + [_i, _i, _f, _p, _p, _p, _i64, _i, _p, _p, _i, _i],
+    "infllmv2_fwd_kvcache_static": [_p] * 10 + [_i] * 7 + [_p] * 6 + [_i, _i, _f, _p, _p, _p, _i64, _i, _p, _p, _i, _i],
     "infllmv2_pack_kv": [_p, _p, _p, _p, _p, _sz, _i, _i64, _i, _i, _i, _p, _p],
 }
 OTHER = {

@@ -19,6 +19,7 @@
 #include "block_walker.h"
 #include "../../include/infllmv2_hip.h"
 #include <math.h>
+#include <mutex>
 
 namespace infllmv2 {
 
@@ -371,7 +372,7 @@ extern "C" size_t infllmv2_fwd_kvcache_workspace_bytes(int batch, int num_heads_
            static_cast<size_t>(batch) * num_heads_k * 16 * kHeadDim * sizeof(bf16_bits);
 }
 
-extern "C" int infllmv2_fwd_kvcache(void* stream, const void* q, void* kcache, void* vcache, const void* k_new,
+static int fwd_kvcache_impl(void* stream, const void* q, void* kcache, void* vcache, const void* k_new,
                                     const void* v_new, const int32_t* cache_seqlens, void* out, float* softmax_lse,
                                     const uint64_t* blockmask, void* workspace, size_t workspace_bytes, int batch,
                                     int seqlen_q, int num_heads, int num_heads_k, int head_dim, int cache_capacity,
@@ -470,4 +471,81 @@ extern "C" int infllmv2_fwd_kvcache(void* stream, const void* q, void* kcache, v
         IV2_LAUNCH_CHECK();
     }
     return 0;
+}
+
+extern "C" int infllmv2_fwd_kvcache(void* stream, const void* q, void* kcache, void* vcache, const void* k_new,
+                                    const void* v_new, const int32_t* cache_seqlens, void* out, float* softmax_lse,
+                                    const uint64_t* blockmask, void* workspace, size_t workspace_bytes, int batch,
+                                    int seqlen_q, int num_heads, int num_heads_k, int head_dim, int cache_capacity,
+                                    int seqlen_new, const int64_t* q_strides, const int64_t* kcache_strides,
+                                    const int64_t* vcache_strides, const int64_t* knew_strides,
+                                    const int64_t* vnew_strides, const int64_t* o_strides, int n_uint64_per_row,
+                                    int num_splits, float softmax_scale, const int32_t* cache_batch_idx,
+                                    const int32_t* cache_leftpad, const int32_t* block_table,
+                                    int64_t block_table_batch_stride, int page_block_size, const void* rotary_cos,
+                                    const void* rotary_sin, int rotary_dim, int rotary_interleaved) {
+    return fwd_kvcache_impl(stream, q, kcache, vcache, k_new, v_new, cache_seqlens, out, softmax_lse, blockmask, workspace,
+                            workspace_bytes, batch, seqlen_q, num_heads, num_heads_k, head_dim, cache_capacity, seqlen_new,
+                            q_strides, kcache_strides, vcache_strides, knew_strides, vnew_strides, o_strides,
+                            n_uint64_per_row, num_splits, softmax_scale, cache_batch_idx, cache_leftpad, block_table,
+                            block_table_batch_stride, page_block_size, rotary_cos, rotary_sin, rotary_dim,
+                            rotary_interleaved);
+}
+
+// ---- decode for callers that cannot allocate ---------------------------------------------------------------------
+//
+// The split partials and the turned query live in a device array that belongs to the library's code object: every GPU
+// the library runs on holds one copy of it, at its own address, from module load to process end.  `scratch` below is
+// only the host-side handle of that array; the device address is looked up once per device with
+// hipGetSymbolAddress and is what the kernels get.  Nothing in the array has to start at zero: every (sequence, KV
+// head, split) workgroup writes its whole partial slot before the combine kernel reads it, and the turned query is
+// written before it is read.  All calls on one GPU share the array, so calls that overlap on one GPU (two streams, two
+// threads) race; calls on one stream are ordered by the stream.
+static __device__ __align__(256) unsigned char scratch[INFLLMV2_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+}  // namespace
+
+extern "C" int infllmv2_fwd_kvcache_static(void* stream, const void* q, void* kcache, void* vcache, const void* k_new,
+                                           const void* v_new, const int32_t* cache_seqlens, void* out,
+                                           float* softmax_lse, const uint64_t* blockmask, int batch, int seqlen_q,
+                                           int num_heads, int num_heads_k, int head_dim, int cache_capacity,
+                                           int seqlen_new, const int64_t* q_strides, const int64_t* kcache_strides,
+                                           const int64_t* vcache_strides, const int64_t* knew_strides,
+                                           const int64_t* vnew_strides, const int64_t* o_strides, int n_uint64_per_row,
+                                           int num_splits, float softmax_scale, const int32_t* cache_batch_idx,
+                                           const int32_t* cache_leftpad, const int32_t* block_table,
+                                           int64_t block_table_batch_stride, int page_block_size,
+                                           const void* rotary_cos, const void* rotary_sin, int rotary_dim,
+                                           int rotary_interleaved) {
+    IV2_CHECK(batch > 0 && num_heads_k > 0 && num_splits >= 1 && num_splits <= 64,
+              "fwd_kvcache_static: batch, num_heads_k must be positive and num_splits in [1, 64]");
+    const size_t need = infllmv2_fwd_kvcache_workspace_bytes(batch, num_heads_k, num_splits);
+    IV2_CHECK(need <= static_cast<size_t>(INFLLMV2_STATIC_SCRATCH_BYTES),
+              "fwd_kvcache_static: batch %d x %d KV heads x %d splits needs %zu bytes of scratch, the built-in buffer holds %zu; "
+              "use fewer splits or infllmv2_fwd_kvcache with a workspace", batch, num_heads_k, num_splits, need,
+              static_cast<size_t>(INFLLMV2_STATIC_SCRATCH_BYTES));
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    IV2_CHECK(e == hipSuccess && dev >= 0 && dev < kMaxDevices, "fwd_kvcache_static: hipGetDevice failed or device index %d out of range", dev);
+    void* ws = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        if (g_scratch_ptr[dev] == nullptr) {
+            void* sym = nullptr;
+            e = hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch));           // this device's copy of the array
+            IV2_CHECK(e == hipSuccess && sym != nullptr, "fwd_kvcache_static: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+            g_scratch_ptr[dev] = sym;
+        }
+        ws = g_scratch_ptr[dev];
+    }
+    return fwd_kvcache_impl(stream, q, kcache, vcache, k_new, v_new, cache_seqlens, out, softmax_lse, blockmask, ws,
+                            static_cast<size_t>(INFLLMV2_STATIC_SCRATCH_BYTES), batch, seqlen_q, num_heads, num_heads_k,
+                            head_dim, cache_capacity, seqlen_new, q_strides, kcache_strides, vcache_strides, knew_strides,
+                            vnew_strides, o_strides, n_uint64_per_row, num_splits, softmax_scale, cache_batch_idx,
+                            cache_leftpad, block_table, block_table_batch_stride, page_block_size, rotary_cos, rotary_sin,
+                            rotary_dim, rotary_interleaved);
 }
