@@ -23,7 +23,7 @@
 extern "C" {
 #endif
 
-#define INFLLMV2_ABI_VERSION 5
+#define INFLLMV2_ABI_VERSION 6
 
 /* ---- library ------------------------------------------------------------------------------ */
 
@@ -120,6 +120,17 @@ int infllmv2_compress_keys(void* stream, const void* k, void* out, const int32_t
                            int32_t* cu_seqlens_out, int batch, int max_seqlen_k, int num_heads_k, int head_dim,
                            int64_t k_row_stride, int64_t k_head_stride, int kernel_size, int stride, int first_row);
 
+/* The same means for per-sequence key caches, as a batched decode loop keeps them: kcache (batch, capacity, Hk, d)
+ * holds new_lens[b] keys of sequence b, out_cache (batch, rows capacity, Hk, d) its compressed keys; strides
+ * {batch, row, head}.  Rows whose windows were completed between old_lens[b] (null: 0) and new_lens[b] tokens are
+ * written, at most max_new_rows per sequence (the caller's bound: 1 for a one-token step with kernel_size a multiple
+ * of stride); out_lens (batch, or null) receives the number of rows the compressed cache then holds.  The caller
+ * side of the reference does this in Python for one sequence at a time (tests/test_stage1_compressed_lse.py:56-99). */
+int infllmv2_compress_keys_cache(void* stream, const void* kcache, void* out_cache, const int32_t* old_lens,
+                                 const int32_t* new_lens, int32_t* out_lens, int batch, int max_new_rows,
+                                 int num_heads_k, int head_dim, const int64_t* kcache_strides,
+                                 const int64_t* out_strides, int kernel_size, int stride);
+
 /* ---- Stage 1: scoring over compressed keys --------------------------------------------------- */
 
 /* csrc/entry.cu:15,211 `varlen_fwd_stage1` = mha_varlen_fwd_stage1
@@ -152,6 +163,33 @@ int infllmv2_varlen_fwd_stage1_pooled(void* stream, const void* q, const void* k
                                       const int64_t* k_strides, const int64_t* v_strides, int out_len,
                                       float softmax_scale, int is_causal, int kernel_size, int stride, int padding,
                                       int block_size, int local_blocks, int init_blocks);
+
+/* Stage 1 for decode: one query token per sequence, a batch of sequences, each against its own compressed keys.  The
+ * reference serves this case with the same `varlen_fwd_stage1` launch (infllm_v2/infllmv2_sparse_attention.py:483-606
+ * with cu_seqlens_q = 0, 1, 2, ...; flash_api.cpp:784-1049), one 32-thread block per sequence and KV head; here the
+ * compressed keys of every (sequence, KV head) are cut into runs that are scored in parallel (memory-bound), which
+ * needs a small workspace for the partial log-sum-exps.
+ * q: row b (or row cu_seqlens_q[b] when cu_seqlens_q is given; sequences with no query are skipped), strides
+ *   {token, head-in-group, kv-head}.
+ * k (fine keys), v (the key set of the log-sum-exp): strides {batch, row, head}; either packed rows with cumulative
+ *   lengths (cu_seqlens_k / cu_seqlens_v, batch stride unused) or per-sequence caches (sequence b at b * batch stride)
+ *   with k_lens / v_lens (batch) rows each: exactly one of the two pointers per key set.
+ * is_causal: 0 = every key is visible (a decode step: all compressed keys lie in the query's past); 1 = the rule of
+ *   mask.h:273-281 for a 1-token query (the last key of each set is hidden).
+ * pooled == 0: out is the score tensor (Hk, rows, >= max_seqlen_k) with the given head / row strides, every column
+ *   < max_seqlen_k of the sequences' rows written.  pooled != 0: out is max_pooling_1d_varlen of those rows
+ *   (csrc/max_pooling_1d.cuh:12-103; window 5/4/1 on 64-token blocks only), out_len entries per row, with the query
+ *   at position cache_lens[b] (or cache_len for all), bit-identical to pooling the score rows of the same call. */
+size_t infllmv2_stage1_decode_workspace_bytes(int batch, int num_heads_k, int max_seqlen_k, int max_seqlen_v);
+int infllmv2_stage1_decode(void* stream, const void* q, const void* k, const void* v, void* out,
+                           const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, const int32_t* k_lens,
+                           const int32_t* cu_seqlens_v, const int32_t* v_lens, void* workspace,
+                           size_t workspace_bytes, int batch, int num_heads, int num_heads_k, int head_dim,
+                           int max_seqlen_k, int max_seqlen_v, const int64_t* q_strides, const int64_t* k_strides,
+                           const int64_t* v_strides, int64_t out_head_stride, int64_t out_row_stride,
+                           float softmax_scale, int is_causal, int pooled, const int32_t* cache_lens, int cache_len,
+                           int out_len, int kernel_size, int stride, int padding, int block_size, int local_blocks,
+                           int init_blocks);
 
 /* ---- Stage 2: block-sparse attention -------------------------------------------------------- */
 

@@ -11,7 +11,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libinfllmv2_hip.so")
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 _p, _i, _i64, _sz, _f = C.c_void_p, C.c_int, C.c_int64, C.c_size_t, C.c_float
 
@@ -29,8 +29,10 @@ SIGNATURES = {
     "infllmv2_topk": [_p, _i, _i, _i, _i, _p, _p, _p],
     "infllmv2_topk_blocks": [_p, _p, _i64, _p, _i64, _i, _i],
     "infllmv2_compress_keys": [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i64, _i64, _i, _i, _i],
+    "infllmv2_compress_keys_cache": [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _p, _p, _i, _i],
     "infllmv2_varlen_fwd_stage1": [_p, _p, _p, _p, _p, _p, _p, _p, _i, _i64, _i, _i, _i, _i, _i, _p, _p, _p, _i64, _i64, _f, _i],
     "infllmv2_varlen_fwd_stage1_pooled": [_p] * 9 + [_i, _i, _i64, _i, _i, _i, _i, _i, _p, _p, _p, _i, _f] + [_i] * 7,
+    "infllmv2_stage1_decode": [_p] * 11 + [_sz] + [_i] * 6 + [_p] * 3 + [_i64, _i64, _f, _i, _i, _p] + [_i] * 8,
     "infllmv2_varlen_fwd": [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _sz, _i, _i, _i64, _i64, _i, _i, _i, _i, _i,
                             _p, _p, _p, _p, _p, _i, _f, _i],
     "infllmv2_varlen_bwd": [_p] * 14 + [_sz, _i, _i64, _i64, _i, _i, _i, _i, _i] + [_p] * 9 + [_i, _f, _i, _i, _i],
@@ -42,6 +44,7 @@ OTHER = {
     "infllmv2_last_error": (C.c_char_p, []),
     "infllmv2_abi_version": (_i, []),
     "infllmv2_kv_image_bytes": (_sz, [_i64, _i, _i]),
+    "infllmv2_stage1_decode_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "infllmv2_fwd_kvcache_workspace_bytes": (_sz, [_i, _i, _i]),
     "infllmv2_fwd_kvcache_num_splits": (_i, [_i, _i, _i]),
     "infllmv2_varlen_bwd_workspace_bytes": (_sz, [_i, _i64, _i64, _i, _i]),

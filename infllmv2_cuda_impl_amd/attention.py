@@ -267,6 +267,61 @@ def infllmv2_attn_stage1_pooled(q, k, v, cu_seqlens_q, cu_seqlens_k, cu_seqlens_
                          block_size, stride)
 
 
+def infllmv2_attn_stage1_kvcache(q, k_fine_cache, k_coarse_cache, fine_lens, coarse_lens, cache_seqlens, local_blocks,
+                                 init_blocks, max_cache_len=None, block_size=64, stride=16, softmax_scale=None,
+                                 causal=False, pooled=True):
+    """Stage 1 of a batched decode step against per-sequence compressed-key caches (no counterpart in the reference's
+    API, whose varlen Stage 1 needs the compressed keys of all sequences packed into one tensor).
+
+    q ``(batch, 1, nheads, 128)``; ``k_fine_cache`` ``(batch, rows, nheads_k, 128)`` holds ``fine_lens[b]`` stride-16
+    compressed keys of sequence b, ``k_coarse_cache`` ``coarse_lens[b]`` keys of the log-sum-exp set (int32
+    ``(batch,)`` device tensors).  ``cache_seqlens`` int32 ``(batch,)`` is the position of each sequence's query
+    (its tokens before this one), as ``cache_lens`` of ``max_pooling_1d_varlen``.  With ``causal=False`` (a decode
+    step) every compressed key is visible.
+
+    ``pooled=True`` returns bf16 ``(batch, nheads_k, ceil((1 + max_cache_len) / block_size))``: the block scores
+    ``max_pooling_1d_varlen`` gives for the rows ``infllmv2_attn_stage1`` computes on the packed equivalent, ready for
+    ``topk_blocks`` (``max_cache_len`` defaults to the token capacity implied by the fine cache, which avoids a host
+    read).  ``pooled=False`` returns the score rows ``(batch, nheads_k, rows)`` themselves."""
+    from .stage1 import stage1_decode
+    if softmax_scale is None:
+        softmax_scale = q.shape[-1] ** (-0.5)
+    if q.dim() != 4 or q.shape[1] != 1:
+        raise RuntimeError("q must have shape (batch_size, 1, num_heads, head_size)")
+    if q.dtype != torch.bfloat16 or k_fine_cache.dtype != q.dtype or k_coarse_cache.dtype != q.dtype:
+        raise RuntimeError("this build only has bf16 kernels")
+    batch, _, Hq, d = q.shape
+    for name, t in (("q", q), ("k_fine_cache", k_fine_cache), ("k_coarse_cache", k_coarse_cache)):
+        require_gpu(t, name)
+        if t.stride(-1) != 1:
+            raise RuntimeError("Input tensor must have contiguous last dimension")
+    if k_fine_cache.dim() != 4 or k_coarse_cache.dim() != 4 or k_fine_cache.shape[0] != batch or \
+            k_coarse_cache.shape[0] != batch:
+        raise RuntimeError("compressed-key caches must have shape (batch_size, rows, num_heads_k, head_size)")
+    Hk = k_fine_cache.shape[2]
+    if d != 128 or Hq != GROUP * Hk or tuple(k_coarse_cache.shape[2:]) != (Hk, d) or k_fine_cache.shape[3] != d:
+        raise RuntimeError("this build requires head dimension 128 and 16 query heads per key/value head")
+    for name, t in (("fine_lens", fine_lens), ("coarse_lens", coarse_lens), ("cache_seqlens", cache_seqlens)):
+        if t.dtype != torch.int32 or tuple(t.shape) != (batch,) or not t.is_contiguous():
+            raise RuntimeError(f"{name} must be a contiguous int32 tensor of shape (batch_size)")
+    rows_f, rows_c = k_fine_cache.shape[1], k_coarse_cache.shape[1]
+    q3 = q[:, 0]
+    if not pooled:
+        out = torch.empty((batch, Hk, rows_f), dtype=torch.bfloat16, device=q.device)
+        return stage1_decode(q3, k_fine_cache, k_coarse_cache, k_lens=fine_lens, v_lens=coarse_lens,
+                             max_seqlen_k=rows_f, max_seqlen_v=rows_c, softmax_scale=softmax_scale, causal=causal,
+                             out=out, out_head_stride=out.stride(1), out_row_stride=out.stride(0))
+    if max_cache_len is None:
+        max_cache_len = (rows_f + 1) * stride + block_size
+    out_len = (1 + max_cache_len + block_size - 1) // block_size
+    out = torch.empty((batch, Hk, out_len), dtype=torch.bfloat16, device=q.device)
+    return stage1_decode(q3, k_fine_cache, k_coarse_cache, k_lens=fine_lens, v_lens=coarse_lens, max_seqlen_k=rows_f,
+                         max_seqlen_v=rows_c, softmax_scale=softmax_scale, causal=causal, out=out,
+                         out_head_stride=out.stride(1), out_row_stride=out.stride(0), pooled=True,
+                         cache_lens=cache_seqlens, out_len=out_len, local_blocks=local_blocks, init_blocks=init_blocks,
+                         block_size=block_size, stride=stride)
+
+
 def infllmv2_attn_with_kvcache(q, k_cache, v_cache, k=None, v=None, rotary_cos=None, rotary_sin=None,
                                cache_seqlens: Optional[Union[int, torch.Tensor]] = None,
                                cache_batch_idx: Optional[torch.Tensor] = None,

@@ -78,6 +78,55 @@ void compress_keys_kernel(const CompressParams p) {
     }
 }
 
+// The same means for per-sequence key caches (decode): sequence b's keys are rows [0, new_lens[b]) of kcache[b]; the
+// rows of its compressed-key cache that windows completed since old_lens[b] tokens are written, the others are left
+// alone.  A decode step (one more token) completes at most one window per set.
+struct CompressCacheParams {
+    const bf16_bits* k;
+    bf16_bits* out;
+    const int* old_lens;             // null: 0 for every sequence (build everything)
+    const int* new_lens;
+    int* out_lens;                   // null, or (batch): rows the compressed cache holds afterwards
+    int64_t k_batch, k_row, k_head, o_batch, o_row, o_head;
+    int units_per_row, units_per_head;
+    int kernel_size, stride;
+};
+
+__global__ __launch_bounds__(256)
+void compress_keys_cache_kernel(const CompressCacheParams p) {
+    const int b = blockIdx.y;
+    const int rows = compressed_rows(p.new_lens[b], p.kernel_size, p.stride);
+    const int first = p.old_lens ? compressed_rows(p.old_lens[b], p.kernel_size, p.stride) : 0;
+    if (blockIdx.x == 0 && threadIdx.x == 0 && p.out_lens) p.out_lens[b] = rows;
+    const int j0 = first + blockIdx.x * kCompressRowsPerWg;
+    for (int item = threadIdx.x; item < kCompressRowsPerWg * p.units_per_row; item += 256) {
+        const int j = j0 + item / p.units_per_row;
+        if (j >= rows) break;
+        const int u = item % p.units_per_row;
+        const int head = u / p.units_per_head, piece = u % p.units_per_head;
+        const bf16_bits* src = p.k + b * p.k_batch + static_cast<int64_t>(j) * p.stride * p.k_row + head * p.k_head + piece * 8;
+        float acc[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+        for (int i = 0; i < p.kernel_size; ++i) {
+            const uint4 raw = *reinterpret_cast<const uint4*>(src + i * p.k_row);
+            const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                acc[2 * e] += __uint_as_float(w[e] << 16);
+                acc[2 * e + 1] += __uint_as_float(w[e] & 0xffff0000u);
+            }
+        }
+        const float n = static_cast<float>(p.kernel_size);
+        uint4 o;
+        o.x = pack_bf16x2(acc[0] / n, acc[1] / n);
+        o.y = pack_bf16x2(acc[2] / n, acc[3] / n);
+        o.z = pack_bf16x2(acc[4] / n, acc[5] / n);
+        o.w = pack_bf16x2(acc[6] / n, acc[7] / n);
+        *reinterpret_cast<uint4*>(p.out + b * p.o_batch + static_cast<int64_t>(j) * p.o_row + head * p.o_head + piece * 8) = o;
+    }
+}
+
 }  // namespace infllmv2
 
 using namespace infllmv2;
@@ -108,6 +157,33 @@ extern "C" int infllmv2_compress_keys(void* stream, const void* k, void* out, co
     p.kernel_size = kernel_size; p.stride = stride; p.first_row = first_row;
     const dim3 grid((max_rows - first_row + kCompressRowsPerWg - 1) / kCompressRowsPerWg, batch);
     hipLaunchKernelGGL(compress_keys_kernel, grid, dim3(256), 0, st, p);
+    IV2_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int infllmv2_compress_keys_cache(void* stream, const void* kcache, void* out_cache, const int32_t* old_lens,
+                                            const int32_t* new_lens, int32_t* out_lens, int batch, int max_new_rows,
+                                            int num_heads_k, int head_dim, const int64_t* kcache_strides,
+                                            const int64_t* out_strides, int kernel_size, int stride) {
+    IV2_CHECK(batch > 0 && batch <= 65535 && max_new_rows >= 0, "compress_keys_cache: bad batch or max_new_rows");
+    IV2_CHECK(kernel_size > 0 && stride > 0, "compress_keys_cache: kernel_size and stride must be positive");
+    IV2_CHECK(kcache && out_cache && new_lens, "compress_keys_cache: null pointer");
+    IV2_CHECK(head_dim > 0 && head_dim % 8 == 0 && num_heads_k > 0, "compress_keys_cache: head_dim must be a multiple of 8");
+    IV2_CHECK(reinterpret_cast<uintptr_t>(kcache) % 16 == 0 && reinterpret_cast<uintptr_t>(out_cache) % 16 == 0,
+              "compress_keys_cache: caches must be 16-byte aligned");
+    for (int s = 0; s < 3; ++s)
+        IV2_CHECK(kcache_strides[s] % 8 == 0 && out_strides[s] % 8 == 0, "compress_keys_cache: strides must be multiples of 8 elements");
+    CompressCacheParams p{};
+    p.k = static_cast<const bf16_bits*>(kcache);
+    p.out = static_cast<bf16_bits*>(out_cache);
+    p.old_lens = old_lens; p.new_lens = new_lens; p.out_lens = out_lens;
+    p.k_batch = kcache_strides[0]; p.k_row = kcache_strides[1]; p.k_head = kcache_strides[2];
+    p.o_batch = out_strides[0]; p.o_row = out_strides[1]; p.o_head = out_strides[2];
+    p.units_per_row = num_heads_k * head_dim / 8; p.units_per_head = head_dim / 8;
+    p.kernel_size = kernel_size; p.stride = stride;
+    // at least one workgroup per sequence so that out_lens is always written
+    const int groups = max_new_rows > 0 ? (max_new_rows + kCompressRowsPerWg - 1) / kCompressRowsPerWg : 1;
+    hipLaunchKernelGGL(compress_keys_cache_kernel, dim3(groups, batch), dim3(256), 0, static_cast<hipStream_t>(stream), p);
     IV2_LAUNCH_CHECK();
     return 0;
 }

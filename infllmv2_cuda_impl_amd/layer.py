@@ -3,8 +3,9 @@
 The reference ships only the operators; its callers (the model code, README.md:36-60, 118-140) build the
 compressed keys, call ``infllmv2_attn_stage1``, pool, take the top-k and call ``infllmv2_attn_varlen_func`` (prefill)
 or ``infllmv2_attn_with_kvcache`` (decode).  This module is that sequence, so that the kernels can be exercised and
-validated inside one layer: a prefill over packed sequences, and a single-sequence decode loop that keeps the K/V
-cache and the two compressed-key caches up to date (a new compressed key every ``stride`` tokens).
+validated inside one layer: a prefill over packed sequences, a single-sequence decode loop and a batched decode step
+(``BatchCache`` / ``decode_batch``) that keep the K/V caches and the two compressed-key caches up to date (a new
+compressed key every ``stride`` tokens).
 
 Conventions (the ones the operators assume):
 * block size 64, compressed keys kernel 32 / stride 16, log-sum-exp over kernel 128 / stride 64;
@@ -23,8 +24,9 @@ from dataclasses import dataclass
 
 import torch
 
-from .attention import infllmv2_attn_stage1_pooled, infllmv2_attn_varlen_func, infllmv2_attn_with_kvcache
-from .selection import compress_keys, select_blocks, topk_blocks
+from .attention import (infllmv2_attn_stage1_kvcache, infllmv2_attn_stage1_pooled, infllmv2_attn_varlen_func,
+                        infllmv2_attn_with_kvcache)
+from .selection import compress_keys, compress_keys_cache, select_blocks, topk_blocks
 
 
 @dataclass
@@ -41,6 +43,27 @@ class SequenceCache:
         z = lambda n: torch.zeros((n, nheads_k, head_dim), dtype=dtype, device=device)
         return SequenceCache(z(capacity).unsqueeze(0), z(capacity).unsqueeze(0), z(capacity // stride + 1),
                              z(capacity // (4 * stride) + 1), 0)
+
+
+@dataclass
+class BatchCache:
+    """K/V caches of a batch of sequences plus their compressed keys, for batched decoding.  All lengths live on the
+    device (no host read per step); ``max_length`` is the host's upper bound of ``lengths``."""
+    k: torch.Tensor                  # (batch, capacity, nheads_k, d)
+    v: torch.Tensor
+    k_fine: torch.Tensor             # (batch, capacity // stride + 1, nheads_k, d)
+    k_coarse: torch.Tensor           # (batch, capacity // (4 * stride) + 1, nheads_k, d)
+    lengths: torch.Tensor            # int32 (batch,): tokens held per sequence
+    fine_lens: torch.Tensor          # int32 (batch,): rows of k_fine that are valid
+    coarse_lens: torch.Tensor
+    max_length: int = 0
+
+    @staticmethod
+    def empty(batch: int, capacity: int, nheads_k: int, head_dim: int, device, stride: int = 16, dtype=torch.bfloat16):
+        z = lambda n: torch.zeros((batch, n, nheads_k, head_dim), dtype=dtype, device=device)
+        i = lambda: torch.zeros(batch, dtype=torch.int32, device=device)
+        return BatchCache(z(capacity), z(capacity), z(capacity // stride + 1), z(capacity // (4 * stride) + 1),
+                          i(), i(), i(), 0)
 
 
 class InfLLMv2Attention(torch.nn.Module):
@@ -115,3 +138,48 @@ class InfLLMv2Attention(torch.nn.Module):
             topk_idx = topk_blocks(pooled, self.topk).unsqueeze(0)                  # (Hk, 1, topk) -> (1, Hk, 1, topk)
         return infllmv2_attn_with_kvcache(q, cache.k, cache.v, k=k_new, v=v_new, cache_seqlens=lens,
                                           softmax_scale=self.softmax_scale, topk_idx=topk_idx)
+
+    # ---- batched decode ----
+    def fill_cache(self, cache: BatchCache, k, v, seqlens):
+        """Stores packed keys/values ``(total, nheads_k, d)`` of ``len(seqlens)`` sequences (host list of lengths) in
+        ``cache`` and builds their compressed keys, as after a prefill."""
+        if len(seqlens) != cache.k.shape[0]:
+            raise RuntimeError("one length per cached sequence")
+        start = 0
+        for b, n in enumerate(seqlens):
+            cache.k[b, :n], cache.v[b, :n] = k[start:start + n].detach(), v[start:start + n].detach()
+            start += n
+        cache.lengths.copy_(torch.tensor(list(seqlens), dtype=torch.int32))
+        cache.max_length = max(seqlens)
+        for buf, lens, ks, st in ((cache.k_fine, cache.fine_lens, self.kernel_size, self.stride),
+                                  (cache.k_coarse, cache.coarse_lens, 4 * self.kernel_size, 4 * self.stride)):
+            compress_keys_cache(cache.k, cache.lengths, ks, st, out=buf, out_lens=lens)
+
+    def decode_batch(self, q, k_new, v_new, cache: BatchCache):
+        """One token for every sequence of the batch: q ``(batch, 1, nheads, d)``, k_new/v_new
+        ``(batch, 1, nheads_k, d)``.  Per sequence exactly what :meth:`decode` does, in a fixed number of launches
+        for the whole batch and without reading anything back to the host: append, extend the compressed keys where a
+        window completes, Stage 1 over each sequence's compressed-key cache, pooling at the sequence's own position,
+        top-k, split decode attention.  Returns ``(batch, 1, nheads, d)``."""
+        batch = q.shape[0]
+        if cache.max_length + 1 > cache.k.shape[1]:
+            raise RuntimeError("the K/V cache is full")
+        old = cache.lengths
+        new = old + 1
+        # the selection needs the new key inside the compressed keys; the decode kernel's own append rewrites the row
+        cache.k[torch.arange(batch, device=q.device), old.long()] = k_new[:, 0]
+        for buf, lens, ks, st in ((cache.k_fine, cache.fine_lens, self.kernel_size, self.stride),
+                                  (cache.k_coarse, cache.coarse_lens, 4 * self.kernel_size, 4 * self.stride)):
+            compress_keys_cache(cache.k, new, ks, st, out=buf, old_lens=old, max_new_rows=1, out_lens=lens)
+        topk_idx = None
+        if cache.max_length + 1 > self.dense_len:
+            pooled = infllmv2_attn_stage1_kvcache(q, cache.k_fine, cache.k_coarse, cache.fine_lens, cache.coarse_lens,
+                                                  old, self.local_blocks, self.init_blocks,
+                                                  max_cache_len=cache.max_length, block_size=self.block_size,
+                                                  stride=self.stride, softmax_scale=self.softmax_scale, causal=False)
+            topk_idx = topk_blocks(pooled, self.topk).unsqueeze(2)                   # (batch, Hk, 1, topk)
+        out = infllmv2_attn_with_kvcache(q, cache.k, cache.v, k=k_new, v=v_new, cache_seqlens=old,
+                                         softmax_scale=self.softmax_scale, topk_idx=topk_idx)
+        cache.lengths = new
+        cache.max_length += 1
+        return out

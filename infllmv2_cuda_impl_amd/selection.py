@@ -64,6 +64,39 @@ def compress_keys(k: torch.Tensor, cu_seqlens_k: torch.Tensor, max_seqlen_k: int
     return out, cu_out
 
 
+def compress_keys_cache(k_cache: torch.Tensor, new_lens: torch.Tensor, kernel_size: int, stride: int, out: torch.Tensor,
+                        old_lens: torch.Tensor | None = None, max_new_rows: int | None = None,
+                        out_lens: torch.Tensor | None = None):
+    """Compressed keys of per-sequence key caches, as a batched decode loop keeps them: ``k_cache``
+    ``(batch, capacity, nheads_k, d)`` holds ``new_lens[b]`` keys of sequence b; rows of ``out``
+    ``(batch, rows, nheads_k, d)`` whose windows were completed since ``old_lens[b]`` tokens (``None``: all of them)
+    are written in place.  ``max_new_rows`` bounds the new rows per sequence (default: every row of ``out``; 1 suffices
+    for a one-token step).  Returns ``out_lens`` int32 ``(batch,)``: the rows each compressed cache now holds."""
+    require_gpu(k_cache, "k_cache")
+    if k_cache.dtype != torch.bfloat16 or out.dtype != torch.bfloat16:
+        raise RuntimeError("this build only has bf16 kernels")
+    if k_cache.dim() != 4 or out.dim() != 4 or k_cache.stride(-1) != 1 or out.stride(-1) != 1 or \
+            out.shape[0] != k_cache.shape[0] or tuple(out.shape[2:]) != tuple(k_cache.shape[2:]):
+        raise RuntimeError("k_cache and out must have shapes (batch, capacity, num_heads_k, head_size) and "
+                           "(batch, rows, num_heads_k, head_size)")
+    batch, cap, Hk, d = k_cache.shape
+    for name, t in (("new_lens", new_lens), ("old_lens", old_lens)):
+        if t is not None and (t.dtype != torch.int32 or tuple(t.shape) != (batch,) or not t.is_contiguous()):
+            raise RuntimeError(f"{name} must be a contiguous int32 tensor of shape (batch_size)")
+    if (cap - kernel_size) // stride + 1 > out.shape[1] and max_new_rows is None:
+        raise RuntimeError("out has fewer rows than the key cache has windows")
+    if max_new_rows is None:
+        max_new_rows = out.shape[1]
+    if out_lens is None:
+        out_lens = torch.empty(batch, dtype=torch.int32, device=k_cache.device)
+    s3 = lambda t: _lib.i64_array([t.stride(0), t.stride(1), t.stride(2)])
+    with torch.cuda.device(k_cache.device):
+        _lib.call("infllmv2_compress_keys_cache", stream_ptr(k_cache.device), k_cache.data_ptr(), out.data_ptr(),
+                  None if old_lens is None else old_lens.data_ptr(), new_lens.data_ptr(), out_lens.data_ptr(), batch,
+                  int(max_new_rows), Hk, d, s3(k_cache), s3(out), kernel_size, stride)
+    return out_lens
+
+
 def select_blocks(q: torch.Tensor, k: torch.Tensor, cu_seqlens_q: torch.Tensor, cu_seqlens_k: torch.Tensor,
                   max_seqlen_q: int, max_seqlen_k: int, topk: int, local_blocks: int, init_blocks: int,
                   cache_lens: torch.Tensor | None = None, max_cache_len: int | None = None, softmax_scale=None,

@@ -183,6 +183,88 @@ def test_config5_decode_batch64(ops):
     assert float((out.float() - out1.float()).abs().max()) <= 8e-3
 
 
+def test_config5_decode_batch64_selection_leg(ops):
+    """BASELINE config 5 end to end: batch 64, one query per sequence, K/V cache lengths drawn from multiples of 64 in
+    [16384, 131072]: compressed-key caches -> Stage 1 (decode-shaped launch) -> pooling at each sequence's own
+    position -> top-k -> mask -> split decode attention.  Stage-1 scores of sampled sequences against the oracle
+    (Stage-1 tolerance); pooled / top-k / mask bit-exact functions of the GPU scores; the fused pooled launch equals
+    pooling of the score launch for every sequence; the attention output of sampled sequences against the oracle's
+    decode on the selected blocks, and against the prefill kernels run on the sampled sequence's last token."""
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(5)
+    B, topk, local, init = 64, 64, 31, 1
+    lens = [int(64 * x) for x in rng.integers(256, 2049, size=B)]        # tokens per sequence, the new one included
+    lens[3], lens[40] = 131072, 16384                                     # both ends of the range are present
+    cap = max(lens)
+    g = torch.Generator(device="cuda").manual_seed(0)
+    q = torch.randn(B, 1, 32, 128, generator=g, device=dev).to(torch.bfloat16)
+    kc = torch.randn(B, cap, 2, 128, generator=g, device=dev).to(torch.bfloat16)
+    vc = torch.randn(B, cap, 2, 128, generator=g, device=dev).to(torch.bfloat16)
+    L = torch.tensor(lens, dtype=torch.int32, device=dev)
+    pos = L - 1                                                           # position of each sequence's query
+    fine = torch.empty(B, cap // 16 + 1, 2, 128, dtype=torch.bfloat16, device=dev)
+    coarse = torch.empty(B, cap // 64 + 1, 2, 128, dtype=torch.bfloat16, device=dev)
+    fl = ops.compress_keys_cache(kc, L, 32, 16, out=fine)
+    cl = ops.compress_keys_cache(kc, L, 128, 64, out=coarse)
+    assert fl.tolist() == [(n - 32) // 16 + 1 for n in lens] and cl.tolist() == [(n - 128) // 64 + 1 for n in lens]
+    score = ops.infllmv2_attn_stage1_kvcache(q, fine, coarse, fl, cl, pos, local, init, causal=False, pooled=False)
+    pooled = ops.infllmv2_attn_stage1_kvcache(q, fine, coarse, fl, cl, pos, local, init, max_cache_len=cap - 1,
+                                              causal=False)
+    nblk = cap // 64
+    assert tuple(pooled.shape) == (B, 2, nblk)
+    idx = ops.topk_blocks(pooled, topk)                                   # (B, Hk, topk)
+    words, _ = ops.topk_to_uint64(idx.unsqueeze(2), cap, 64)
+    # pooled == pooling of the score rows, all sequences (GPU pooling operator on the packed equivalent)
+    cu_q = torch.arange(B + 1, dtype=torch.int32, device=dev)
+    rows_f = fine.shape[1]
+    cu_rows = torch.arange(B + 1, dtype=torch.int32, device=dev) * rows_f
+    for b in (0, 3, 40, 63):
+        one = lambda n: torch.tensor([0, n], dtype=torch.int32, device=dev)
+        two_calls = ops.max_pooling_1d_varlen(score[b][:, None, :int(fl[b])].contiguous(), one(1), one(int(fl[b])),
+                                              pos[b:b + 1].contiguous(), 1, int(fl[b]), local, init, max_cache_len=cap - 1)
+        assert torch.equal(two_calls[:, 0].view(torch.int16), pooled[b].view(torch.int16))
+    for b in (3, 17, 40):
+        n, Lf, Lc = lens[b], int(fl[b]), int(cl[b])
+        got = bf16_np(score[b])                                           # (Hk, rows)
+        assert np.all(got[:, Lf:] == 0)
+        qq = bf16_np(q[b, 0]).reshape(2, 16, 128).astype(np.float64)
+        # compressed keys themselves: bit-exact windowed means of the cache
+        assert torch.equal(fine[b, :Lf], compress(kc[b, :n], 32, 16)) or \
+            float((fine[b, :Lf].float() - compress(kc[b, :n], 32, 16).float()).abs().max()) <= 2.0 ** -8 * 4
+        kf_np, kc_np = bf16_np(fine[b, :Lf]).astype(np.float64), bf16_np(coarse[b, :Lc]).astype(np.float64)
+        for h in range(2):
+            sc_c = qq[h] @ kc_np[:, h].T * 128 ** -0.5
+            mx = sc_c.max(-1, keepdims=True)
+            lse = np.log(np.exp(sc_c - mx).sum(-1, keepdims=True)) + mx
+            ref = np.exp(qq[h] @ kf_np[:, h].T * 128 ** -0.5 - lse).sum(0)
+            assert (np.abs(got[h, :Lf] - ref) <= 2.0 ** -7 * np.abs(ref) + 2e-3).all()
+        # pooled / top-k / mask from the GPU scores by the oracle
+        want_pool = O.max_pooling_1d_fast(got[:, None, :Lf], nblk, local, init, row_cache_lens=np.array([n - 1]),
+                                          row_qidx=np.array([0]), row_klen=np.array([Lf]))
+        assert np.array_equal(bf16_np(pooled[b])[:, None], want_pool)
+        want_idx = O.topk_blocks(want_pool, topk)
+        assert np.array_equal(idx[b].cpu().numpy()[:, None], want_idx)
+        assert np.array_equal(words_np(words[b]), O.topk_to_uint64(want_idx, cap, 64)[0])
+        sel = set(want_idx[0, 0].tolist())
+        bq = (n - 1) // 64
+        assert 0 in sel and all(bq - d in sel for d in range(32)) and max(sel) <= bq
+    # Stage 2 on the selected blocks
+    out, lse = ops.infllmv2_attn_with_kvcache(q, kc, vc, cache_seqlens=L, topk_idx=idx.unsqueeze(2), return_softmax_lse=True)
+    for b in (3, 17, 40):
+        n = lens[b]
+        w = O.topk_to_uint64(idx[b:b + 1].unsqueeze(2).cpu().numpy(), cap, 64)[0]
+        ro, rl = O.decode_forward(bf16_np(q[b:b + 1]), bf16_np(kc[b:b + 1, :n]), bf16_np(vc[b:b + 1, :n]), [n], w, 128 ** -0.5)
+        err = np.abs(bf16_np(out[b:b + 1]) - ro)
+        assert err.max() <= 2e-2 and err.mean() <= 1e-3
+        assert np.abs(lse[b:b + 1].cpu().numpy() - rl).max() <= 2e-3
+        # the prefill kernels on the same sequence's last token with the same selection
+        one = lambda m: torch.tensor([0, m], dtype=torch.int32, device=dev)
+        pre = ops.infllmv2_attn_varlen_func(q[b], kc[b, :n], vc[b, :n], one(1), one(n), 1, n, causal=True,
+                                            topk_idx=idx[b][:, None, :].contiguous())
+        e2 = (pre.float() - out[b].float()).abs()
+        assert float(e2.max()) <= 2e-2 and float(e2.mean()) <= 1e-3
+
+
 def test_config4_prefill_128k_fused_front_end(ops):
     """BASELINE config 4 (131072 tokens): the one-call selection, which never writes the 4.3 GB score tensor, against
     the separate calls (bit-exact pooled scores and identical top-k), selection invariants over all rows, and the

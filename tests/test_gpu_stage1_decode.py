@@ -1,0 +1,189 @@
+"""GPU parity of Stage 1 with one query per sequence (the selection half of a batched decode step).
+
+Scores against the CPU oracle to the Stage-1 tolerance (|got - ref| <= 2^-7 |ref| + 2e-3); the pooled output bit for
+bit against pooling the same launch's score rows (max_pooling_1d_varlen on the GPU and the oracle's pooling on the CPU:
+one differing bit could change a selection); packed keys and per-sequence key caches give the same bits; the
+batched decode step of the layer reproduces the single-sequence decode loop.  The reference covers this case with
+its varlen Stage 1 on cu_seqlens_q = 0, 1, 2, ... and tests/test_cache_lens.py:4-98 (per-sequence cache_lens)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import infllmv2_oracle as O
+from conftest import bf16_np
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import infllmv2_cuda_impl_amd as ops
+    return ops
+
+
+def to_dev(a, dt=None):
+    t = torch.from_numpy(np.ascontiguousarray(a))
+    return (t if dt is None else t.to(dt)).to(DEV)
+
+
+def same_bits(a, b):
+    return torch.equal(a.contiguous().view(torch.int16), b.contiguous().view(torch.int16))
+
+
+def close(got, ref):
+    err = np.abs(got - ref)
+    tol = 2.0 ** -7 * np.abs(ref) + 2e-3
+    assert (err <= tol).all(), (err.max(), np.unravel_index(np.argmax(err - tol), err.shape))
+
+
+def batch_inputs(seed, lens, Hk=2, exact=False):
+    """One query per sequence; the sequences' keys packed; compressed keys by the oracle."""
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    B = len(lens)
+    q = torch.randn(B, 16 * Hk, 128, generator=g).to(torch.bfloat16)
+    k = torch.randn(sum(lens), Hk, 128, generator=g).to(torch.bfloat16)
+    cu = np.cumsum([0] + list(lens)).astype(np.int32)
+    kf, cu_f = O.compress_keys(bf16_np(k), cu, 32, 16)
+    kc, cu_c = (kf, cu_f) if exact else O.compress_keys(bf16_np(k), cu, 128, 64)
+    return q, k, cu, kf, cu_f, kc, cu_c
+
+
+@pytest.mark.parametrize("lens,causal,exact", [
+    ([1000, 40, 3000, 128, 129, 31, 2047], False, False),     # no fine key, no coarse key, one coarse key, ...
+    ([1000, 40, 3000, 128, 129, 31, 2047], True, False),      # causal rule of a 1-token query: the last key of each set hidden
+    ([20000], False, False),                                   # one sequence: many runs per (sequence, head)
+    ([5000, 700], False, True),                                # exact softmax: the log-sum-exp over the fine keys themselves
+    ([64 * 17 + 5] * 40, False, False),                       # more (sequence, head) pairs than runs wanted: short runs
+])
+def test_scores_pooled_and_layouts(ops, lens, causal, exact):
+    q, k, cu, kf, cu_f, kc, cu_c = batch_inputs(1, lens, exact=exact)
+    B = len(lens)
+    Lk = int(np.diff(cu_f).max())
+    cu_q = np.arange(B + 1, dtype=np.int32)
+    qd, kfd, kcd = q.to(DEV), to_dev(kf, torch.bfloat16), to_dev(kc, torch.bfloat16)
+    args = (qd, kfd, kcd, to_dev(cu_q), to_dev(cu_f), to_dev(cu_c), 1, Lk)
+    score = ops.infllmv2_attn_stage1(*args, causal=causal)
+    assert tuple(score.shape) == (2, B, Lk) and score.dtype == torch.bfloat16
+    ref = O.stage1_scores(bf16_np(q), kf, kc, cu_q, cu_f, cu_c, Lk, 128 ** -0.5, causal, round_output=False)
+    close(bf16_np(score), ref)
+    # pooled: the query of sequence b sits at position lens[b] - 1 (its cache holds the tokens before it)
+    cache_lens = np.array([n - 1 for n in lens], dtype=np.int32)
+    for local, init in ((1, 1), (31, 1), (0, 0)):
+        fused = ops.infllmv2_attn_stage1_pooled(*args, local, init, cache_lens=to_dev(cache_lens), causal=causal)
+        two_calls = ops.max_pooling_1d_varlen(score, to_dev(cu_q), to_dev(cu_f), to_dev(cache_lens), 1, Lk, local, init)
+        assert tuple(fused.shape) == tuple(two_calls.shape) == (2, B, (max(lens) + 63) // 64)
+        assert same_bits(fused, two_calls)
+        want = O.max_pooling_1d_varlen(bf16_np(score), cu_q, cu_f, cache_lens, 1, Lk, local, init)
+        assert np.array_equal(bf16_np(fused), want)
+    # per-sequence compressed-key caches instead of packed keys: same bits
+    rows_f = Lk + 3
+    rows_c = int(np.diff(cu_c).max()) + 2
+    fcache = torch.randn(B, rows_f, 2, 128).to(torch.bfloat16)          # stale rows beyond each sequence's keys
+    ccache = torch.randn(B, rows_c, 2, 128).to(torch.bfloat16)
+    for b in range(B):
+        fcache[b, :cu_f[b + 1] - cu_f[b]] = torch.from_numpy(kf[cu_f[b]:cu_f[b + 1]]).to(torch.bfloat16)
+        ccache[b, :cu_c[b + 1] - cu_c[b]] = torch.from_numpy(kc[cu_c[b]:cu_c[b + 1]]).to(torch.bfloat16)
+    fl, cl = to_dev(np.diff(cu_f).astype(np.int32)), to_dev(np.diff(cu_c).astype(np.int32))
+    if not exact:
+        q4 = qd[:, None]
+        sc2 = ops.infllmv2_attn_stage1_kvcache(q4, fcache.to(DEV), ccache.to(DEV), fl, cl, to_dev(cache_lens), 1, 1,
+                                               causal=causal, pooled=False)
+        assert same_bits(sc2[:, :, :Lk].transpose(0, 1), score)
+        assert float(sc2[:, :, Lk:].abs().max()) == 0.0
+        p2 = ops.infllmv2_attn_stage1_kvcache(q4, fcache.to(DEV), ccache.to(DEV), fl, cl, to_dev(cache_lens), 1, 1,
+                                              max_cache_len=max(lens) - 1, causal=causal)
+        fused = ops.infllmv2_attn_stage1_pooled(*args, 1, 1, cache_lens=to_dev(cache_lens), causal=causal)
+        assert same_bits(p2.transpose(0, 1), fused)
+
+
+def test_decode_kernel_agrees_with_the_prefill_shaped_kernel(ops):
+    """The generic Stage-1 launch (C ABI infllmv2_varlen_fwd_stage1) on the same one-query sequences: different kernel,
+    different summation order of the log-sum-exp, same scores to the Stage-1 tolerance."""
+    from infllmv2_cuda_impl_amd import _lib
+    lens = [3000, 500, 64 * 40]
+    q, k, cu, kf, cu_f, kc, cu_c = batch_inputs(4, lens)
+    B, Lk = len(lens), int(np.diff(cu_f).max())
+    cu_q = to_dev(np.arange(B + 1, dtype=np.int32))
+    qd, kfd, kcd, cfd, ccd = q.to(DEV), to_dev(kf, torch.bfloat16), to_dev(kc, torch.bfloat16), to_dev(cu_f), to_dev(cu_c)
+    for causal in (False, True):
+        fast = ops.infllmv2_attn_stage1(qd, kfd, kcd, cu_q, cfd, ccd, 1, Lk, causal=causal)
+        slow = torch.empty_like(fast)
+        _lib.call("infllmv2_varlen_fwd_stage1", torch.cuda.current_stream().cuda_stream, qd.data_ptr(), kfd.data_ptr(),
+                  kcd.data_ptr(), slow.data_ptr(), cu_q.data_ptr(), cfd.data_ptr(), ccd.data_ptr(), B, B, 32, 2, 128, 1, Lk,
+                  _lib.i64_array([qd.stride(0), qd.stride(1), 16 * qd.stride(1)]),
+                  _lib.i64_array([kfd.stride(0), kfd.stride(1)]), _lib.i64_array([kcd.stride(0), kcd.stride(1)]),
+                  slow.stride(0), slow.stride(1), 128 ** -0.5, int(causal))
+        close(bf16_np(fast), bf16_np(slow).astype(np.float64))
+
+
+def test_compressed_key_caches_follow_the_key_caches(ops):
+    """compress_keys_cache == compress_keys of each sequence; a one-token step adds exactly the rows whose window the
+    new token completes and touches nothing else."""
+    lens = [100, 31, 32, 127, 128, 1000, 47]
+    B, cap = len(lens), 1100
+    g = torch.Generator(device="cpu").manual_seed(5)
+    kcache = torch.randn(B, cap, 2, 128, generator=g).to(torch.bfloat16).to(DEV)
+    L = torch.tensor(lens, dtype=torch.int32, device=DEV)
+    for ks, st in ((32, 16), (128, 64)):
+        out = torch.full((B, cap // st + 1, 2, 128), 7.0, dtype=torch.bfloat16, device=DEV)
+        rows = ops.compress_keys_cache(kcache, L, ks, st, out=out)
+        for b, n in enumerate(lens):
+            one = torch.tensor([0, n], dtype=torch.int32, device=DEV)
+            ref, _ = ops.compress_keys(kcache[b, :n], one, n, ks, st)
+            r = ref.shape[0]
+            assert int(rows[b]) == r == O.compressed_len(n, ks, st)
+            assert torch.equal(out[b, :r], ref) and bool((out[b, r:] == 7.0).all())
+        for step in range(1, 20):                              # one token at a time
+            new = L + step
+            rows2 = ops.compress_keys_cache(kcache, new, ks, st, out=out, old_lens=new - 1, max_new_rows=1)
+            for b, n in enumerate(lens):
+                r = O.compressed_len(n + step, ks, st)
+                assert int(rows2[b]) == r
+                if r:
+                    ref, _ = ops.compress_keys(kcache[b, :n + step], torch.tensor([0, n + step], dtype=torch.int32, device=DEV),
+                                               n + step, ks, st)
+                    assert torch.equal(out[b, :r], ref)
+                assert bool((out[b, r:] == 7.0).all())
+
+
+def test_batched_decode_steps_equal_single_sequence_decode(ops):
+    """decode_batch on sequences of different lengths == the single-sequence decode loop run on each of them: same
+    caches afterwards (bit for bit), outputs to the Stage-2 tolerance (the two paths cut the compressed keys into
+    different runs, so a score can differ in its last bit and tip a tie between two barely-selected blocks)."""
+    lens, steps, cap = [1000, 300, 2047, 130], 20, 2200
+    B = len(lens)
+    g = torch.Generator(device="cpu").manual_seed(6)
+    mk = lambda n, h: torch.randn(n, h, 128, generator=g).to(torch.bfloat16).to(DEV)
+    total = [n + steps for n in lens]
+    qs, ks, vs = [mk(n, 32) for n in total], [mk(n, 2) for n in total], [mk(n, 2) for n in total]
+    layer = ops.InfLLMv2Attention(topk=8, local_blocks=2, init_blocks=1)
+    singles = []
+    for b in range(B):
+        c = ops.SequenceCache.empty(cap, 2, 128, DEV)
+        n = lens[b]
+        layer(qs[b][:n], ks[b][:n], vs[b][:n], torch.tensor([0, n], dtype=torch.int32, device=DEV), n, cache=c)
+        singles.append(c)
+    cache = ops.BatchCache.empty(B, cap, 2, 128, DEV)
+    layer.fill_cache(cache, torch.cat([ks[b][:lens[b]] for b in range(B)]), torch.cat([vs[b][:lens[b]] for b in range(B)]), lens)
+    for b in range(B):
+        assert torch.equal(cache.k_fine[b, :int(cache.fine_lens[b])], singles[b].k_fine[:int(cache.fine_lens[b])])
+    for s in range(steps):
+        q = torch.stack([qs[b][lens[b] + s] for b in range(B)])[:, None]
+        kn = torch.stack([ks[b][lens[b] + s] for b in range(B)])[:, None]
+        vn = torch.stack([vs[b][lens[b] + s] for b in range(B)])[:, None]
+        out = layer.decode_batch(q, kn, vn, cache)
+        assert tuple(out.shape) == (B, 1, 32, 128)
+        for b in range(B):
+            ref = layer.decode(q[b:b + 1], kn[b:b + 1], vn[b:b + 1], singles[b])
+            err = (out[b].float() - ref[0].float()).abs()
+            assert float(err.max()) <= 2e-2 and float(err.mean()) <= 1e-3, (s, b, float(err.max()))
+    assert cache.max_length == max(lens) + steps
+    assert cache.lengths.tolist() == total
+    for b in range(B):
+        n = total[b]
+        assert torch.equal(cache.k[b, :n], singles[b].k[0, :n]) and torch.equal(cache.v[b, :n], singles[b].v[0, :n])
+        rf, rc = O.compressed_len(n, 32, 16), O.compressed_len(n, 128, 64)
+        assert int(cache.fine_lens[b]) == rf and int(cache.coarse_lens[b]) == rc
+        assert torch.equal(cache.k_fine[b, :rf], singles[b].k_fine[:rf])
+        assert torch.equal(cache.k_coarse[b, :rc], singles[b].k_coarse[:rc])
