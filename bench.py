@@ -11,13 +11,17 @@ Inputs (q, k, v and the caller-side compressed keys) are resident in HBM before 
 `value` = Stage-2 algorithmic sparse FLOPs (4*16*64*128 per selected causal block per token and KV head)
 divided by the time of the WHOLE step, in TFLOP/s.  The JSON line also carries the per-stage times, the
 Stage-2 forward kernel's own roofline figures (HIP events around the kernel alone, K/V images
-prepacked) and the CPU oracle timed on BASELINE config 1.
+prepacked), forward + backward, the other BASELINE configurations as extra keys (config 3: four packed sequences
+forward + backward; config 4: 131072 tokens per stage; config 5: batched decode, selection and attention), a measured
+device-copy bandwidth and the CPU oracle timed per stage on BASELINE config 1.
 """
 from __future__ import annotations
 
 import argparse
+import hashlib
 import json
 import os
+import re
 import sys
 import time
 
@@ -25,12 +29,40 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-# HBM bytes per launch of the dominant kernel at the default workload: 2.00 x FETCH_SIZE + 1.00 x WRITE_SIZE of the two
-# rocprofv3 --pmc runs summarised in profiles/stage2_fwd_config2_hbm_traffic.md (counters cannot be read from inside
-# this process); null for any other workload
-MEASURED_FWD_TRAFFIC_BYTES = 5.86e9
 PEAK_BF16_TFLOPS = 2500.0      # MI355X dense bf16 MFMA peak (vendor figure, no sparsity)
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E peak
+FLOPS_PER_BLOCK = 4 * 16 * 64 * 128
+
+# the Stage-2 forward kernel's HBM traffic cannot be read from inside this process (rocprofv3 --pmc counters); it is
+# taken from the tracked summary below, which names the sources it was measured on by their hash
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "stage2_fwd_config2_hbm_traffic.md")
+FWD_KERNEL_SOURCES = ["stage2_fwd_hybrid.hip", "stage2_fwd.hip", "stage2_fwd.h", "kv_image.h", "block_walker.h", "common.h"]
+
+
+def fwd_kernel_source_hash() -> str:
+    h = hashlib.sha256()
+    for name in FWD_KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "infllmv2_cuda_impl_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def profiled_traffic_bytes(seqlen: int, topk: int):
+    """HBM bytes per launch of the Stage-2 forward kernel from the tracked rocprofv3 summary, or None when the summary
+    was measured on other kernel sources or another workload."""
+    try:
+        text = open(TRAFFIC_PROFILE).read()
+    except OSError:
+        return None
+    fields = dict(re.findall(r"^(kernel_source_hash|traffic_bytes_per_launch|seqlen|topk):\s*(\S+)\s*$", text, re.M))
+    if fields.get("kernel_source_hash") != fwd_kernel_source_hash():
+        return None
+    if fields.get("seqlen") != str(seqlen) or fields.get("topk") != str(topk):
+        return None
+    try:
+        return float(fields["traffic_bytes_per_launch"])
+    except (KeyError, ValueError):
+        return None
 
 
 def parse_args():
@@ -47,8 +79,12 @@ def parse_args():
     ap.add_argument("--no-shared-selection", action="store_true",
                     help="skip the extra leg with selections shared inside each query block (keeps a profile of the "
                          "Stage-2 kernel to one workload)")
-    ap.add_argument("--calibrate-copy", action="store_true",
-                    help="also run three plain 1 GiB device copies (a kernel of known traffic for scaling rocprofv3 --pmc counters)")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="skip BASELINE configs 3, 4 and 5 (keeps a profile to the default workload)")
+    ap.add_argument("--only-config", type=int, default=0, choices=[0, 3, 4, 5],
+                    help="run one of the extra configurations alone (for profiling it) and print its record")
+    ap.add_argument("--print-source-hash", action="store_true",
+                    help="print the hash of the Stage-2 forward kernel sources (what a traffic summary must name) and exit")
     return ap.parse_args()
 
 
@@ -77,35 +113,165 @@ def event_ms(torch, fn, iters, warmup=2):
     return e0.elapsed_time(e1) / iters
 
 
-def decode_bench(torch, ops, dev):
-    """BASELINE config 5: batch 64, one query token, cache lengths 64*U[256,2048], topk 64 (1 init + 32 local forced)."""
+def selected_causal_blocks(torch, ops, idx, cu_lens, max_len, dev):
+    """Number of (token, KV head, block) triples the Stage-2 kernels work on: set bits of the mask at or below each
+    token's own block."""
+    words, _ = ops.topk_to_uint64(idx, max_len, 64)
+    nblk = (max_len + 63) // 64
+    bits = ops.uint64_to_bool(words, nblk)
+    total = 0
+    start = 0
+    for n in cu_lens:
+        tok = torch.arange(n, device=dev)
+        causal_blk = torch.arange(nblk, device=dev)[None, :] <= (tok // 64)[:, None]
+        total += int((bits[:, start:start + n] & causal_blk[None]).sum())
+        start += n
+    return total
+
+
+def copy_bandwidth(torch, dev):
+    """A plain device copy of 1 GiB (read + write = 2 GiB of traffic): the practical ceiling for the HBM-bound kernels."""
+    src = torch.ones(1 << 30, dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    ms = event_ms(torch, lambda: dst.copy_(src), 10)
+    return {"gbs": 2 * src.numel() / ms / 1e6, "ms": ms, "what": "torch copy_ of 1 GiB, read + write bytes"}
+
+
+def config3_bench(torch, ops, dev):
+    """BASELINE config 3: four packed sequences, lengths 64*U[64,384] (seeded), forward + backward, topk 64."""
     import numpy as np
     rng = np.random.default_rng(1)
-    B = 64
-    lens = [int(64 * x) for x in rng.integers(256, 2049, size=B)]
+    lens = [int(64 * x) for x in rng.integers(64, 385, size=4)]
+    T, mx = sum(lens), max(lens)
+    cu = torch.tensor(np.cumsum([0] + lens), dtype=torch.int32, device=dev)
+    g = torch.Generator(device="cuda").manual_seed(3)
+    mkt = lambda h: torch.randn(T, h, 128, generator=g, device=dev).to(torch.bfloat16)
+    q, k, v, dout = mkt(32), mkt(2), mkt(2), mkt(32)
+    zeros = torch.zeros(4, dtype=torch.int32, device=dev)
+    sel = lambda: ops.select_blocks(q, k, cu, cu, mx, mx, 64, 31, 1, cache_lens=zeros, max_cache_len=0)
+    idx = sel()
+    nsel = selected_causal_blocks(torch, ops, idx, lens, mx, dev)
+    flops = FLOPS_PER_BLOCK * nsel
+    sel_ms = event_ms(torch, sel, 5)
+    fwd_ms = event_ms(torch, lambda: ops.infllmv2_attn_varlen_func(q, k, v, cu, cu, mx, mx, causal=True, topk_idx=idx), 5)
+    qg, kg, vg = [t.clone().requires_grad_(True) for t in (q, k, v)]
+
+    def fwd_bwd():
+        ops.infllmv2_attn_varlen_func(qg, kg, vg, cu, cu, mx, mx, causal=True, topk_idx=idx).backward(dout)
+        qg.grad = kg.grad = vg.grad = None
+    fb_ms = event_ms(torch, fwd_bwd, 3)
+    return {"workload": f"BASELINE config 3: 4 packed sequences {lens} = {T} tokens, GQA 32q/2kv, d=128, block 64, topk=64, "
+                        "causal; selection (compress + fused Stage-1/pool + top-k) timed apart from Stage 2",
+            "tokens": T, "selected_causal_blocks_per_token_head": nsel / (2 * T), "selection_ms": sel_ms,
+            "stage2_fwd_ms": fwd_ms, "stage2_fwd_tflops": flops / fwd_ms / 1e9,
+            "stage2_fwd_frac_peak": flops / fwd_ms / 1e9 / PEAK_BF16_TFLOPS,
+            "stage2_fwd_bwd_ms": fb_ms, "stage2_fwd_bwd_tflops": 3.5 * flops / fb_ms / 1e9,
+            "stage2_fwd_bwd_frac_peak": 3.5 * flops / fb_ms / 1e9 / PEAK_BF16_TFLOPS}
+
+
+def config4_bench(torch, ops, dev):
+    """BASELINE config 4: one sequence of 131072 tokens, forward, per stage."""
+    S, topk = 131072, 64
+    g = torch.Generator(device="cuda").manual_seed(4)
+    mkt = lambda h: torch.randn(S, h, 128, generator=g, device=dev).to(torch.bfloat16)
+    q, k, v = mkt(32), mkt(2), mkt(2)
+    cu = torch.tensor([0, S], dtype=torch.int32, device=dev)
+    kf, cu_f = ops.compress_keys(k, cu, S, 32, 16)
+    kc, cu_c = ops.compress_keys(k, cu, S, 128, 64)
+    Lk, nblk = kf.shape[0], S // 64
+    s1 = lambda: ops.infllmv2_attn_stage1_pooled(q, kf, kc, cu, cu_f, cu_c, S, Lk, 31, 1, causal=True)
+    pooled = s1()
+    idx = ops.topk_blocks(pooled, topk)
+    nsel = selected_causal_blocks(torch, ops, idx, [S], S, dev)
+    flops = FLOPS_PER_BLOCK * nsel
+    s1_flops = 2 * 16 * 128 * 2 * sum(max(0, (t + 1) // 16 - 1) + max(0, (t + 1) // 64 - 1) for t in range(S))
+    ms = {
+        "compress_keys": event_ms(torch, lambda: (ops.compress_keys(k, cu, S, 32, 16), ops.compress_keys(k, cu, S, 128, 64)), 5),
+        "stage1_pooled_fused": event_ms(torch, s1, 3),
+        "topk": event_ms(torch, lambda: ops.topk_blocks(pooled, topk), 5),
+        "pack_mask": event_ms(torch, lambda: ops.topk_to_uint64(idx, S, 64), 5),
+        "stage2_fwd_op": event_ms(torch, lambda: ops.infllmv2_attn_varlen_func(q, k, v, cu, cu, S, S, causal=True, topk_idx=idx), 3),
+    }
+
+    def step():
+        p = s1()
+        i = ops.topk_blocks(p, topk)
+        return ops.infllmv2_attn_varlen_func(q, k, v, cu, cu, S, S, causal=True, topk_idx=i)
+    step_ms = event_ms(torch, step, 3, warmup=1)
+    n64 = (nblk + 63) // 64
+    return {"workload": f"BASELINE config 4: prefill forward, 1 x {S} tokens, GQA 32q/2kv, d=128, block 64, topk={topk}, "
+                        "causal; fused Stage-1/pool + top-k + pack + Stage-2 fwd",
+            "selected_causal_blocks_per_token_head": nsel / (2 * S), "stages_ms": ms, "ms_per_step": step_ms,
+            "tflops_whole_step": flops / step_ms / 1e9, "stage2_fwd_tflops": flops / ms["stage2_fwd_op"] / 1e9,
+            "stage2_fwd_frac_peak": flops / ms["stage2_fwd_op"] / 1e9 / PEAK_BF16_TFLOPS,
+            "stage1_tflops": s1_flops / ms["stage1_pooled_fused"] / 1e9,
+            "stage1_frac_peak": s1_flops / ms["stage1_pooled_fused"] / 1e9 / PEAK_BF16_TFLOPS,
+            "stage1_topk_share_of_fwd": (ms["stage1_pooled_fused"] + ms["topk"]) / step_ms,
+            "stages_hbm_gbs": {"topk": (2 * S * nblk * 2 + 2 * S * topk * 4) / ms["topk"] / 1e6,
+                               "pack_mask": (2 * S * topk * 4 + 2 * S * n64 * 8) / ms["pack_mask"] / 1e6}}
+
+
+def decode_bench(torch, ops, dev):
+    """BASELINE config 5: batch 64, one query token per sequence, cache lengths 64*U[256,2048], topk 64 (1 init + 32
+    local forced): the selection leg (Stage 1 over each sequence's compressed-key caches, pooled at the sequence's
+    position, top-k) and the attention leg (mask packing + split decode kernel), each against the HBM roofline."""
+    import numpy as np
+    rng = np.random.default_rng(1)
+    B, topk = 64, 64
+    lens = [int(64 * x) for x in rng.integers(256, 2049, size=B)]      # tokens per sequence, the new one included
     cap = max(lens)
     g = torch.Generator(device="cuda").manual_seed(0)
     q = torch.randn(B, 1, 32, 128, generator=g, device=dev).to(torch.bfloat16)
     kc = torch.randn(B, cap, 2, 128, generator=g, device=dev).to(torch.bfloat16)
     vc = torch.randn(B, cap, 2, 128, generator=g, device=dev).to(torch.bfloat16)
-    idx = torch.full((B, 2, 1, 64), -1, dtype=torch.int32)
-    cg = torch.Generator(device="cpu").manual_seed(2)
-    for b in range(B):
-        nb = lens[b] // 64
-        for h in range(2):
-            rest = torch.arange(1, nb - 32)
-            pick = rest[torch.randperm(len(rest), generator=cg)[:31]]
-            idx[b, h, 0] = torch.cat([torch.tensor([0]), torch.arange(nb - 32, nb), pick]).sort().values.to(torch.int32)
-    idx = idx.to(dev)
     L = torch.tensor(lens, dtype=torch.int32, device=dev)
-    ms = event_ms(torch, lambda: ops.infllmv2_attn_with_kvcache(q, kc, vc, cache_seqlens=L, topk_idx=idx), 20)
-    bytes_ = B * 2 * 64 * 64 * 128 * 2 * 2 + 2 * B * 32 * 128 * 2
-    return {"ms": ms, "algorithmic_bytes": bytes_, "hbm_gbs": bytes_ / ms / 1e6, "frac_hbm_peak": bytes_ / ms / 1e6 / PEAK_HBM_GBS,
-            "workload": "BASELINE config 5: batch 64, seqlen_q 1, cache lengths 64*U[256,2048], topk 64, Stage-2 decode incl. mask packing"}
+    pos = (L - 1).contiguous()
+    fine = torch.empty(B, cap // 16 + 1, 2, 128, dtype=torch.bfloat16, device=dev)
+    coarse = torch.empty(B, cap // 64 + 1, 2, 128, dtype=torch.bfloat16, device=dev)
+    fl = ops.compress_keys_cache(kc, L, 32, 16, out=fine)
+    cl = ops.compress_keys_cache(kc, L, 128, 64, out=coarse)
+    s1 = lambda: ops.infllmv2_attn_stage1_kvcache(q, fine, coarse, fl, cl, pos, 31, 1, max_cache_len=cap - 1, causal=False)
+    pooled = s1()
+    idx = ops.topk_blocks(pooled, topk).unsqueeze(2)
+    s1_ms = event_ms(torch, s1, 20)
+    topk_ms = event_ms(torch, lambda: ops.topk_blocks(pooled, topk), 20)
+    append_ms = event_ms(torch, lambda: (ops.compress_keys_cache(kc, L, 32, 16, out=fine, old_lens=pos, max_new_rows=1),
+                                         ops.compress_keys_cache(kc, L, 128, 64, out=coarse, old_lens=pos, max_new_rows=1)), 20)
+    s2_ms = event_ms(torch, lambda: ops.infllmv2_attn_with_kvcache(q, kc, vc, cache_seqlens=L, topk_idx=idx), 20)
+
+    def step():
+        p = s1()
+        i = ops.topk_blocks(p, topk).unsqueeze(2)
+        return ops.infllmv2_attn_with_kvcache(q, kc, vc, cache_seqlens=L, topk_idx=i)
+    step_ms = event_ms(torch, step, 20)
+    s1_bytes = 2 * 128 * 2 * (int(fl.sum()) + int(cl.sum()))           # Hk * (Lk_b + Lc_b) * d * 2 bytes over the batch
+    s2_bytes = B * 2 * 64 * 64 * 128 * 2 * 2 + 2 * B * 32 * 128 * 2
+    gbs = lambda b, ms: b / ms / 1e6
+    return {"workload": "BASELINE config 5: batch 64, seqlen_q 1, cache lengths 64*U[256,2048], topk 64; Stage 1 over "
+                        "per-sequence compressed-key caches + pooling + top-k, then mask packing + Stage-2 decode",
+            "ms": s2_ms, "algorithmic_bytes": s2_bytes, "hbm_gbs": gbs(s2_bytes, s2_ms),
+            "frac_hbm_peak": gbs(s2_bytes, s2_ms) / PEAK_HBM_GBS,
+            "stage1_ms": s1_ms, "stage1_algorithmic_bytes": s1_bytes, "stage1_hbm_gbs": gbs(s1_bytes, s1_ms),
+            "stage1_frac_hbm_peak": gbs(s1_bytes, s1_ms) / PEAK_HBM_GBS,
+            "topk_ms": topk_ms, "compressed_key_append_ms": append_ms, "step_ms": step_ms,
+            "step_hbm_gbs": gbs(s1_bytes + s2_bytes, step_ms),
+            "step_frac_hbm_peak": gbs(s1_bytes + s2_bytes, step_ms) / PEAK_HBM_GBS}
 
 
-def cpu_baseline():
-    """The CPU oracle on BASELINE config 1 (2048 tokens, topk 16, block 0 + 2 local blocks forced)."""
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_baseline(runs: int = 5):
+    """The CPU oracle on BASELINE config 1 (2048 tokens, topk 16, block 0 + 2 local blocks forced), per stage and end
+    to end: one warm-up run, then the median of `runs` runs."""
     import numpy as np
     from oracle import infllmv2_oracle as O
     try:
@@ -121,28 +287,42 @@ def cpu_baseline():
     cu = np.array([0, S], np.int32)
     kf, cu_f = O.compress_keys(k, cu, 32, 16)
     kc, cu_c = O.compress_keys(k, cu, 128, 64)
-    times = []
+    stage_names = ["stage1", "pool", "topk", "pack_mask", "stage2_fwd"]
+    samples = {n: [] for n in stage_names + ["total"]}
     flops = 0
-    for _ in range(3):
-        t0 = time.perf_counter()
+    for run in range(runs + 1):
+        t = [time.perf_counter()]
         score = O.stage1_scores(q, kf, kc, cu, cu_f, cu_c, int(cu_f[-1]), 128 ** -0.5, True)
+        t.append(time.perf_counter())
         pooled = O.max_pooling_1d_fast(score, 0, 1, 1)
+        t.append(time.perf_counter())
         idx = O.topk_blocks(pooled, topk)
+        t.append(time.perf_counter())
         words, kb = O.topk_to_uint64(idx, S, 64)
+        t.append(time.perf_counter())
         O.stage2_forward(q, k, v, cu, cu, words, 128 ** -0.5, True, dtype=np.float32)
-        times.append(time.perf_counter() - t0)
-        bits = O.uint64_to_bool(words, kb)
-        causal = np.arange(kb)[None, :] <= (np.arange(S) // 64)[:, None]
-        flops = 4 * 16 * 64 * 128 * int((bits & causal[None]).sum())
-    t = sorted(times)[1]
-    return {"value": flops / t / 1e12, "unit": "TFLOP/s", "cores": int(threads), "kind": "port",
+        t.append(time.perf_counter())
+        if run == 0:                                           # warm-up: also yields the FLOP count
+            bits = O.uint64_to_bool(words, kb)
+            causal = np.arange(kb)[None, :] <= (np.arange(S) // 64)[:, None]
+            flops = FLOPS_PER_BLOCK * int((bits & causal[None]).sum())
+            continue
+        for i, n in enumerate(stage_names):
+            samples[n].append(t[i + 1] - t[i])
+        samples["total"].append(t[-1] - t[0])
+    med = {n: sorted(x)[len(x) // 2] for n, x in samples.items()}
+    return {"value": flops / med["total"] / 1e12, "unit": "TFLOP/s", "cores": int(threads), "kind": "port",
+            "cpu_model": cpu_model(), "host_cpus": os.cpu_count(),
             "sample": f"BASELINE config 1 (2048 tokens, 32q/2kv, d=128, topk=16, init 1 + 2 local blocks), whole "
-                      f"pipeline in the numpy oracle, median of 3 runs = {t:.2f} s",
-            "seconds": t}
+                      f"pipeline in the numpy oracle, 1 warm-up + median of {runs} runs = {med['total']:.2f} s",
+            "seconds": med["total"], "stage_seconds": {n: med[n] for n in stage_names}, "runs": runs}
 
 
 def main():
     args = parse_args()
+    if args.print_source_hash:
+        print(fwd_kernel_source_hash())
+        return
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU; --gpus must be 1 "
               "(the path shards by KV head or query range with no collective in the kernels; no multi-GPU figure is produced)",
@@ -153,6 +333,10 @@ def main():
     from infllmv2_cuda_impl_amd import _lib
 
     dev = torch.device("cuda:0")
+    if args.only_config:
+        fn = {3: config3_bench, 4: config4_bench, 5: decode_bench}[args.only_config]
+        print(json.dumps(fn(torch, ops, dev)))
+        return
     S, topk = args.seqlen, args.topk
     nblk = (S + 63) // 64
     local_blocks, init_blocks = 31, 1
@@ -183,16 +367,18 @@ def main():
     bits = ops.uint64_to_bool(words, nblk)
     causal_blk = torch.arange(nblk, device=dev)[None, :] <= (torch.arange(S, device=dev) // 64)[:, None]
     nsel = int((bits & causal_blk[None]).sum())
-    fwd_flops = 4 * 16 * 64 * 128 * nsel
+    fwd_flops = FLOPS_PER_BLOCK * nsel
     s1_flops = 2 * 16 * 128 * 2 * sum(max(0, (t + 1) // 16 - 1) + max(0, (t + 1) // 64 - 1) for t in range(S))
+    baseline_config = "BASELINE config 2" if (S, topk) == (32768, 64) else \
+        ("BASELINE config 4" if (S, topk) == (131072, 64) else "not a BASELINE configuration")
 
     result = {
         "metric": "sparse_attn_fwd_tflops_32k", "value": fwd_flops / ms_per_step / 1e9, "unit": "TFLOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": f"BASELINE config 2: prefill forward, 1 x {S} tokens, GQA 32q/2kv, d=128, "
+        "config": {"workload": f"{baseline_config}: prefill forward, 1 x {S} tokens, GQA 32q/2kv, d=128, "
                                f"kernel 32/stride 16 compressed keys, block 64, topk={topk} "
-                               f"(1 init + 32 local forced), causal; "
+                               f"({init_blocks} init + {local_blocks + 1} local forced), causal; "
                                + ("Stage-1 + pool" if args.unfused_front_end else "fused Stage-1/pool")
                                + " + top-k + pack + Stage-2 fwd",
                    "seqlen": S, "topk": topk, "selected_causal_blocks_per_token_head": nsel / (2 * S)},
@@ -228,6 +414,7 @@ def main():
         result["stage1_pool_topk_share_of_fwd"] = sel_ms / (sel_ms + stages["pack_mask"] + stages["stage2_fwd_op"])
         sel_ms = stages["stage1_pooled_fused"] + stages["topk"]
         result["fused_front_end_share_of_fwd"] = sel_ms / (sel_ms + stages["pack_mask"] + stages["stage2_fwd_op"])
+        del score, pooled
 
         # the dominant kernel alone: K/V images prepacked, mask packed, HIP events on the launch stream
         out_k = torch.empty_like(q)
@@ -247,7 +434,8 @@ def main():
         achieved = fwd_flops / k_ms / 1e9
         result["roofline"] = {"bound": "mfma", "kernel": "stage2_fwd_hybrid_kernel<causal>", "achieved": achieved,
                               "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS,
-                              "traffic": MEASURED_FWD_TRAFFIC_BYTES if (S, topk) == (32768, 64) else None, "kernel_ms": k_ms}
+                              "traffic": profiled_traffic_bytes(S, topk), "kernel_ms": k_ms,
+                              "kernel_source_hash": fwd_kernel_source_hash()}
         if S % 8 == 0:
             # the K/V gather bound reported beside the MFMA one: a block common to the 8 tokens of a workgroup is
             # fetched once per workgroup, every other selected block once per token, 32 KiB each, and a CU's
@@ -266,34 +454,34 @@ def main():
             sh_ms = event_ms(torch, lambda: ops.infllmv2_attn_varlen_func(q, k, v, cu_q, cu_q, S, S, causal=True,
                                                                          topk_idx=idx_shared), 10)
             sh_bits = ops.uint64_to_bool(ops.topk_to_uint64(idx_shared, S, 64)[0], nblk) & causal_blk[None]
-            sh_flops = 4 * 16 * 64 * 128 * int(sh_bits.sum())
+            sh_flops = FLOPS_PER_BLOCK * int(sh_bits.sum())
             result["stage2_fwd_block_shared_selection"] = {"ms": sh_ms, "tflops": sh_flops / sh_ms / 1e9,
                                                            "frac_peak": sh_flops / sh_ms / 1e9 / PEAK_BF16_TFLOPS}
-        try:
-            from infllmv2_cuda_impl_amd.backward import HAVE_BACKWARD  # noqa: F401
-            qg, kg, vg = [t.clone().requires_grad_(True) for t in (q, k, v)]
-            dout = torch.randn_like(q)
+        qg, kg, vg = [t.clone().requires_grad_(True) for t in (q, k, v)]
+        dout = torch.randn_like(q)
 
-            def fwd_bwd():
-                o = ops.infllmv2_attn_varlen_func(qg, kg, vg, cu_q, cu_q, S, S, causal=True, topk_idx=idx)
-                o.backward(dout)
-                qg.grad = kg.grad = vg.grad = None
-            fb_ms = event_ms(torch, fwd_bwd, 5)
-            result["stage2_fwd_bwd_ms"] = fb_ms
-            result["stage2_bwd_ms"] = fb_ms - stages["stage2_fwd_op"]          # the backward alone (incl. its packing and mask transpose)
-            result["stage2_fwd_bwd_tflops"] = 3.5 * fwd_flops / fb_ms / 1e9
-            result["stage2_fwd_bwd_frac_peak"] = 3.5 * fwd_flops / fb_ms / 1e9 / PEAK_BF16_TFLOPS
-        except ImportError:
-            pass
+        def fwd_bwd():
+            o = ops.infllmv2_attn_varlen_func(qg, kg, vg, cu_q, cu_q, S, S, causal=True, topk_idx=idx)
+            o.backward(dout)
+            qg.grad = kg.grad = vg.grad = None
+        fb_ms = event_ms(torch, fwd_bwd, 5)
+        result["stage2_fwd_bwd_ms"] = fb_ms
+        result["stage2_bwd_ms"] = fb_ms - stages["stage2_fwd_op"]          # the backward alone (incl. its packing and mask transpose)
+        result["stage2_fwd_bwd_tflops"] = 3.5 * fwd_flops / fb_ms / 1e9
+        result["stage2_fwd_bwd_frac_peak"] = 3.5 * fwd_flops / fb_ms / 1e9 / PEAK_BF16_TFLOPS
+        del qg, kg, vg, dout, out_k, lse, ws
 
-    if not args.no_stages:
+    if not args.no_stages and not args.no_other_configs:
+        del q, k, v, kf, kc, out, idx, words, bits
+        torch.cuda.empty_cache()
+        result["config3_varlen_fwd_bwd"] = config3_bench(torch, ops, dev)
+        torch.cuda.empty_cache()
+        result["config4_prefill_128k"] = config4_bench(torch, ops, dev)
+        torch.cuda.empty_cache()
         result["decode_config5"] = decode_bench(torch, ops, dev)
-    if args.calibrate_copy:
-        src = torch.ones(1 << 30, dtype=torch.uint8, device=dev)
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            dst.copy_(src)
-        torch.cuda.synchronize()
+        torch.cuda.empty_cache()
+    if not args.no_stages:
+        result["device_copy_bandwidth"] = copy_bandwidth(torch, dev)
 
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline()
