@@ -25,7 +25,8 @@ Pinning status (how each function is checked independently of its own formula, s
   [16j, 16j+32)"; row sums equal 16.
 * stage-1 compressed LSE: closed form, reduces to exact mode when v is k.
 * stage-2 forward: dense masked softmax; stage-2 backward: central finite
-  differences in fp64 on tiny shapes + softmax-Jacobian identities.
+  differences in fp64 on tiny shapes + softmax-Jacobian identities; the one-key-block
+  form used at full size (stage2_backward_key_block) equals slices of fp64 autograd gradients.
 * decode: the stage-2 forward oracle with one query token; its options (paged cache,
   cache_batch_idx, left padding) are gathers checked by relabelling invariance, rotary by
   complex multiplication, norm preservation, angle addition and the identity at angle 0.
@@ -406,6 +407,46 @@ def stage2_backward(q, k, v, dout, cu_seqlens_q, cu_seqlens_k, fwd_mask_words,
                 dq[q0:q1, hq] = softmax_scale * (ds @ k[k0:k1, h])
                 dk[k0:k1, h] += softmax_scale * (ds.T @ q[q0:q1, hq])
     return dq, dk, dv
+
+
+def stage2_backward_key_block(q, k, v, dout, row_words, kb: int, head: int, softmax_scale: float,
+                              dtype=np.float32):
+    """dK and dV of ONE 64-key block ``kb`` of ONE sequence and KV head (the unit a column-parallel backward works on,
+    flash_bwd_kernel.h:80-856), computed token by token from the tokens whose mask row selects the block, so that a
+    full-size problem costs only those tokens: for such a token i (causal, q_len == k_len) the keys are its selected
+    blocks up to its own, cut at key i; P = softmax(scale * q K^T) over them, O = P V, D = rowsum(dO * O),
+    dP = dO V_kb^T, dS = P_kb * (dP - D); dV_kb += P_kb^T dO, dK_kb += scale * dS^T q, summed over the 16 heads.
+
+    q, dout (S, Hq, d), k, v (S, Hk, d): ONE sequence; row_words (S, n64) uint64: the mask rows of that sequence for
+    KV head ``head``.  Returns (dk_block, dv_block, tokens) with the blocks (rows, d) and the contributing tokens."""
+    S = q.shape[0]
+    G = q.shape[1] // k.shape[1]
+    lo, hi = kb * BLOCK, min((kb + 1) * BLOCK, S)
+    nb = (S + BLOCK - 1) // BLOCK
+    bits = uint64_to_bool(row_words, nb)                          # (S, nb)
+    tokens = [i for i in range(lo, S) if bits[i, kb]]
+    kh = np.asarray(k[:, head], dtype=dtype)
+    vh = np.asarray(v[:, head], dtype=dtype)
+    dk = np.zeros((hi - lo, k.shape[2]), dtype=np.float64)
+    dv = np.zeros((hi - lo, k.shape[2]), dtype=np.float64)
+    for i in tokens:
+        blocks = np.nonzero(bits[i, :i // BLOCK + 1])[0]
+        keys = np.concatenate([np.arange(b * BLOCK, min((b + 1) * BLOCK, i + 1)) for b in blocks])
+        in_kb = (keys >= lo) & (keys < hi)
+        qi = np.asarray(q[i, head * G:(head + 1) * G], dtype=dtype)       # (G, d)
+        do = np.asarray(dout[i, head * G:(head + 1) * G], dtype=dtype)
+        s = (qi @ kh[keys].T).astype(np.float64) * softmax_scale
+        p = np.exp(s - s.max(axis=1, keepdims=True))
+        p /= p.sum(axis=1, keepdims=True)
+        o = p @ vh[keys].astype(np.float64)
+        D = (do.astype(np.float64) * o).sum(axis=1, keepdims=True)
+        pk = p[:, in_kb]                                                  # (G, rows of the block visible to i)
+        rows = keys[in_kb] - lo
+        dp = do.astype(np.float64) @ vh[lo + rows].astype(np.float64).T
+        ds = pk * (dp - D)
+        dv[rows] += pk.T @ do.astype(np.float64)
+        dk[rows] += softmax_scale * (ds.T @ qi.astype(np.float64))
+    return dk, dv, tokens
 
 
 def decode_forward(q, k_cache, v_cache, cache_seqlens, fwd_mask_words, softmax_scale: float,

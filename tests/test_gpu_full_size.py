@@ -97,7 +97,7 @@ def test_config2_prefill_32k(ops):
         assert err.max() <= 2e-2 and err.mean() <= 1e-3, (r, err.max(), err.mean())
 
 
-def test_config3_varlen_fwd_bwd_64k(ops):
+def test_config3_varlen_fwd_bwd_64k(ops, monkeypatch):
     dev = torch.device("cuda:0")
     rng = np.random.default_rng(1)
     lens = [int(64 * x) for x in rng.integers(64, 385, size=4)]
@@ -148,6 +148,44 @@ def test_config3_varlen_fwd_bwd_64k(ops):
         dk_scale = float(kg.grad[sl].float().abs().sum(0).max())
         assert float(dk_sum.abs().max()) <= 2e-2 * dk_scale
     assert bool(torch.isfinite(qg.grad.float()).all() and torch.isfinite(kg.grad.float()).all())
+    # dK / dV element by element on sampled key blocks: per sequence one late block (few tokens, all near its diagonal:
+    # a light slice that the column kernel merges with others) and one mid-prefix block that many distant tokens
+    # chose by score (many 512-token slices, multi-slice accumulation); never block 0.  The oracle only needs the
+    # tokens whose mask row selects the block.  Three backward modes: S/dP recomputed in the dQ kernel (default),
+    # the dS hand-off (a ~19 GB workspace here), and deterministic accumulation.
+    samples = []
+    for b in range(4):
+        nb = lens[b] // 64
+        sl = slice(int(cu_l[b]), int(cu_l[b + 1]))
+        for kb, h in ((nb - 3, b % 2), (nb // 3, (b + 1) % 2)):
+            dk_ref, dv_ref, toks = O.stage2_backward_key_block(bf16_np(q[sl]), bf16_np(k[sl]), bf16_np(v[sl]),
+                                                                bf16_np(dout[sl]), words[h, sl], kb, h, 128 ** -0.5)
+            assert len(toks) >= 64 and kb > 0
+            samples.append((b, kb, h, dk_ref, dv_ref, len(toks)))
+    assert max(n for *_, n in samples) >= 2500                 # a heavy block spanning several token slices is among them
+
+    def check_blocks(dk, dv, what):
+        for b, kb, h, dk_ref, dv_ref, _ in samples:
+            rows = slice(int(cu_l[b]) + kb * 64, int(cu_l[b]) + kb * 64 + 64)
+            for name, got, ref in (("dk", dk[rows, h], dk_ref), ("dv", dv[rows, h], dv_ref)):
+                sc = max(1.0, float(np.abs(ref).max()))
+                err = np.abs(bf16_np(got) - ref)
+                assert err.max() <= 2e-2 * sc and err.mean() <= 1e-3 * sc, (what, name, b, kb, h, err.max(), err.mean(), sc)
+    check_blocks(kg.grad, vg.grad, "recompute")
+    dq_default = qg.grad.clone()
+    monkeypatch.setenv("INFLLMV2_BWD_HANDOFF", "1")
+    monkeypatch.setenv("INFLLMV2_BWD_HANDOFF_MAX_BYTES", str(40 << 30))
+    qg.grad = kg.grad = vg.grad = None
+    ops.infllmv2_attn_varlen_func(qg, kg, vg, cu, cu, max(lens), max(lens), causal=True, topk_idx=idx).backward(dout)
+    check_blocks(kg.grad, vg.grad, "hand-off")
+    dq_err = (qg.grad.float() - dq_default.float()).abs()
+    assert float(dq_err.max()) <= 2e-2 * max(1.0, float(dq_default.float().abs().max()))
+    monkeypatch.setenv("INFLLMV2_BWD_HANDOFF", "0")
+    qg.grad = kg.grad = vg.grad = None
+    ops.infllmv2_attn_varlen_func(qg, kg, vg, cu, cu, max(lens), max(lens), causal=True, topk_idx=idx,
+                                  deterministic=True).backward(dout)
+    check_blocks(kg.grad, vg.grad, "deterministic")
+    assert torch.equal(qg.grad, dq_default)                    # dQ is bit-reproducible in every mode that recomputes
 
 
 def test_config5_decode_batch64(ops):

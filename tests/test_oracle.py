@@ -347,6 +347,24 @@ def _dead_rows_alive(bits, cu_q, cu_k, causal):
     return alive
 
 
+@pytest.mark.parametrize("S,k_sel", [(300, 2), (200, 4), (130, 1)])
+def test_key_block_backward_is_a_slice_of_the_library_gradients(S, k_sel):
+    """stage2_backward_key_block (token-by-token, only the tokens that select the block) against autograd of the
+    masked-softmax attention in fp64: every key block and KV head, including blocks no token selects and the ragged
+    last block."""
+    q, k, v, cu_q, cu_k, words, bits = _random_case(21, [S], [S], k_sel, True)
+    scale = 128 ** -0.5
+    dout = rng(22).standard_normal(q.shape).astype(np.float32)
+    _, _, ref_dk, ref_dv = _torch_stage2(q, k, v, cu_q, cu_k, bits, scale, True, dout)
+    for h in range(2):
+        for kb in range((S + 63) // 64):
+            dk, dv, toks = O.stage2_backward_key_block(q, k, v, dout, words[h], kb, h, scale, dtype=np.float64)
+            lo, hi = kb * 64, min(kb * 64 + 64, S)
+            assert dk.shape == (hi - lo, 128)
+            assert np.abs(dk - ref_dk[lo:hi, h]).max() < 1e-9 and np.abs(dv - ref_dv[lo:hi, h]).max() < 1e-9
+            assert all(bits[h, t, kb] and t >= lo for t in toks)
+
+
 def test_stage2_dense_equals_all_blocks_selected():
     q, k, v, cu_q, cu_k, _, _ = _random_case(13, [90], [150], 1, True)
     full = np.tile(np.arange(3, dtype=np.int32), (2, 90, 1))
