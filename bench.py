@@ -188,27 +188,25 @@ def config4_bench(torch, ops, dev):
     ms = {
         "compress_keys": event_ms(torch, lambda: (ops.compress_keys(k, cu, S, 32, 16), ops.compress_keys(k, cu, S, 128, 64)), 5),
         "stage1_pooled_fused": event_ms(torch, s1, 3),
-        "topk": event_ms(torch, lambda: ops.topk_blocks(pooled, topk), 5),
-        "pack_mask": event_ms(torch, lambda: ops.topk_to_uint64(idx, S, 64), 5),
+        "topk_with_mask": event_ms(torch, lambda: ops.topk_blocks(pooled, topk, return_mask=True), 5),
         "stage2_fwd_op": event_ms(torch, lambda: ops.infllmv2_attn_varlen_func(q, k, v, cu, cu, S, S, causal=True, topk_idx=idx), 3),
     }
 
     def step():
         p = s1()
-        i = ops.topk_blocks(p, topk)
-        return ops.infllmv2_attn_varlen_func(q, k, v, cu, cu, S, S, causal=True, topk_idx=i)
+        i, m = ops.topk_blocks(p, topk, return_mask=True)
+        return ops.infllmv2_attn_varlen_func(q, k, v, cu, cu, S, S, causal=True, topk_idx=i, block_mask=m)
     step_ms = event_ms(torch, step, 3, warmup=1)
     n64 = (nblk + 63) // 64
     return {"workload": f"BASELINE config 4: prefill forward, 1 x {S} tokens, GQA 32q/2kv, d=128, block 64, topk={topk}, "
-                        "causal; fused Stage-1/pool + top-k + pack + Stage-2 fwd",
+                        "causal; fused Stage-1/pool + top-k with mask words + Stage-2 fwd",
             "selected_causal_blocks_per_token_head": nsel / (2 * S), "stages_ms": ms, "ms_per_step": step_ms,
             "tflops_whole_step": flops / step_ms / 1e9, "stage2_fwd_tflops": flops / ms["stage2_fwd_op"] / 1e9,
             "stage2_fwd_frac_peak": flops / ms["stage2_fwd_op"] / 1e9 / PEAK_BF16_TFLOPS,
             "stage1_tflops": s1_flops / ms["stage1_pooled_fused"] / 1e9,
             "stage1_frac_peak": s1_flops / ms["stage1_pooled_fused"] / 1e9 / PEAK_BF16_TFLOPS,
-            "stage1_topk_share_of_fwd": (ms["stage1_pooled_fused"] + ms["topk"]) / step_ms,
-            "stages_hbm_gbs": {"topk": (2 * S * nblk * 2 + 2 * S * topk * 4) / ms["topk"] / 1e6,
-                               "pack_mask": (2 * S * topk * 4 + 2 * S * n64 * 8) / ms["pack_mask"] / 1e6}}
+            "stage1_topk_share_of_fwd": (ms["stage1_pooled_fused"] + ms["topk_with_mask"]) / step_ms,
+            "stages_hbm_gbs": {"topk_with_mask": (2 * S * nblk * 2 + 2 * S * topk * 4 + 2 * S * n64 * 8) / ms["topk_with_mask"] / 1e6}}
 
 
 def decode_bench(torch, ops, dev):
@@ -234,21 +232,21 @@ def decode_bench(torch, ops, dev):
     pooled = s1()
     idx = ops.topk_blocks(pooled, topk).unsqueeze(2)
     s1_ms = event_ms(torch, s1, 20)
-    topk_ms = event_ms(torch, lambda: ops.topk_blocks(pooled, topk), 20)
+    topk_ms = event_ms(torch, lambda: ops.topk_blocks(pooled, topk, return_mask=True, by_index=True), 20)
     append_ms = event_ms(torch, lambda: (ops.compress_keys_cache(kc, L, 32, 16, out=fine, old_lens=pos, max_new_rows=1),
                                          ops.compress_keys_cache(kc, L, 128, 64, out=coarse, old_lens=pos, max_new_rows=1)), 20)
     s2_ms = event_ms(torch, lambda: ops.infllmv2_attn_with_kvcache(q, kc, vc, cache_seqlens=L, topk_idx=idx), 20)
 
     def step():
         p = s1()
-        i = ops.topk_blocks(p, topk).unsqueeze(2)
-        return ops.infllmv2_attn_with_kvcache(q, kc, vc, cache_seqlens=L, topk_idx=i)
+        _, m = ops.topk_blocks(p, topk, return_mask=True, by_index=True)
+        return ops.infllmv2_attn_with_kvcache(q, kc, vc, cache_seqlens=L, block_mask=m.unsqueeze(2))
     step_ms = event_ms(torch, step, 20)
     s1_bytes = 2 * 128 * 2 * (int(fl.sum()) + int(cl.sum()))           # Hk * (Lk_b + Lc_b) * d * 2 bytes over the batch
     s2_bytes = B * 2 * 64 * 64 * 128 * 2 * 2 + 2 * B * 32 * 128 * 2
     gbs = lambda b, ms: b / ms / 1e6
     return {"workload": "BASELINE config 5: batch 64, seqlen_q 1, cache lengths 64*U[256,2048], topk 64; Stage 1 over "
-                        "per-sequence compressed-key caches + pooling + top-k, then mask packing + Stage-2 decode",
+                        "per-sequence compressed-key caches + pooling + top-k with mask words, then Stage-2 decode (ms: mask packing + decode from an index list)",
             "ms": s2_ms, "algorithmic_bytes": s2_bytes, "hbm_gbs": gbs(s2_bytes, s2_ms),
             "frac_hbm_peak": gbs(s2_bytes, s2_ms) / PEAK_HBM_GBS,
             "stage1_ms": s1_ms, "stage1_algorithmic_bytes": s1_bytes, "stage1_hbm_gbs": gbs(s1_bytes, s1_ms),
@@ -350,8 +348,8 @@ def main():
         else:                           # same pooled tensor, bit for bit, in one launch
             pooled = ops.infllmv2_attn_stage1_pooled(q, kf, kc, cu_q, cu_f, cu_c, S, Lk, local_blocks, init_blocks,
                                                      causal=True)
-        idx = ops.topk_blocks(pooled, topk)
-        return ops.infllmv2_attn_varlen_func(q, k, v, cu_q, cu_q, S, S, causal=True, topk_idx=idx), idx
+        idx, mask = ops.topk_blocks(pooled, topk, return_mask=True)      # the selection launch writes the packed mask too
+        return ops.infllmv2_attn_varlen_func(q, k, v, cu_q, cu_q, S, S, causal=True, topk_idx=idx, block_mask=mask), idx
 
     for _ in range(args.warmup):
         step()
@@ -380,7 +378,7 @@ def main():
                                f"kernel 32/stride 16 compressed keys, block 64, topk={topk} "
                                f"({init_blocks} init + {local_blocks + 1} local forced), causal; "
                                + ("Stage-1 + pool" if args.unfused_front_end else "fused Stage-1/pool")
-                               + " + top-k + pack + Stage-2 fwd",
+                               + " + top-k with mask words + Stage-2 fwd",
                    "seqlen": S, "topk": topk, "selected_causal_blocks_per_token_head": nsel / (2 * S)},
         "stage2_fwd_algorithmic_flops": fwd_flops, "stage1_algorithmic_flops": s1_flops,
         "frac_bf16_mfma_peak_whole_step": fwd_flops / ms_per_step / 1e9 / PEAK_BF16_TFLOPS,
@@ -396,14 +394,19 @@ def main():
             "stage1_pooled_fused": event_ms(torch, lambda: ops.infllmv2_attn_stage1_pooled(
                 q, kf, kc, cu_q, cu_f, cu_c, S, Lk, local_blocks, init_blocks, causal=True), 10),
             "topk": event_ms(torch, lambda: ops.topk_blocks(pooled, topk), 10),
+            "topk_with_mask": event_ms(torch, lambda: ops.topk_blocks(pooled, topk, return_mask=True), 10),
+            "topk_by_index_with_mask": event_ms(torch, lambda: ops.topk_blocks(pooled, topk, return_mask=True, by_index=True), 10),
             "pack_mask": event_ms(torch, lambda: ops.topk_to_uint64(idx, S, 64), 10),
-            "stage2_fwd_op": event_ms(torch, lambda: ops.infllmv2_attn_varlen_func(q, k, v, cu_q, cu_q, S, S, causal=True, topk_idx=idx), 10),
+            "stage2_fwd_op": event_ms(torch, lambda: ops.infllmv2_attn_varlen_func(q, k, v, cu_q, cu_q, S, S, causal=True, topk_idx=idx,
+                                                                               block_mask=words), 10),
             "transpose_mask": event_ms(torch, lambda: ops.transpose_blockmask(words, nblk), 10),
         }
         n64 = words.shape[-1]
         stages_gbs = {
             "pool": (2 * S * Lk * 2 + 2 * S * nblk * 2) / stages["pool"] / 1e6,
             "topk": (2 * S * nblk * 2 + 2 * S * topk * 4) / stages["topk"] / 1e6,
+            "topk_with_mask": (2 * S * nblk * 2 + 2 * S * topk * 4 + 2 * S * n64 * 8) / stages["topk_with_mask"] / 1e6,
+            "topk_by_index_with_mask": (2 * S * nblk * 2 + 2 * S * topk * 4 + 2 * S * n64 * 8) / stages["topk_by_index_with_mask"] / 1e6,
             "pack_mask": (2 * S * topk * 4 + 2 * S * n64 * 8) / stages["pack_mask"] / 1e6,
             "transpose_mask": (2 * 2 * S * n64 * 8) / stages["transpose_mask"] / 1e6,
         }
@@ -412,8 +415,8 @@ def main():
         result["stage1_tflops"] = s1_flops / stages["stage1"] / 1e9
         sel_ms = stages["stage1"] + stages["pool"] + stages["topk"]
         result["stage1_pool_topk_share_of_fwd"] = sel_ms / (sel_ms + stages["pack_mask"] + stages["stage2_fwd_op"])
-        sel_ms = stages["stage1_pooled_fused"] + stages["topk"]
-        result["fused_front_end_share_of_fwd"] = sel_ms / (sel_ms + stages["pack_mask"] + stages["stage2_fwd_op"])
+        sel_ms = stages["stage1_pooled_fused"] + stages["topk_with_mask"]
+        result["fused_front_end_share_of_fwd"] = sel_ms / (sel_ms + stages["stage2_fwd_op"])
         del score, pooled
 
         # the dominant kernel alone: K/V images prepacked, mask packed, HIP events on the launch stream

@@ -23,7 +23,7 @@
 extern "C" {
 #endif
 
-#define INFLLMV2_ABI_VERSION 6
+#define INFLLMV2_ABI_VERSION 7
 
 /* ---- library ------------------------------------------------------------------------------ */
 
@@ -106,6 +106,17 @@ int infllmv2_topk(void* stream, int num_tokens, int dim, int top, int dtype, con
  * topk_idx (rows, k) int32 = first k columns of a stable descending sort, -1 padded. */
 int infllmv2_topk_blocks(void* stream, const void* pooled, int64_t row_stride, int32_t* topk_idx,
                          int64_t rows, int n, int k);
+
+/* The same selection with the packing of csrc/topk_to_uint64.cuh:10-52 done by the same wavefronts: mask_words
+ * (rows, n_uint64_per_row; null = not wanted) receives bit (c % 64) of word c / 64 for every selected column c,
+ * i.e. what infllmv2_topk_to_uint64 computes from topk_idx, so that Stage 2 needs no separate packing launch.
+ * dtype 0 = fp16, 1 = bf16.  by_index != 0 writes the selected columns in ascending order instead of value order
+ * (the order the reference's callers sort them into, tests/utils.py:124-126; no ordering work).  drop_neg_inf != 0
+ * never selects a column whose score is -inf (a block with no visible key: the future of a causal query), so rows
+ * with fewer than k reachable blocks are padded with -1 instead. */
+int infllmv2_topk_select(void* stream, const void* pooled, int64_t row_stride, int dtype, int32_t* topk_idx,
+                         uint64_t* mask_words, int64_t rows, int n, int k, int n_uint64_per_row, int by_index,
+                         int drop_neg_inf);
 
 /* ---- Compressed keys (caller-side in the reference) ----------------------------------------- */
 

@@ -11,7 +11,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libinfllmv2_hip.so")
 
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 _p, _i, _i64, _sz, _f = C.c_void_p, C.c_int, C.c_int64, C.c_size_t, C.c_float
 
@@ -28,6 +28,7 @@ SIGNATURES = {
     "infllmv2_max_pooling_1d_varlen_strided": [_p, _p, _p, _p, _p, _p] + [_i] * 6 + [_i64, _i64] + [_i] * 7,
     "infllmv2_topk": [_p, _i, _i, _i, _i, _p, _p, _p],
     "infllmv2_topk_blocks": [_p, _p, _i64, _p, _i64, _i, _i],
+    "infllmv2_topk_select": [_p, _p, _i64, _i, _p, _p, _i64, _i, _i, _i, _i, _i],
     "infllmv2_compress_keys": [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i64, _i64, _i, _i, _i],
     "infllmv2_compress_keys_cache": [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _p, _p, _i, _i],
     "infllmv2_varlen_fwd_stage1": [_p, _p, _p, _p, _p, _p, _p, _p, _i, _i64, _i, _i, _i, _i, _i, _p, _p, _p, _i64, _i64, _f, _i],

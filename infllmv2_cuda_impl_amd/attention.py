@@ -145,7 +145,8 @@ class Infllmv2AttnVarlenFunc(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p, softmax_scale,
-                causal, window_size, softcap, alibi_slopes, deterministic, return_softmax, block_table, topk_idx):
+                causal, window_size, softcap, alibi_slopes, deterministic, return_softmax, block_table, topk_idx,
+                block_mask=None):
         if softmax_scale is None:
             softmax_scale = q.shape[-1] ** (-0.5)
         causal = _reject_unsupported(dropout_p, window_size, softcap, alibi_slopes, causal, max_seqlen_k)
@@ -154,20 +155,28 @@ class Infllmv2AttnVarlenFunc(torch.autograd.Function):
         q, k, v = [_dense_last_dim(x) for x in (q, k, v)]
         _check_qkv(q, k, v, cu_seqlens_q, cu_seqlens_k)
         fwd_mask = None
-        if topk_idx is not None:
+        sparse = topk_idx is not None or block_mask is not None
+        if block_mask is not None:
+            # the packed selection itself (topk_blocks(return_mask=True)): nothing to pack
+            n64 = ((max_seqlen_k + BLOCK_N - 1) // BLOCK_N + 63) // 64
+            if block_mask.dtype != torch.int64 or tuple(block_mask.shape) != (k.shape[1], q.shape[0], n64):
+                raise RuntimeError("block_mask must be int64 of shape (num_heads_k, total_q, ceil(ceil(max_seqlen_k / 64) / 64))")
+            require_gpu(block_mask, "block_mask")
+            fwd_mask = block_mask.contiguous()
+        elif topk_idx is not None:
             assert topk_idx.dtype == torch.int32
             fwd_mask, _ = topk_to_uint64(topk_idx, max_seqlen_k, BLOCK_N)
             if fwd_mask.dim() != 3 or fwd_mask.shape[0] != k.shape[1] or fwd_mask.shape[1] != q.shape[0]:
                 raise RuntimeError("topk_idx must have shape (num_heads_k, total_q, k)")
         out, lse = _sparse_forward(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
-                                   softmax_scale, causal, fwd_mask, lse_expanded=topk_idx is not None)
+                                   softmax_scale, causal, fwd_mask, lse_expanded=sparse)
         ctx.save_for_backward(q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, fwd_mask)
         ctx.max_seqlen_q = max_seqlen_q
         ctx.max_seqlen_k = max_seqlen_k
         ctx.softmax_scale = softmax_scale
         ctx.causal = causal
         ctx.deterministic = deterministic
-        ctx.sparse = topk_idx is not None
+        ctx.sparse = sparse
         ctx.max_selected = topk_idx.shape[-1] if topk_idx is not None else 0     # a mask row has at most k set bits
         if not return_softmax:
             return out
@@ -184,13 +193,13 @@ class Infllmv2AttnVarlenFunc(torch.autograd.Function):
         dq, dk, dv = sparse_backward(dout, q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, ctx.max_seqlen_q,
                                      ctx.max_seqlen_k, ctx.softmax_scale, ctx.causal, fwd_mask, ctx.sparse,
                                      ctx.deterministic, ctx.max_selected)
-        return (dq, dk, dv) + (None,) * 14
+        return (dq, dk, dv) + (None,) * 15
 
 
 def infllmv2_attn_varlen_func(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p=0.0,
                               softmax_scale=None, causal=False, window_size=(-1, -1), softcap=0.0,
                               alibi_slopes=None, deterministic=False, return_attn_probs=False, block_table=None,
-                              topk_idx=None):
+                              topk_idx=None, block_mask=None):
     """Block-sparse (or, with ``topk_idx=None``, dense) attention over packed variable-length sequences.
 
     q ``(total_q, nheads, 128)``, k/v ``(total_k, nheads_k, 128)`` bf16 with ``nheads == 16*nheads_k``;
@@ -203,10 +212,13 @@ def infllmv2_attn_varlen_func(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q,
     where ``softmax_lse`` is fp32 ``(nheads_k, total_q*16)`` with column ``t*16 + g`` on the sparse path
     (``(nheads, total_q)`` on the dense path) and ``S_dmask`` is empty.  dropout, softcap, ALiBi, sliding
     windows and paged KV are rejected exactly as the reference build rejects them.
+    ``block_mask`` (not in the reference's signature) is the packed form of the same selection, int64
+    ``(nheads_k, total_q, ceil(ceil(max_seqlen_k / 64) / 64))`` as ``topk_to_uint64`` / ``topk_blocks(return_mask=True)``
+    produce it; when given it is used as is and ``topk_idx`` only bounds the blocks per row for the backward.
     """
     return Infllmv2AttnVarlenFunc.apply(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p,
                                         softmax_scale, causal, window_size, softcap, alibi_slopes, deterministic,
-                                        return_attn_probs, block_table, topk_idx)
+                                        return_attn_probs, block_table, topk_idx, block_mask)
 
 
 def infllmv2_attn_stage1(q, k, v, cu_seqlens_q, cu_seqlens_k, cu_seqlens_v, max_seqlen_q, max_seqlen_k,
@@ -328,7 +340,7 @@ def infllmv2_attn_with_kvcache(q, k_cache, v_cache, k=None, v=None, rotary_cos=N
                                cache_leftpad: Optional[torch.Tensor] = None,
                                block_table: Optional[torch.Tensor] = None, softmax_scale=None, causal=False,
                                window_size=(-1, -1), softcap=0.0, rotary_interleaved=True, alibi_slopes=None,
-                               num_splits=0, return_softmax_lse=False, topk_idx=None):
+                               num_splits=0, return_softmax_lse=False, topk_idx=None, block_mask=None):
     """Decode step against a KV cache, restricted to the blocks in ``topk_idx``.
 
     q ``(batch, 1, nheads, 128)``; caches ``(batch, capacity, nheads_k, 128)``; ``cache_seqlens`` int or int32
@@ -351,7 +363,12 @@ def infllmv2_attn_with_kvcache(q, k_cache, v_cache, k=None, v=None, rotary_cos=N
     if cache_seqlens is not None and isinstance(cache_seqlens, int):
         cache_seqlens = torch.full((q.shape[0],), cache_seqlens, dtype=torch.int32, device=k_cache.device)
     mask = None
-    if topk_idx is not None:
+    if block_mask is not None:
+        # the packed selection (batch, nheads_k, 1, words) as topk_blocks(return_mask=True) writes it
+        if block_mask.dtype != torch.int64 or block_mask.dim() != 4:
+            raise RuntimeError("block_mask must be int64 of shape (batch_size, num_heads_k, 1, words)")
+        mask = block_mask.contiguous()
+    elif topk_idx is not None:
         assert topk_idx.dtype == torch.int32
         # the mask spans the sequence's whole key capacity; with a paged cache that is pages x page size (the
         # reference sizes it from k_cache.shape[1], which for a paged cache is one page)

@@ -81,16 +81,19 @@ class InfLLMv2Attention(torch.nn.Module):
     def forward(self, q, k, v, cu_seqlens, max_seqlen: int, cache: SequenceCache | None = None):
         """q ``(total, nheads, d)``, k/v ``(total, nheads_k, d)`` packed; returns ``(total, nheads, d)``.
         With ``cache`` (one sequence only) the keys, values and compressed keys are also stored for decoding."""
-        topk_idx = None
+        topk_idx = mask = None
         if max_seqlen > self.dense_len:
             batch = cu_seqlens.numel() - 1
             cache_lens = torch.zeros(batch, dtype=torch.int32, device=q.device) if batch > 1 else None
-            topk_idx = select_blocks(q.detach(), k.detach(), cu_seqlens, cu_seqlens, max_seqlen, max_seqlen, self.topk,
-                                     self.local_blocks, self.init_blocks, cache_lens=cache_lens, max_cache_len=0,
-                                     softmax_scale=self.softmax_scale, causal=True, kernel_size=self.kernel_size,
-                                     stride=self.stride, block_size=self.block_size)
+            # the selection launch also writes the packed mask Stage 2 walks
+            topk_idx, mask = select_blocks(q.detach(), k.detach(), cu_seqlens, cu_seqlens, max_seqlen, max_seqlen,
+                                           self.topk, self.local_blocks, self.init_blocks, cache_lens=cache_lens,
+                                           max_cache_len=0, softmax_scale=self.softmax_scale, causal=True,
+                                           kernel_size=self.kernel_size, stride=self.stride,
+                                           block_size=self.block_size, return_mask=True)
         out = infllmv2_attn_varlen_func(q, k, v, cu_seqlens, cu_seqlens, max_seqlen, max_seqlen,
-                                        softmax_scale=self.softmax_scale, causal=True, topk_idx=topk_idx)
+                                        softmax_scale=self.softmax_scale, causal=True, topk_idx=topk_idx,
+                                        block_mask=mask)
         if cache is not None:
             if cu_seqlens.numel() != 2:
                 raise RuntimeError("a SequenceCache holds one sequence")
@@ -171,15 +174,16 @@ class InfLLMv2Attention(torch.nn.Module):
         for buf, lens, ks, st in ((cache.k_fine, cache.fine_lens, self.kernel_size, self.stride),
                                   (cache.k_coarse, cache.coarse_lens, 4 * self.kernel_size, 4 * self.stride)):
             compress_keys_cache(cache.k, new, ks, st, out=buf, old_lens=old, max_new_rows=1, out_lens=lens)
-        topk_idx = None
+        mask = None
         if cache.max_length + 1 > self.dense_len:
             pooled = infllmv2_attn_stage1_kvcache(q, cache.k_fine, cache.k_coarse, cache.fine_lens, cache.coarse_lens,
                                                   old, self.local_blocks, self.init_blocks,
                                                   max_cache_len=cache.max_length, block_size=self.block_size,
                                                   stride=self.stride, softmax_scale=self.softmax_scale, causal=False)
-            topk_idx = topk_blocks(pooled, self.topk).unsqueeze(2)                   # (batch, Hk, 1, topk)
+            _, mask = topk_blocks(pooled, self.topk, return_mask=True, by_index=True)
+            mask = mask.unsqueeze(2)                                                 # (batch, Hk, 1, words)
         out = infllmv2_attn_with_kvcache(q, cache.k, cache.v, k=k_new, v=v_new, cache_seqlens=old,
-                                         softmax_scale=self.softmax_scale, topk_idx=topk_idx)
+                                         softmax_scale=self.softmax_scale, block_mask=mask)
         cache.lengths = new
         cache.max_length += 1
         return out

@@ -12,18 +12,35 @@ from . import _lib
 from ._util import flat_rows, require_gpu, stream_ptr
 
 
-def topk_blocks(pooled: torch.Tensor, k: int) -> torch.Tensor:
+def topk_blocks(pooled: torch.Tensor, k: int, *, return_mask: bool = False, by_index: bool = False,
+                drop_unreachable: bool = False, n_uint64_per_row: int | None = None):
     """pooled ``(..., n_blocks)`` fp16/bf16 -> int32 ``(..., k)``: the first ``k`` columns of a stable
-    descending sort of every row; rows with fewer than ``k`` columns are padded with ``-1``."""
+    descending sort of every row; rows with fewer than ``k`` columns are padded with ``-1``.
+
+    Options (all off by default, none changes WHICH blocks of reachable score are selected):
+    ``return_mask`` also returns the packed selection ``(..., n_uint64_per_row)`` int64, equal to
+    ``topk_to_uint64`` of the indices (default width ``ceil(n_blocks / 64)``), written by the same launch, so that
+    Stage 2 (``block_mask=``) needs no packing launch; ``by_index`` lists the selected blocks in ascending block
+    order (what the reference's callers sort them into) instead of score order; ``drop_unreachable`` never selects
+    a block whose pooled score is ``-inf`` (no visible key: blocks in a causal query's future), so a query with
+    fewer than ``k`` reachable blocks gets ``-1`` padding instead of unreachable blocks."""
     assert pooled.dtype == torch.float16 or pooled.dtype == torch.bfloat16
     require_gpu(pooled, "pooled")
     x = pooled if pooled.is_contiguous() else pooled.contiguous()
     n = x.shape[-1]
     out = torch.empty(tuple(x.shape[:-1]) + (k,), dtype=torch.int32, device=x.device)
+    rows = flat_rows(x.shape[:-1])
+    if not (return_mask or by_index or drop_unreachable):
+        with torch.cuda.device(x.device):
+            _lib.call("infllmv2_topk_blocks", stream_ptr(x.device), x.data_ptr(), n, out.data_ptr(), rows, n, k)
+        return out
+    n64 = (n + 63) // 64 if n_uint64_per_row is None else int(n_uint64_per_row)
+    mask = torch.empty(tuple(x.shape[:-1]) + (n64,), dtype=torch.int64, device=x.device) if return_mask else None
     with torch.cuda.device(x.device):
-        _lib.call("infllmv2_topk_blocks", stream_ptr(x.device), x.data_ptr(), n, out.data_ptr(),
-                  flat_rows(x.shape[:-1]), n, k)
-    return out
+        _lib.call("infllmv2_topk_select", stream_ptr(x.device), x.data_ptr(), n, int(x.dtype == torch.bfloat16),
+                  out.data_ptr(), None if mask is None else mask.data_ptr(), rows, n, k, n64, int(bool(by_index)),
+                  int(bool(drop_unreachable)))
+    return (out, mask) if return_mask else out
 
 
 def compress_keys(k: torch.Tensor, cu_seqlens_k: torch.Tensor, max_seqlen_k: int, kernel_size: int, stride: int,
@@ -101,13 +118,17 @@ def select_blocks(q: torch.Tensor, k: torch.Tensor, cu_seqlens_q: torch.Tensor, 
                   max_seqlen_q: int, max_seqlen_k: int, topk: int, local_blocks: int, init_blocks: int,
                   cache_lens: torch.Tensor | None = None, max_cache_len: int | None = None, softmax_scale=None,
                   causal: bool = True, kernel_size: int = 32, stride: int = 16, block_size: int = 64,
-                  exact_lse: bool = False) -> torch.Tensor:
+                  exact_lse: bool = False, return_mask: bool = False, by_index: bool = False,
+                  drop_unreachable: bool = False):
     """The selection front end in one call: compressed keys (kernel ``kernel_size`` / stride ``stride``; the
     log-sum-exp over the 4x coarser set, or over the same set with ``exact_lse``), Stage-1 scores pooled onto
     ``block_size``-token key blocks in one launch, top-k.  Returns ``topk_idx`` int32 ``(nheads_k, total_q, topk)``
     for :func:`infllmv2_attn_varlen_func`, equal to what the reference's sequence of calls
     (compress, ``infllmv2_attn_stage1``, ``max_pooling_1d(_varlen)``, top-k) selects; the score tensor is never
     materialised.  Packed batches need ``cache_lens`` (zeros for plain prefill), as ``max_pooling_1d_varlen`` does.
+    ``return_mask`` / ``by_index`` / ``drop_unreachable`` as in :func:`topk_blocks`; with ``return_mask`` the result is
+    ``(topk_idx, block_mask)`` and the mask (as wide as ``max_seqlen_k`` needs) can be handed to
+    ``infllmv2_attn_varlen_func(block_mask=...)``.
     """
     from .attention import infllmv2_attn_stage1_pooled
     kf, cu_f = compress_keys(k, cu_seqlens_k, max_seqlen_k, kernel_size, stride)
@@ -120,4 +141,8 @@ def select_blocks(q: torch.Tensor, k: torch.Tensor, cu_seqlens_q: torch.Tensor, 
                                          init_blocks, cache_lens=cache_lens, max_cache_len=max_cache_len,
                                          block_size=block_size, stride=stride, softmax_scale=softmax_scale,
                                          causal=causal)
-    return topk_blocks(pooled, topk)
+    n64 = ((max_seqlen_k + block_size - 1) // block_size + 63) // 64
+    if n64 * 64 < pooled.shape[-1]:                           # cached tokens widen the pooled rows beyond max_seqlen_k
+        n64 = (pooled.shape[-1] + 63) // 64
+    return topk_blocks(pooled, topk, return_mask=return_mask, by_index=by_index, drop_unreachable=drop_unreachable,
+                       n_uint64_per_row=n64)

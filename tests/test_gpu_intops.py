@@ -175,3 +175,97 @@ def test_topk_blocks_many_ties_full_size(ops):
     assert np.array_equal(got.cpu().numpy(), ref)
     w, _ = ops.topk_to_uint64(got, n * 64, 64)
     assert np.array_equal(words_np(w), O.topk_to_uint64(ref, n * 64, 64)[0])
+
+
+def _postprocess(ref_idx, x_np, by_index, drop):
+    """Oracle-side statement of the options of topk_blocks: drop columns whose score is -inf, then (by_index) sort
+    the survivors by column; -1 pads the end either way."""
+    out = np.full_like(ref_idx, -1)
+    flat_i, flat_o = ref_idx.reshape(-1, ref_idx.shape[-1]), out.reshape(-1, ref_idx.shape[-1])
+    flat_x = x_np.reshape(-1, x_np.shape[-1])
+    for r in range(flat_i.shape[0]):
+        keep = [int(c) for c in flat_i[r] if c >= 0 and not (drop and np.isneginf(flat_x[r, c]))]
+        if by_index:
+            keep.sort()
+        flat_o[r, :len(keep)] = keep
+    return out
+
+
+@pytest.mark.parametrize("rows,n,k", [((2, 130), 512, 64), ((3, 40), 100, 16), ((2, 30), 2048, 64), ((2, 9), 700, 256),
+                                      ((1, 70), 33, 64), ((2, 33), 4100, 16)])
+@pytest.mark.parametrize("by_index,drop", [(False, False), (True, False), (False, True), (True, True)])
+def test_topk_select_options_and_fused_mask(ops, rows, n, k, by_index, drop):
+    """The fused selection: indices in score or block order, -inf columns optionally never selected, and the packed
+    mask written by the same launch == topk_to_uint64 of the indices == the oracle's packing.  Consecutive rows are
+    made to differ wildly (the search of a row starts at its neighbour's threshold): scale jumps by orders of
+    magnitude, rows of all ties, rows with only a handful of reachable columns."""
+    g = torch.Generator(device="cpu").manual_seed(11)
+    x = torch.randn(rows + (n,), generator=g)
+    R = rows[-1]
+    for r in range(R):
+        x[:, r] *= float(10.0 ** ((r * 7) % 9 - 4))           # 1e-4 .. 1e4 from one row to the next
+        if r % 5 == 1:
+            x[:, r] = 0.25                                     # every column ties
+        if r % 5 == 2:
+            x[:, r, min(7, n - 1):] = float("-inf")            # fewer reachable columns than k
+        if r % 5 == 3:
+            x[:, r, : min(40, n)] = float("inf")               # forced columns, ties at +inf
+            x[:, r, n // 2:] = float("-inf")
+        if r % 7 == 4:
+            x[:, r] = -x[:, r].abs()                           # all negative
+    x = x.to(torch.bfloat16).to(dev())
+    idx, mask = ops.topk_blocks(x, k, by_index=by_index, drop_unreachable=drop, return_mask=True)
+    x_np = bf16_np(x)
+    want = _postprocess(O.topk_blocks(x_np, k), x_np, by_index, drop)
+    assert np.array_equal(idx.cpu().numpy(), want)
+    n64 = (n + 63) // 64
+    assert tuple(mask.shape) == rows + (n64,) and mask.dtype == torch.int64
+    assert np.array_equal(words_np(mask), O.topk_to_uint64(want, n * 64, 64)[0])
+    again, _ = ops.topk_to_uint64(idx, n * 64, 64)
+    assert torch.equal(again, mask)
+    # without the mask and with a wider mask row
+    assert torch.equal(ops.topk_blocks(x, k, by_index=by_index, drop_unreachable=drop), idx)
+    _, wide = ops.topk_blocks(x, k, by_index=by_index, drop_unreachable=drop, return_mask=True, n_uint64_per_row=n64 + 3)
+    assert torch.equal(wide[..., :n64], mask) and not bool(wide[..., n64:].any())
+
+
+def test_topk_select_fp16_drops_fp16_minus_infinity(ops):
+    x = torch.randn(2, 20, 200, device=dev()).to(torch.float16)
+    x[..., 150:] = float("-inf")
+    idx = ops.topk_blocks(x, 180, drop_unreachable=True, by_index=True)
+    want = torch.arange(150, device=dev(), dtype=torch.int32).expand(2, 20, 150)
+    assert torch.equal(idx[..., :150], want) and bool((idx[..., 150:] == -1).all())
+
+
+def test_block_mask_argument_equals_topk_idx_argument(ops):
+    """Stage 2 fed with the fused launch's mask == Stage 2 fed with the index list (which it packs itself); forward
+    and backward, and the decode operator."""
+    torch.manual_seed(12)
+    S, k_sel = 700, 6
+    mk = lambda h: torch.randn(S, h, 128, device=dev()).to(torch.bfloat16)
+    q, k, v = mk(32), mk(2), mk(2)
+    cu = torch.tensor([0, S], dtype=torch.int32, device=dev())
+    idx, mask = ops.select_blocks(q, k, cu, cu, S, S, k_sel, 1, 1, return_mask=True)
+    assert torch.equal(idx, ops.select_blocks(q, k, cu, cu, S, S, k_sel, 1, 1))
+    outs = []
+    for kw in (dict(topk_idx=idx), dict(topk_idx=idx, block_mask=mask), dict(block_mask=mask)):
+        qg, kg, vg = [t.clone().requires_grad_(True) for t in (q, k, v)]
+        o = ops.infllmv2_attn_varlen_func(qg, kg, vg, cu, cu, S, S, causal=True, **kw)
+        o.backward(torch.ones_like(o))
+        outs.append((o.detach(), qg.grad, kg.grad.float(), vg.grad.float()))
+    for o, dq, dk, dv in outs[1:]:
+        assert torch.equal(o, outs[0][0]) and torch.equal(dq, outs[0][1])
+        assert float((dk - outs[0][2]).abs().max()) <= 2e-2 * float(outs[0][2].abs().max())
+        assert float((dv - outs[0][3]).abs().max()) <= 2e-2 * float(outs[0][3].abs().max())
+    with pytest.raises(RuntimeError, match="block_mask"):
+        ops.infllmv2_attn_varlen_func(q, k, v, cu, cu, S, S, causal=True, block_mask=mask[:, :, :0])
+    B, cap = 3, 640
+    qd = torch.randn(B, 1, 32, 128, device=dev()).to(torch.bfloat16)
+    kc = torch.randn(B, cap, 2, 128, device=dev()).to(torch.bfloat16)
+    vc = torch.randn(B, cap, 2, 128, device=dev()).to(torch.bfloat16)
+    L = torch.tensor([640, 300, 65], dtype=torch.int32, device=dev())
+    pooled = torch.rand(B, 2, 1, cap // 64, device=dev()).to(torch.bfloat16)
+    di, dm = ops.topk_blocks(pooled, 4, return_mask=True)
+    a = ops.infllmv2_attn_with_kvcache(qd, kc, vc, cache_seqlens=L, topk_idx=di)
+    b = ops.infllmv2_attn_with_kvcache(qd, kc, vc, cache_seqlens=L, block_mask=dm)
+    assert torch.equal(a, b)
