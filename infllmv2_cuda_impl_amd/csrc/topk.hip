@@ -58,12 +58,15 @@ __device__ __forceinline__ int lanes_below(uint64_t mask, int base) {          /
     return __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(mask >> 32),
                                      __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(mask), static_cast<uint32_t>(base)));
 }
-// old with lane `which` (a constant) replaced by the wavefront-uniform value
-__device__ __forceinline__ uint32_t write_lane(uint32_t old, uint32_t uniform_value, int which) {
-    asm volatile("v_writelane_b32 %0, %1, %2" : "+v"(old) : "s"(uniform_value), "n"(which));
-    return old;
+// lane `which` (a constant) of the pair (lo, hi) replaced by the two halves of a wavefront-uniform 64-bit value.
+// The value usually comes straight out of a vector compare: a vector instruction must not read a scalar register
+// in the two slots after a vector instruction wrote it, and the compiler does not look inside asm (s_nop 1).
+__device__ __forceinline__ void write_lane64(uint32_t& lo, uint32_t& hi, uint64_t uniform_value, int which) {
+    asm volatile("s_nop 1\n\tv_writelane_b32 %0, %2, %4\n\tv_writelane_b32 %1, %3, %4"
+                 : "+v"(lo), "+v"(hi)
+                 : "s"(static_cast<uint32_t>(uniform_value)), "s"(static_cast<uint32_t>(uniform_value >> 32)), "n"(which));
 }
-// b where the lane's bit of the lane mask is set, else a
+// b where the lane's bit of the lane mask (a compile-time constant, so no vector instruction wrote it) is set, else a
 __device__ __forceinline__ uint32_t select_by_lane_mask(uint32_t a, uint32_t b, uint64_t lane_mask) {
     uint32_t r;
     asm("v_cndmask_b32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "s"(lane_mask));
@@ -222,24 +225,24 @@ void topk_rows_kernel(const TopkParams p) {
         int base = 0;
         uint32_t words0_lo = 0, words0_hi = 0, words1_lo = 0, words1_hi = 0;   // lane e holds mask word e (e + 64)
         const uint32_t inv_lane = 0xffffu - static_cast<uint32_t>(lane);
-        auto emit = [&](int e, uint64_t take_mask) {
+        auto emit = [&](int e, bool take, uint64_t take_mask) {
             const int slot = lanes_below(take_mask, base);
             uint32_t val;
             if constexpr (kByIndex) val = static_cast<uint32_t>(e * 64 + lane);
             else val = (key[e] << 16) | (inv_lane - static_cast<uint32_t>(e * 64));
-            sel[select_by_lane_mask(dummy, slot, take_mask)] = val;
+            sel[take ? slot : dummy] = val;
             base += __builtin_popcountll(take_mask);
             if constexpr (kMask) {                             // the ballot is the mask word
-                const uint32_t lo32 = static_cast<uint32_t>(take_mask), hi32 = static_cast<uint32_t>(take_mask >> 32);
-                uint32_t& wl = e < 64 ? words0_lo : words1_lo;
-                uint32_t& wh = e < 64 ? words0_hi : words1_hi;
-                wl = write_lane(wl, lo32, e & 63);
-                wh = write_lane(wh, hi32, e & 63);
+                if (e < 64) write_lane64(words0_lo, words0_hi, take_mask, e & 63);
+                else write_lane64(words1_lo, words1_hi, take_mask, e & 63);
             }
         };
         if (all_ge) {
 #pragma unroll
-            for (int e = 0; e < kItems; ++e) emit(e, __builtin_amdgcn_ballot_w64(key[e] >= thr));
+            for (int e = 0; e < kItems; ++e) {
+                const bool take = key[e] >= thr;
+                emit(e, take, __builtin_amdgcn_ballot_w64(take));
+            }
         } else {
             int ties_left = k_sel - count_ge(thr + 1);
 #pragma unroll
@@ -247,7 +250,7 @@ void topk_rows_kernel(const TopkParams p) {
                 const bool eq = key[e] == thr;
                 const uint64_t eq_mask = __builtin_amdgcn_ballot_w64(eq);
                 const bool take = key[e] > thr || (eq && lanes_below(eq_mask, 0) < ties_left);
-                emit(e, __builtin_amdgcn_ballot_w64(take));
+                emit(e, take, __builtin_amdgcn_ballot_w64(take));
                 const int eq_total = __builtin_popcountll(eq_mask);
                 ties_left -= eq_total < ties_left ? eq_total : ties_left;
             }
