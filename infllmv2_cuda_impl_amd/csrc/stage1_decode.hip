@@ -220,6 +220,10 @@ void stage1_decode_score_kernel(const S1DecodeParams p) {
 
     bf16x8 qf[4];
     s1d_load_q(qf, p, sq, h, n, g);
+    // the first two tiles are requested before anything waits on memory
+    bf16x8 ta[16], tb[16];
+    if (t0 < t1) s1d_load_tile(ta, sq.kbase, p.k_row_stride, t0 * 64, sq.Lk, n, g);
+    if (t0 + 1 < t1) s1d_load_tile(tb, sq.kbase, p.k_row_stride, (t0 + 1) * 64, sq.Lk, n, g);
     // log-sum-exp of head 4g + e: the partials of the coarse runs merged in run order
     float lse2[4];
     {
@@ -292,9 +296,6 @@ void stage1_decode_score_kernel(const S1DecodeParams p) {
         }
     };
 
-    bf16x8 ta[16], tb[16];
-    if (t0 < t1) s1d_load_tile(ta, sq.kbase, p.k_row_stride, t0 * 64, sq.Lk, n, g);
-    if (t0 + 1 < t1) s1d_load_tile(tb, sq.kbase, p.k_row_stride, (t0 + 1) * 64, sq.Lk, n, g);
     for (int ti = t0; ti < t1; ti += 2) {
         consume(ta, ti);
         if (ti + 2 < t1) s1d_load_tile(ta, sq.kbase, p.k_row_stride, (ti + 2) * 64, sq.Lk, n, g);
