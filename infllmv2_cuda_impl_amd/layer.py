@@ -26,6 +26,7 @@ import torch
 
 from .attention import (infllmv2_attn_stage1_kvcache, infllmv2_attn_stage1_pooled, infllmv2_attn_varlen_func,
                         infllmv2_attn_with_kvcache)
+from .pooling import max_pooling_1d_varlen
 from .selection import compress_keys, compress_keys_cache, select_blocks, topk_blocks
 
 
@@ -67,23 +68,49 @@ class BatchCache:
 
 
 class InfLLMv2Attention(torch.nn.Module):
-    """Sparse attention over 64-token key blocks chosen per query token and KV head (no parameters)."""
+    """Sparse attention over 64-token key blocks chosen per query token and KV head (no parameters).
+
+    ``selection`` picks the branch a model layer runs: ``"sparse"`` (default) scores the compressed keys and takes the
+    top-k blocks; ``"window"`` attends only the forced blocks (the first ``init_blocks`` and the query's own block with
+    the ``local_blocks`` before it: a sliding window in 64-token blocks plus attention sinks, no scoring at all);
+    ``"dense"`` attends everything.  Sequences of at most ``dense_len`` tokens are dense whatever the branch."""
 
     def __init__(self, topk: int = 64, local_blocks: int = 31, init_blocks: int = 1, dense_len: int = 0,
-                 kernel_size: int = 32, stride: int = 16, block_size: int = 64, softmax_scale: float | None = None):
+                 kernel_size: int = 32, stride: int = 16, block_size: int = 64, softmax_scale: float | None = None,
+                 selection: str = "sparse"):
         super().__init__()
+        if selection not in ("sparse", "window", "dense"):
+            raise ValueError("selection must be 'sparse', 'window' or 'dense'")
+        self.selection = selection
         self.topk, self.local_blocks, self.init_blocks = topk, local_blocks, init_blocks
         self.dense_len = dense_len
         self.kernel_size, self.stride, self.block_size = kernel_size, stride, block_size
         self.softmax_scale = softmax_scale
+
+    def _window_blocks(self, nheads_k: int, rows: int, cu_seqlens_q, positions, max_seqlen_q: int, max_position: int,
+                       device):
+        """The forced blocks alone as a selection: what the pooling operator marks +inf on a score tensor with no
+        columns, with every other block dropped.  ``rows``: packed query tokens; ``positions`` int32 (batch): tokens before each
+        sequence's first query.  Returns ``(topk_idx, block_mask)`` with ``init_blocks + local_blocks + 1`` index slots."""
+        batch = cu_seqlens_q.numel() - 1
+        empty = torch.empty((nheads_k, rows, 0), dtype=torch.bfloat16, device=device)
+        no_keys = torch.zeros(batch + 1, dtype=torch.int32, device=device)
+        pooled = max_pooling_1d_varlen(empty, cu_seqlens_q, no_keys, positions, max_seqlen_q, 0, self.local_blocks,
+                                       self.init_blocks, block_size=self.block_size, stride=self.stride,
+                                       max_cache_len=max_position)
+        return topk_blocks(pooled, self.init_blocks + self.local_blocks + 1, return_mask=True, by_index=True,
+                           drop_unreachable=True)
 
     # ---- prefill / training ----
     def forward(self, q, k, v, cu_seqlens, max_seqlen: int, cache: SequenceCache | None = None):
         """q ``(total, nheads, d)``, k/v ``(total, nheads_k, d)`` packed; returns ``(total, nheads, d)``.
         With ``cache`` (one sequence only) the keys, values and compressed keys are also stored for decoding."""
         topk_idx = mask = None
-        if max_seqlen > self.dense_len:
-            batch = cu_seqlens.numel() - 1
+        batch = cu_seqlens.numel() - 1
+        if self.selection == "window" and max_seqlen > self.dense_len:
+            topk_idx, mask = self._window_blocks(k.shape[1], q.shape[0], cu_seqlens, torch.zeros(batch, dtype=torch.int32, device=q.device),
+                                                 max_seqlen, 0, q.device)
+        elif self.selection == "sparse" and max_seqlen > self.dense_len:
             cache_lens = torch.zeros(batch, dtype=torch.int32, device=q.device) if batch > 1 else None
             # the selection launch also writes the packed mask Stage 2 walks
             topk_idx, mask = select_blocks(q.detach(), k.detach(), cu_seqlens, cu_seqlens, max_seqlen, max_seqlen,
@@ -130,7 +157,11 @@ class InfLLMv2Attention(torch.nn.Module):
         n = cache.length
         lens = torch.tensor([old], dtype=torch.int32, device=dev)
         topk_idx = None
-        if n > self.dense_len:
+        if self.selection == "window" and n > self.dense_len:
+            topk_idx, _ = self._window_blocks(cache.k.shape[2], 1, torch.tensor([0, 1], dtype=torch.int32, device=dev), lens,
+                                              1, pos, dev)
+            topk_idx = topk_idx.unsqueeze(0)
+        elif self.selection == "sparse" and n > self.dense_len:
             rows = lambda ks, st: (n - ks) // st + 1 if n >= ks else 0
             lf, lc = rows(self.kernel_size, self.stride), rows(4 * self.kernel_size, 4 * self.stride)
             one = lambda x: torch.tensor([0, x], dtype=torch.int32, device=dev)
@@ -175,7 +206,11 @@ class InfLLMv2Attention(torch.nn.Module):
                                   (cache.k_coarse, cache.coarse_lens, 4 * self.kernel_size, 4 * self.stride)):
             compress_keys_cache(cache.k, new, ks, st, out=buf, old_lens=old, max_new_rows=1, out_lens=lens)
         mask = None
-        if cache.max_length + 1 > self.dense_len:
+        if self.selection == "window" and cache.max_length + 1 > self.dense_len:
+            cu_one = torch.arange(batch + 1, dtype=torch.int32, device=q.device)
+            _, mask = self._window_blocks(cache.k.shape[2], batch, cu_one, old, 1, cache.max_length, q.device)
+            mask = mask.transpose(0, 1).unsqueeze(2).contiguous()                    # (Hk, batch, words) -> (batch, Hk, 1, words)
+        elif self.selection == "sparse" and cache.max_length + 1 > self.dense_len:
             pooled = infllmv2_attn_stage1_kvcache(q, cache.k_fine, cache.k_coarse, cache.fine_lens, cache.coarse_lens,
                                                   old, self.local_blocks, self.init_blocks,
                                                   max_cache_len=cache.max_length, block_size=self.block_size,
