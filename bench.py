@@ -83,6 +83,9 @@ def parse_args():
                     help="skip BASELINE configs 3, 4 and 5 (keeps a profile to the default workload)")
     ap.add_argument("--only-config", type=int, default=0, choices=[0, 3, 4, 5],
                     help="run one of the extra configurations alone (for profiling it) and print its record")
+    ap.add_argument("--probe", action="store_true",
+                    help="run the streaming probes (bytes per clock a CU gets through its L1 return path and from LDS) "
+                         "and print their record instead of the benchmark")
     ap.add_argument("--print-source-hash", action="store_true",
                     help="print the hash of the Stage-2 forward kernel sources (what a traffic summary must name) and exit")
     return ap.parse_args()
@@ -236,6 +239,9 @@ def decode_bench(torch, ops, dev):
     append_ms = event_ms(torch, lambda: (ops.compress_keys_cache(kc, L, 32, 16, out=fine, old_lens=pos, max_new_rows=1),
                                          ops.compress_keys_cache(kc, L, 128, 64, out=coarse, old_lens=pos, max_new_rows=1)), 20)
     s2_ms = event_ms(torch, lambda: ops.infllmv2_attn_with_kvcache(q, kc, vc, cache_seqlens=L, topk_idx=idx), 20)
+    _, bm = ops.topk_blocks(pooled, topk, return_mask=True, by_index=True)
+    bm = bm.unsqueeze(2)
+    s2_mask_ms = event_ms(torch, lambda: ops.infllmv2_attn_with_kvcache(q, kc, vc, cache_seqlens=L, block_mask=bm), 20)
 
     def step():
         p = s1()
@@ -249,11 +255,37 @@ def decode_bench(torch, ops, dev):
                         "per-sequence compressed-key caches + pooling + top-k with mask words, then Stage-2 decode (ms: mask packing + decode from an index list)",
             "ms": s2_ms, "algorithmic_bytes": s2_bytes, "hbm_gbs": gbs(s2_bytes, s2_ms),
             "frac_hbm_peak": gbs(s2_bytes, s2_ms) / PEAK_HBM_GBS,
+            "ms_with_block_mask": s2_mask_ms, "hbm_gbs_with_block_mask": gbs(s2_bytes, s2_mask_ms),
+            "frac_hbm_peak_with_block_mask": gbs(s2_bytes, s2_mask_ms) / PEAK_HBM_GBS,
             "stage1_ms": s1_ms, "stage1_algorithmic_bytes": s1_bytes, "stage1_hbm_gbs": gbs(s1_bytes, s1_ms),
             "stage1_frac_hbm_peak": gbs(s1_bytes, s1_ms) / PEAK_HBM_GBS,
             "topk_ms": topk_ms, "compressed_key_append_ms": append_ms, "step_ms": step_ms,
             "step_hbm_gbs": gbs(s1_bytes + s2_bytes, step_ms),
             "step_frac_hbm_peak": gbs(s1_bytes + s2_bytes, step_ms) / PEAK_HBM_GBS}
+
+
+def stream_probes(torch, _lib, dev):
+    """What one CU receives per unit time from L2-resident data through global_load_dwordx4 and through LDS-DMA (the
+    L1 return path that bounds the Stage-2 gather) and from LDS through ds_read_b128.  One workgroup of eight
+    wavefronts per CU, 256 CUs; wall time from HIP events, ticks from the kernel's own cycle counter."""
+    import numpy as np
+    wgs, iters = 256, 400
+    src = torch.arange(wgs * 131072 // 4, dtype=torch.int32, device=dev)
+    out = torch.zeros(2 * wgs, dtype=torch.int64, device=dev)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    record = {}
+    for mode, name in ((0, "global_load_dwordx4"), (1, "lds_dma_dwordx4"), (2, "ds_read_b128")):
+        launch = lambda: _lib.call("infllmv2_probe_stream", stream, src.data_ptr(), src.numel() * 4, out.data_ptr(),
+                                   wgs, iters, mode)
+        ms = min(event_ms(torch, launch, 3) for _ in range(3))
+        o = out.cpu().numpy().reshape(wgs, 2).astype(np.float64)
+        record[name] = {"tbs_all_cus": wgs * iters * 131072 / ms / 1e9,
+                        "gbs_per_cu": iters * 131072 / ms / 1e6,
+                        "bytes_per_counter_tick_per_cu": float(np.median(o[:, 1] / o[:, 0]))}
+    record["what"] = ("each of 256 workgroups (8 wavefronts, one per CU) re-reads its own 128 KiB 400 times, 16 KiB "
+                      "in flight per wavefront; wall time from HIP events (includes the 128 KiB LDS fill and the launch), "
+                      "ticks from s_memtime inside the kernel, median over workgroups")
+    return record
 
 
 def cpu_model():
@@ -331,6 +363,9 @@ def main():
     from infllmv2_cuda_impl_amd import _lib
 
     dev = torch.device("cuda:0")
+    if args.probe:
+        print(json.dumps(stream_probes(torch, _lib, dev)))
+        return
     if args.only_config:
         fn = {3: config3_bench, 4: config4_bench, 5: decode_bench}[args.only_config]
         print(json.dumps(fn(torch, ops, dev)))
