@@ -121,8 +121,8 @@ def test_config3_varlen_fwd_bwd_64k(ops, monkeypatch):
         seg = pooled[:, cu_l[b]:cu_l[b + 1]]
         seg[:, forced] = float("inf")
         seg[:, future & ~forced] = float("-inf")
-    idx = ops.topk_blocks(pooled, 64)
-    idx = torch.where(torch.gather(pooled, 2, idx.long().clamp(min=0)) == float("-inf"), torch.full_like(idx, -1), idx)
+    idx = ops.topk_blocks(pooled, 64, drop_unreachable=True)   # blocks in a token's future are never selected: -1 padding
+    assert not bool((torch.gather(pooled, 2, idx.long().clamp(min=0)) == float("-inf"))[idx >= 0].any())
     qg, kg, vg = [t.clone().requires_grad_(True) for t in (q, k, v)]
     out = ops.infllmv2_attn_varlen_func(qg, kg, vg, cu, cu, max(lens), max(lens), causal=True, topk_idx=idx)
     out.backward(dout)
