@@ -12,6 +12,9 @@
  * checkout) that it replaces.  Where the reference's pybind function takes at::Tensor arguments
  * the tensor is flattened here into pointer + sizes + strides, and outputs/scratch that the
  * reference allocates internally are passed in by the caller.
+ *
+ * Element types: the entry points below take bfloat16 tensors wherever a 16-bit tensor is meant,
+ * unless they have a `dtype` argument; their IEEE-half twins are declared at the end of the file.
  */
 #ifndef INFLLMV2_HIP_H
 #define INFLLMV2_HIP_H
@@ -23,7 +26,7 @@
 extern "C" {
 #endif
 
-#define INFLLMV2_ABI_VERSION 7
+#define INFLLMV2_ABI_VERSION 8
 
 /* ---- library ------------------------------------------------------------------------------ */
 
@@ -342,6 +345,78 @@ int infllmv2_fwd_kvcache_static(void* stream, const void* q, void* kcache, void*
                                 const int32_t* block_table, int64_t block_table_batch_stride, int page_block_size,
                                 const void* rotary_cos, const void* rotary_sin, int rotary_dim,
                                 int rotary_interleaved);
+
+/* ---- IEEE half (fp16) twins ---------------------------------------------------------------------
+ *
+ * The reference switches between half and bfloat16 on the tensors' dtype (csrc/entry.cu:20-29; its build
+ * instantiates bfloat16 only).  Here every entry point that reads or writes attention tensors exists once per element
+ * type: the plain name takes bfloat16, the name with the suffix _f16 takes IEEE half, with the same arguments, the
+ * same semantics and the same workspace sizes (both types are two bytes wide; infllmv2_pack_kv, infllmv2_kv_image_bytes
+ * and the other size queries serve both).  All 16-bit tensors of one call have the one element type: q, k, v, out,
+ * dout, dq, dk, dv, caches, compressed keys, scores, rotary tables.  fp32 accumulation, one rounding of P, dS and of
+ * each output to the element type, as for bfloat16.  Pooling, top-k and the mask operations take their element type
+ * as an argument or have none.  infllmv2_fwd_kvcache_static has no fp16 twin. */
+int infllmv2_compress_keys_f16(void* stream, const void* k, void* out, const int32_t* cu_seqlens_k,
+                               int32_t* cu_seqlens_out, int batch, int max_seqlen_k, int num_heads_k, int head_dim,
+                               int64_t k_row_stride, int64_t k_head_stride, int kernel_size, int stride, int first_row);
+int infllmv2_compress_keys_cache_f16(void* stream, const void* kcache, void* out_cache, const int32_t* old_lens,
+                                     const int32_t* new_lens, int32_t* out_lens, int batch, int max_new_rows,
+                                     int num_heads_k, int head_dim, const int64_t* kcache_strides,
+                                     const int64_t* out_strides, int kernel_size, int stride);
+int infllmv2_varlen_fwd_stage1_f16(void* stream, const void* q, const void* k, const void* v, void* score,
+                                   const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                                   const int32_t* cu_seqlens_v, int batch, int64_t total_q, int num_heads,
+                                   int num_heads_k, int head_dim, int max_seqlen_q, int max_seqlen_k,
+                                   const int64_t* q_strides, const int64_t* k_strides,
+                                   const int64_t* v_strides, int64_t score_head_stride,
+                                   int64_t score_row_stride, float softmax_scale, int is_causal);
+int infllmv2_varlen_fwd_stage1_pooled_f16(void* stream, const void* q, const void* k, const void* v, void* pooled,
+                                          const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                                          const int32_t* cu_seqlens_v, const int32_t* cache_lens, int cache_len,
+                                          int batch, int64_t total_q, int num_heads, int num_heads_k, int head_dim,
+                                          int max_seqlen_q, int max_seqlen_k, const int64_t* q_strides,
+                                          const int64_t* k_strides, const int64_t* v_strides, int out_len,
+                                          float softmax_scale, int is_causal, int kernel_size, int stride, int padding,
+                                          int block_size, int local_blocks, int init_blocks);
+int infllmv2_stage1_decode_f16(void* stream, const void* q, const void* k, const void* v, void* out,
+                               const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, const int32_t* k_lens,
+                               const int32_t* cu_seqlens_v, const int32_t* v_lens, void* workspace,
+                               size_t workspace_bytes, int batch, int num_heads, int num_heads_k, int head_dim,
+                               int max_seqlen_k, int max_seqlen_v, const int64_t* q_strides, const int64_t* k_strides,
+                               const int64_t* v_strides, int64_t out_head_stride, int64_t out_row_stride,
+                               float softmax_scale, int is_causal, int pooled, const int32_t* cache_lens, int cache_len,
+                               int out_len, int kernel_size, int stride, int padding, int block_size, int local_blocks,
+                               int init_blocks);
+int infllmv2_varlen_fwd_f16(void* stream, const void* q, const void* k, const void* v, void* out,
+                            float* softmax_lse, const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                            const uint64_t* blockmask, void* workspace, size_t workspace_bytes,
+                            int kv_prepacked, int batch, int64_t total_q, int64_t total_k, int num_heads,
+                            int num_heads_k, int head_dim, int max_seqlen_q, int max_seqlen_k,
+                            const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                            const int64_t* o_strides, const int64_t* lse_strides, int n_uint64_per_row,
+                            float softmax_scale, int is_causal);
+int infllmv2_varlen_bwd_f16(void* stream, const void* dout, const void* q, const void* k, const void* v,
+                            const void* out, const float* softmax_lse, void* dq, void* dk, void* dv,
+                            const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                            const uint64_t* fwd_blockmask, void* workspace, size_t workspace_bytes, int batch,
+                            int64_t total_q, int64_t total_k, int num_heads, int num_heads_k, int head_dim,
+                            int max_seqlen_q, int max_seqlen_k, const int64_t* q_strides,
+                            const int64_t* k_strides, const int64_t* v_strides, const int64_t* o_strides,
+                            const int64_t* do_strides, const int64_t* dq_strides, const int64_t* dk_strides,
+                            const int64_t* dv_strides, const int64_t* lse_strides, int n_uint64_per_row,
+                            float softmax_scale, int is_causal, int deterministic,
+                            int max_selected_blocks);
+int infllmv2_fwd_kvcache_f16(void* stream, const void* q, void* kcache, void* vcache, const void* k_new,
+                             const void* v_new, const int32_t* cache_seqlens, void* out, float* softmax_lse,
+                             const uint64_t* blockmask, void* workspace, size_t workspace_bytes, int batch,
+                             int seqlen_q, int num_heads, int num_heads_k, int head_dim, int cache_capacity,
+                             int seqlen_new, const int64_t* q_strides, const int64_t* kcache_strides,
+                             const int64_t* vcache_strides, const int64_t* knew_strides,
+                             const int64_t* vnew_strides, const int64_t* o_strides, int n_uint64_per_row,
+                             int num_splits, float softmax_scale, const int32_t* cache_batch_idx,
+                             const int32_t* cache_leftpad, const int32_t* block_table,
+                             int64_t block_table_batch_stride, int page_block_size, const void* rotary_cos,
+                             const void* rotary_sin, int rotary_dim, int rotary_interleaved);
 
 #ifdef __cplusplus
 }

@@ -75,8 +75,6 @@ def _common_checks(q, k, v, cu_seqlens_q, cu_seqlens_k):
         raise RuntimeError("query and key must have the same dtype")
     if v.dtype != q.dtype:
         raise RuntimeError("query and value must have the same dtype")
-    if q.dtype != torch.bfloat16:
-        raise RuntimeError("this build only has bf16 kernels")
     if cu_seqlens_q.dtype != torch.int32:
         raise RuntimeError("cu_seqlens_q must have dtype int32")
     if cu_seqlens_k.dtype != torch.int32:
@@ -129,7 +127,7 @@ def varlen_fwd(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftpad_k_,
     ws = torch.empty(max(_lib.lib.infllmv2_kv_image_bytes(total_k, batch, Hk), 16), dtype=torch.uint8, device=q.device)
     n64 = 0 if blockmask_ is None else blockmask_.shape[-1]
     with torch.cuda.device(q.device):
-        _lib.call("infllmv2_varlen_fwd", stream_ptr(q.device), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+        _lib.call_for(q.dtype, "infllmv2_varlen_fwd", stream_ptr(q.device), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
                   lse.data_ptr(), cu_q.data_ptr(), cu_seqlens_k.data_ptr(), ptr(blockmask_), ws.data_ptr(), ws.numel(), 0,
                   batch, total_q, total_k, Hq, Hk, q.shape[-1], max_q, max_seqlen_k, _layout(q, expanded), _kv(k), _kv(v),
                   _layout(out, expanded), lse_strides, n64, float(softmax_scale), int(bool(is_causal)))
@@ -154,10 +152,10 @@ def varlen_fwd_stage1(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, cu_seqlens_v, s
     batch = cu_seqlens_q.numel() - 1
     cu_q = torch.div(cu_seqlens_q, GROUP, rounding_mode="floor").to(torch.int32)
     row = (max_seqlen_k + 127) // 128 * 128
-    p = torch.zeros((Hk, total_q, row), dtype=torch.bfloat16, device=q.device) if row != max_seqlen_k else \
-        torch.empty((Hk, total_q, row), dtype=torch.bfloat16, device=q.device)
+    p = torch.zeros((Hk, total_q, row), dtype=q.dtype, device=q.device) if row != max_seqlen_k else \
+        torch.empty((Hk, total_q, row), dtype=q.dtype, device=q.device)
     with torch.cuda.device(q.device):
-        _lib.call("infllmv2_varlen_fwd_stage1", stream_ptr(q.device), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+        _lib.call_for(q.dtype, "infllmv2_varlen_fwd_stage1", stream_ptr(q.device), q.data_ptr(), k.data_ptr(), v.data_ptr(),
                   p.data_ptr(), cu_q.data_ptr(), cu_seqlens_k.data_ptr(), cu_seqlens_v.data_ptr(), batch, total_q,
                   Hk * GROUP, Hk, q.shape[-1], max_seqlen_q // GROUP, max_seqlen_k, _layout(q, True), _kv(k), _kv(v),
                   p.stride(0), p.stride(1), float(softmax_scale), int(bool(is_causal)))
@@ -203,7 +201,7 @@ def varlen_bwd(dout, q, k, v, out, softmax_lse, dq_, dk_, dv_, cu_seqlens_q, cu_
     ws_bytes = size_query(batch, total_q, total_k, Hk, max_seqlen_k)
     ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=q.device)
     with torch.cuda.device(q.device):
-        _lib.call("infllmv2_varlen_bwd", stream_ptr(q.device), dout.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+        _lib.call_for(q.dtype, "infllmv2_varlen_bwd", stream_ptr(q.device), dout.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
                   out.data_ptr(), softmax_lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), cu_q.data_ptr(),
                   cu_seqlens_k.data_ptr(), ptr(fwd_mask), ws.data_ptr(), ws.numel(), batch, total_q, total_k, Hq, Hk,
                   q.shape[-1], max_q, max_seqlen_k, _layout(q, expanded), _kv(k), _kv(v), _layout(out, expanded),

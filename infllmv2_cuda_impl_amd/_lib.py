@@ -11,7 +11,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libinfllmv2_hip.so")
 
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 _p, _i, _i64, _sz, _f = C.c_void_p, C.c_int, C.c_int64, C.c_size_t, C.c_float
 
@@ -42,6 +42,12 @@ SIGNATURES = {
     "infllmv2_fwd_kvcache_static": [_p] * 10 + [_i] * 7 + [_p] * 6 + [_i, _i, _f, _p, _p, _p, _i64, _i, _p, _p, _i, _i],
     "infllmv2_pack_kv": [_p, _p, _p, _p, _p, _sz, _i, _i64, _i, _i, _i, _p, _p],
 }
+# entry points that exist once per element type: the plain name takes bfloat16, name + "_f16" IEEE half
+PER_ELEMENT_TYPE = ["infllmv2_compress_keys", "infllmv2_compress_keys_cache", "infllmv2_varlen_fwd_stage1",
+                    "infllmv2_varlen_fwd_stage1_pooled", "infllmv2_stage1_decode", "infllmv2_varlen_fwd",
+                    "infllmv2_varlen_bwd", "infllmv2_fwd_kvcache"]
+for _name in PER_ELEMENT_TYPE:
+    SIGNATURES[_name + "_f16"] = SIGNATURES[_name]
 OTHER = {
     "infllmv2_last_error": (C.c_char_p, []),
     "infllmv2_abi_version": (_i, []),
@@ -86,6 +92,17 @@ def call(name: str, *args) -> None:
     rc = getattr(lib, name)(*args)
     if rc != 0:
         raise RuntimeError(lib.infllmv2_last_error().decode("utf-8", "replace") or f"{name} failed with code {rc}")
+
+
+def call_for(dtype, name: str, *args) -> None:
+    """`call` of the instantiation of a per-element-type entry point for torch dtype `dtype` (bfloat16 or float16)."""
+    import torch
+    if dtype == torch.bfloat16:
+        call(name, *args)
+    elif dtype == torch.float16:
+        call(name + "_f16", *args)
+    else:
+        raise RuntimeError("FlashAttention only support fp16 and bf16 data type")
 
 
 def i64_array(values):

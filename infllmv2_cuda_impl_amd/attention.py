@@ -70,9 +70,6 @@ def _check_qkv(q, k, v, cu_seqlens_q, cu_seqlens_k, same_kv_len=True):
         raise RuntimeError("query and key must have the same dtype")
     if v.dtype != q.dtype:
         raise RuntimeError("query and value must have the same dtype")
-    if q.dtype != torch.bfloat16:
-        # the reference build instantiates bf16 kernels only (static_switch.h:79-83)
-        raise RuntimeError("this build only has bf16 kernels")
     if cu_seqlens_q.dtype != torch.int32:
         raise RuntimeError("cu_seqlens_q must have dtype int32")
     if cu_seqlens_k.dtype != torch.int32:
@@ -131,7 +128,7 @@ def _sparse_forward(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqle
     workspace = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=q.device)
     n64 = 0 if fwd_mask is None else fwd_mask.shape[-1]
     with torch.cuda.device(q.device):
-        _lib.call("infllmv2_varlen_fwd", stream_ptr(q.device), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+        _lib.call_for(q.dtype, "infllmv2_varlen_fwd", stream_ptr(q.device), q.data_ptr(), k.data_ptr(), v.data_ptr(),
                   out.data_ptr(), lse.data_ptr(), cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), ptr(fwd_mask),
                   workspace.data_ptr(), workspace.numel(), 0, batch, total_q, total_k, Hq, Hk, d, max_seqlen_q,
                   max_seqlen_k, _natural_strides(q), _lib.i64_array([k.stride(0), k.stride(1)]),
@@ -300,8 +297,10 @@ def infllmv2_attn_stage1_kvcache(q, k_fine_cache, k_coarse_cache, fine_lens, coa
         softmax_scale = q.shape[-1] ** (-0.5)
     if q.dim() != 4 or q.shape[1] != 1:
         raise RuntimeError("q must have shape (batch_size, 1, num_heads, head_size)")
-    if q.dtype != torch.bfloat16 or k_fine_cache.dtype != q.dtype or k_coarse_cache.dtype != q.dtype:
-        raise RuntimeError("this build only has bf16 kernels")
+    if q.dtype not in (torch.float16, torch.bfloat16):
+        raise RuntimeError("FlashAttention only support fp16 and bf16 data type")
+    if k_fine_cache.dtype != q.dtype or k_coarse_cache.dtype != q.dtype:
+        raise RuntimeError("query and key must have the same dtype")
     batch, _, Hq, d = q.shape
     for name, t in (("q", q), ("k_fine_cache", k_fine_cache), ("k_coarse_cache", k_coarse_cache)):
         require_gpu(t, name)
@@ -319,14 +318,14 @@ def infllmv2_attn_stage1_kvcache(q, k_fine_cache, k_coarse_cache, fine_lens, coa
     rows_f, rows_c = k_fine_cache.shape[1], k_coarse_cache.shape[1]
     q3 = q[:, 0]
     if not pooled:
-        out = torch.empty((batch, Hk, rows_f), dtype=torch.bfloat16, device=q.device)
+        out = torch.empty((batch, Hk, rows_f), dtype=q.dtype, device=q.device)
         return stage1_decode(q3, k_fine_cache, k_coarse_cache, k_lens=fine_lens, v_lens=coarse_lens,
                              max_seqlen_k=rows_f, max_seqlen_v=rows_c, softmax_scale=softmax_scale, causal=causal,
                              out=out, out_head_stride=out.stride(1), out_row_stride=out.stride(0))
     if max_cache_len is None:
         max_cache_len = (rows_f + 1) * stride + block_size
     out_len = (1 + max_cache_len + block_size - 1) // block_size
-    out = torch.empty((batch, Hk, out_len), dtype=torch.bfloat16, device=q.device)
+    out = torch.empty((batch, Hk, out_len), dtype=q.dtype, device=q.device)
     return stage1_decode(q3, k_fine_cache, k_coarse_cache, k_lens=fine_lens, v_lens=coarse_lens, max_seqlen_k=rows_f,
                          max_seqlen_v=rows_c, softmax_scale=softmax_scale, causal=causal, out=out,
                          out_head_stride=out.stride(1), out_row_stride=out.stride(0), pooled=True,

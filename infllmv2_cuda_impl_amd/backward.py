@@ -70,7 +70,7 @@ def sparse_backward(dout, q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, max_seq
         workspace = allocate(0)
     kv = lambda t: _lib.i64_array([t.stride(0), t.stride(1)])
     with torch.cuda.device(q.device):
-        _lib.call("infllmv2_varlen_bwd", stream_ptr(q.device), dout.data_ptr(), q.data_ptr(), k.data_ptr(),
+        _lib.call_for(q.dtype, "infllmv2_varlen_bwd", stream_ptr(q.device), dout.data_ptr(), q.data_ptr(), k.data_ptr(),
                   v.data_ptr(), out.data_ptr(), lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
                   cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), ptr(fwd_mask), workspace.data_ptr(),
                   workspace.numel(), batch, total_q, total_k, Hq, Hk, d, max_seqlen_q, max_seqlen_k,

@@ -2,7 +2,7 @@
 #pragma once
 #include "common.h"
 
-namespace infllmv2 {
+namespace IV2_NS {
 
 // Walks the set bits of one mask row in ascending block order, clipped to [0, last_blk].
 struct BlockWalker {
@@ -73,4 +73,4 @@ __device__ __forceinline__ float wave_sum_over_g(float x) {
     return a + b;
 }
 
-}  // namespace infllmv2
+}  // namespace IV2_NS

@@ -25,13 +25,28 @@ HIPCC_FLAGS = [
 ]
 
 
+# translation units that hold attention kernels: compiled twice, for bfloat16 (plain entry-point names) and, with
+# -DIV2_F16, for IEEE half (entry points with the suffix _f16); the other files are element-type independent or take
+# the type at run time
+PER_ELEMENT_TYPE = {"compress.hip", "decode.hip", "stage1.hip", "stage1_decode.hip", "stage2_bwd.hip",
+                    "stage2_bwd_dkdv.hip", "stage2_bwd_dq.hip", "stage2_bwd_dq_handoff.hip", "stage2_fwd.hip",
+                    "stage2_fwd_hybrid.hip"}
+
+
 def sources():
-    return sorted(f for f in os.listdir(CSRC) if f.endswith(".hip"))
+    """(source file, extra flags, object name) of every compilation."""
+    out = []
+    for f in sorted(f for f in os.listdir(CSRC) if f.endswith(".hip")):
+        out.append((f, [], f[:-4] + ".o"))
+        if f in PER_ELEMENT_TYPE:
+            out.append((f, ["-DIV2_F16=1"], f[:-4] + "_f16.o"))
+    return out
 
 
-def _compile(src: str, verbose: bool) -> str:
-    obj = os.path.join(OBJ_DIR, src[:-4] + ".o")
-    cmd = ["hipcc", *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+def _compile(unit, verbose: bool) -> str:
+    src, extra, obj_name = unit
+    obj = os.path.join(OBJ_DIR, obj_name)
+    cmd = ["hipcc", *HIPCC_FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
     if r.returncode != 0:

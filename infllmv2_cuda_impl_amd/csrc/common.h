@@ -5,19 +5,43 @@
 #include <stdio.h>
 #include <stdarg.h>
 
+// The attention kernels exist once per element type: a translation unit compiled with -DIV2_F16 holds the IEEE-half
+// instantiation (namespace infllmv2_f16, C entry points with the suffix _f16), one compiled without it the bfloat16
+// one (namespace infllmv2, the plain entry-point names).  The two differ in the MFMA instruction, the conversions
+// between fp32 and the element type, and nothing else: operand layouts, images and LDS traffic are the same bytes.
+#ifdef IV2_F16
+#define IV2_NS infllmv2_f16
+#define IV2_ENTRY(name) name##_f16
+#define IV2_MFMA(a, b, c, x, y, z) __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, x, y, z)
+#define IV2_MFMA_ASM "v_mfma_f32_16x16x32_f16"
+#else
+#define IV2_NS infllmv2
+#define IV2_ENTRY(name) name
+#define IV2_MFMA(a, b, c, x, y, z) __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, x, y, z)
+#define IV2_MFMA_ASM "v_mfma_f32_16x16x32_bf16"
+#endif
+
 namespace infllmv2 {
+// Thread-local text of the last failure; every C entry point returns 0 on success.
+void set_error(const char* fmt, ...);
+}  // namespace infllmv2
+
+namespace IV2_NS {
 
 constexpr int kWave = 64;          // CDNA wavefront width
 constexpr int kHeadDim = 128;      // only head size the reference build instantiates (static_switch.h:79-89)
 constexpr int kGroup = 16;         // query heads per KV head (flash_api.cpp:941)
 constexpr int kBlockN = 64;        // key-block size of the sparse mask (flash_api.cpp:706-710)
 
-typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+#ifdef IV2_F16
+typedef _Float16 elem_t;
+#else
+typedef __bf16 elem_t;
+#endif
+typedef __attribute__((__vector_size__(8 * sizeof(elem_t)))) elem_t elem8;     // one lane's MFMA operand
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 typedef uint16_t bf16_bits;
-
-// Thread-local text of the last failure; every C entry point returns 0 on success.
-void set_error(const char* fmt, ...);
+typedef uint16_t elem_bits;                                  // an element as it lies in memory
 
 #define IV2_CHECK(cond, ...)                         \
     do {                                             \
@@ -58,4 +82,27 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
     return static_cast<uint32_t>(f32_to_bf16(lo)) | (static_cast<uint32_t>(f32_to_bf16(hi)) << 16);
 }
 
-}  // namespace infllmv2
+// ---- the element type of this translation unit ----
+#ifdef IV2_F16
+constexpr elem_bits kElemPosInf = 0x7c00, kElemNegInf = 0xfc00;
+__device__ __forceinline__ float elem_to_f32(elem_bits b) { return f16_to_f32(b); }
+// round-to-nearest-even (v_cvt_f16_f32 in the default rounding mode); NaN stays NaN, overflow gives inf
+__device__ __forceinline__ elem_bits f32_to_elem(float f) {
+    const _Float16 x = static_cast<_Float16>(f);
+    elem_bits b;
+    __builtin_memcpy(&b, &x, 2);
+    return b;
+}
+#else
+constexpr elem_bits kElemPosInf = 0x7f80, kElemNegInf = 0xff80;
+__device__ __forceinline__ float elem_to_f32(elem_bits b) { return bf16_to_f32(b); }
+__device__ __forceinline__ elem_bits f32_to_elem(float f) { return f32_to_bf16(f); }
+#endif
+__device__ __forceinline__ uint32_t pack_elem2(float lo, float hi) {
+    return static_cast<uint32_t>(f32_to_elem(lo)) | (static_cast<uint32_t>(f32_to_elem(hi)) << 16);
+}
+// the two elements of a 32-bit word
+__device__ __forceinline__ float elem_lo_to_f32(uint32_t w) { return elem_to_f32(static_cast<elem_bits>(w & 0xffffu)); }
+__device__ __forceinline__ float elem_hi_to_f32(uint32_t w) { return elem_to_f32(static_cast<elem_bits>(w >> 16)); }
+
+}  // namespace IV2_NS

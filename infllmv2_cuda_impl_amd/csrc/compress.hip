@@ -11,7 +11,7 @@
 #include "common.h"
 #include "../../include/infllmv2_hip.h"
 
-namespace infllmv2 {
+namespace IV2_NS {
 
 __device__ __forceinline__ int compressed_rows(int len, int kernel_size, int stride) {
     return len >= kernel_size ? (len - kernel_size) / stride + 1 : 0;
@@ -30,8 +30,8 @@ __global__ void compressed_cu_seqlens_kernel(const int* __restrict__ cu_k, int* 
 }
 
 struct CompressParams {
-    const bf16_bits* k;
-    bf16_bits* out;
+    const elem_bits* k;
+    elem_bits* out;
     const int* cu_k;
     const int* cu_out;
     int64_t k_row_stride, k_head_stride;
@@ -54,7 +54,7 @@ void compress_keys_kernel(const CompressParams p) {
         if (j >= rows) break;                                  // items are ordered by row
         const int u = item % p.units_per_row;
         const int head = u / p.units_per_head, piece = u % p.units_per_head;
-        const bf16_bits* src = p.k + (static_cast<int64_t>(k0) + static_cast<int64_t>(j) * p.stride) * p.k_row_stride +
+        const elem_bits* src = p.k + (static_cast<int64_t>(k0) + static_cast<int64_t>(j) * p.stride) * p.k_row_stride +
                                head * p.k_head_stride + piece * 8;
         float acc[8];
 #pragma unroll
@@ -64,16 +64,16 @@ void compress_keys_kernel(const CompressParams p) {
             const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                acc[2 * e] += __uint_as_float(w[e] << 16);
-                acc[2 * e + 1] += __uint_as_float(w[e] & 0xffff0000u);
+                acc[2 * e] += elem_lo_to_f32(w[e]);
+                acc[2 * e + 1] += elem_hi_to_f32(w[e]);
             }
         }
         const float n = static_cast<float>(p.kernel_size);
         uint4 o;
-        o.x = pack_bf16x2(acc[0] / n, acc[1] / n);
-        o.y = pack_bf16x2(acc[2] / n, acc[3] / n);
-        o.z = pack_bf16x2(acc[4] / n, acc[5] / n);
-        o.w = pack_bf16x2(acc[6] / n, acc[7] / n);
+        o.x = pack_elem2(acc[0] / n, acc[1] / n);
+        o.y = pack_elem2(acc[2] / n, acc[3] / n);
+        o.z = pack_elem2(acc[4] / n, acc[5] / n);
+        o.w = pack_elem2(acc[6] / n, acc[7] / n);
         *reinterpret_cast<uint4*>(p.out + (static_cast<int64_t>(p.cu_out[b]) + j) * p.units_per_row * 8 + u * 8) = o;
     }
 }
@@ -82,8 +82,8 @@ void compress_keys_kernel(const CompressParams p) {
 // rows of its compressed-key cache that windows completed since old_lens[b] tokens are written, the others are left
 // alone.  A decode step (one more token) completes at most one window per set.
 struct CompressCacheParams {
-    const bf16_bits* k;
-    bf16_bits* out;
+    const elem_bits* k;
+    elem_bits* out;
     const int* old_lens;             // null: 0 for every sequence (build everything)
     const int* new_lens;
     int* out_lens;                   // null, or (batch): rows the compressed cache holds afterwards
@@ -104,7 +104,7 @@ void compress_keys_cache_kernel(const CompressCacheParams p) {
         if (j >= rows) break;
         const int u = item % p.units_per_row;
         const int head = u / p.units_per_head, piece = u % p.units_per_head;
-        const bf16_bits* src = p.k + b * p.k_batch + static_cast<int64_t>(j) * p.stride * p.k_row + head * p.k_head + piece * 8;
+        const elem_bits* src = p.k + b * p.k_batch + static_cast<int64_t>(j) * p.stride * p.k_row + head * p.k_head + piece * 8;
         float acc[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) acc[e] = 0.f;
@@ -113,25 +113,25 @@ void compress_keys_cache_kernel(const CompressCacheParams p) {
             const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                acc[2 * e] += __uint_as_float(w[e] << 16);
-                acc[2 * e + 1] += __uint_as_float(w[e] & 0xffff0000u);
+                acc[2 * e] += elem_lo_to_f32(w[e]);
+                acc[2 * e + 1] += elem_hi_to_f32(w[e]);
             }
         }
         const float n = static_cast<float>(p.kernel_size);
         uint4 o;
-        o.x = pack_bf16x2(acc[0] / n, acc[1] / n);
-        o.y = pack_bf16x2(acc[2] / n, acc[3] / n);
-        o.z = pack_bf16x2(acc[4] / n, acc[5] / n);
-        o.w = pack_bf16x2(acc[6] / n, acc[7] / n);
+        o.x = pack_elem2(acc[0] / n, acc[1] / n);
+        o.y = pack_elem2(acc[2] / n, acc[3] / n);
+        o.z = pack_elem2(acc[4] / n, acc[5] / n);
+        o.w = pack_elem2(acc[6] / n, acc[7] / n);
         *reinterpret_cast<uint4*>(p.out + b * p.o_batch + static_cast<int64_t>(j) * p.o_row + head * p.o_head + piece * 8) = o;
     }
 }
 
-}  // namespace infllmv2
+}  // namespace IV2_NS
 
-using namespace infllmv2;
+using namespace IV2_NS;
 
-extern "C" int infllmv2_compress_keys(void* stream, const void* k, void* out, const int32_t* cu_seqlens_k,
+extern "C" int IV2_ENTRY(infllmv2_compress_keys)(void* stream, const void* k, void* out, const int32_t* cu_seqlens_k,
                                       int32_t* cu_seqlens_out, int batch, int max_seqlen_k, int num_heads_k,
                                       int head_dim, int64_t k_row_stride, int64_t k_head_stride, int kernel_size,
                                       int stride, int first_row) {
@@ -149,8 +149,8 @@ extern "C" int infllmv2_compress_keys(void* stream, const void* k, void* out, co
     const int max_rows = max_seqlen_k >= kernel_size ? (max_seqlen_k - kernel_size) / stride + 1 : 0;
     if (max_rows <= first_row) return 0;
     CompressParams p{};
-    p.k = static_cast<const bf16_bits*>(k);
-    p.out = static_cast<bf16_bits*>(out);
+    p.k = static_cast<const elem_bits*>(k);
+    p.out = static_cast<elem_bits*>(out);
     p.cu_k = cu_seqlens_k; p.cu_out = cu_seqlens_out;
     p.k_row_stride = k_row_stride; p.k_head_stride = k_head_stride;
     p.units_per_row = units; p.units_per_head = head_dim / 8;
@@ -161,7 +161,7 @@ extern "C" int infllmv2_compress_keys(void* stream, const void* k, void* out, co
     return 0;
 }
 
-extern "C" int infllmv2_compress_keys_cache(void* stream, const void* kcache, void* out_cache, const int32_t* old_lens,
+extern "C" int IV2_ENTRY(infllmv2_compress_keys_cache)(void* stream, const void* kcache, void* out_cache, const int32_t* old_lens,
                                             const int32_t* new_lens, int32_t* out_lens, int batch, int max_new_rows,
                                             int num_heads_k, int head_dim, const int64_t* kcache_strides,
                                             const int64_t* out_strides, int kernel_size, int stride) {
@@ -174,8 +174,8 @@ extern "C" int infllmv2_compress_keys_cache(void* stream, const void* kcache, vo
     for (int s = 0; s < 3; ++s)
         IV2_CHECK(kcache_strides[s] % 8 == 0 && out_strides[s] % 8 == 0, "compress_keys_cache: strides must be multiples of 8 elements");
     CompressCacheParams p{};
-    p.k = static_cast<const bf16_bits*>(kcache);
-    p.out = static_cast<bf16_bits*>(out_cache);
+    p.k = static_cast<const elem_bits*>(kcache);
+    p.out = static_cast<elem_bits*>(out_cache);
     p.old_lens = old_lens; p.new_lens = new_lens; p.out_lens = out_lens;
     p.k_batch = kcache_strides[0]; p.k_row = kcache_strides[1]; p.k_head = kcache_strides[2];
     p.o_batch = out_strides[0]; p.o_row = out_strides[1]; p.o_head = out_strides[2];

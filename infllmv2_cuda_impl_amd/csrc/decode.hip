@@ -21,15 +21,15 @@
 #include <math.h>
 #include <mutex>
 
-namespace infllmv2 {
+namespace IV2_NS {
 
 struct DecodeParams {
-    const bf16_bits* q;
-    bf16_bits* kcache;
-    bf16_bits* vcache;
-    const bf16_bits* knew;
-    const bf16_bits* vnew;
-    bf16_bits* out;
+    const elem_bits* q;
+    elem_bits* kcache;
+    elem_bits* vcache;
+    const elem_bits* knew;
+    const elem_bits* vnew;
+    elem_bits* out;
     float* lse;                     // (batch, Hq)
     float* o_part;                  // (batch, Hk, splits, 16, 128) fp32, normalised per split
     float* lse_part;                // (batch, Hk, splits, 16)
@@ -48,10 +48,10 @@ struct DecodeParams {
     int64_t bt_batch;
     int page_size;
     // rotary embedding of the appended keys and of the query (flash_fwd_kernel.h:787-929, rotary.h)
-    const bf16_bits* rot_cos;       // (seqlen_ro, rotary_dim / 2)
-    const bf16_bits* rot_sin;
+    const elem_bits* rot_cos;       // (seqlen_ro, rotary_dim / 2)
+    const elem_bits* rot_sin;
     int rotary_dim, rotary_interleaved;
-    bf16_bits* q_rot;               // (batch, Hq, 128): the turned query, in the workspace
+    elem_bits* q_rot;               // (batch, Hq, 128): the turned query, in the workspace
 };
 
 // element offset of cache row `row` of sequence b (head 0)
@@ -68,7 +68,7 @@ __device__ __forceinline__ int64_t cache_row_offset(const DecodeParams& p, int b
 // One 16-byte chunk (8 values, d = 8 chunk ...) of a head vector turned at position pos.  Interleaved: pairs
 // (2i, 2i+1) lie inside the chunk; contiguous: the partner of d is d +- rotary_dim / 2, in another chunk of the
 // same head vector.  (a, b) -> (a cos - b sin, a sin + b cos) in fp32, one rounding (rotary.h:57-62, 131-133).
-__device__ __forceinline__ uint4 rotary_chunk(const DecodeParams& p, const bf16_bits* head_vec, int chunk, int pos) {
+__device__ __forceinline__ uint4 rotary_chunk(const DecodeParams& p, const elem_bits* head_vec, int chunk, int pos) {
     const uint4 raw = *reinterpret_cast<const uint4*>(head_vec + chunk * 8);
     const int d0 = chunk * 8, half = p.rotary_dim >> 1;
     if (d0 >= p.rotary_dim) return raw;
@@ -76,15 +76,15 @@ __device__ __forceinline__ uint4 rotary_chunk(const DecodeParams& p, const bf16_
     float x[8], y[8];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-        x[2 * e] = __uint_as_float(w[e] << 16);
-        x[2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
+        x[2 * e] = elem_lo_to_f32(w[e]);
+        x[2 * e + 1] = elem_hi_to_f32(w[e]);
     }
-    const bf16_bits* cs = p.rot_cos + static_cast<int64_t>(pos) * half;
-    const bf16_bits* sn = p.rot_sin + static_cast<int64_t>(pos) * half;
+    const elem_bits* cs = p.rot_cos + static_cast<int64_t>(pos) * half;
+    const elem_bits* sn = p.rot_sin + static_cast<int64_t>(pos) * half;
     if (p.rotary_interleaved) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const float c = bf16_to_f32(cs[(d0 >> 1) + i]), s = bf16_to_f32(sn[(d0 >> 1) + i]);
+            const float c = elem_to_f32(cs[(d0 >> 1) + i]), s = elem_to_f32(sn[(d0 >> 1) + i]);
             y[2 * i] = x[2 * i] * c - x[2 * i + 1] * s;
             y[2 * i + 1] = x[2 * i] * s + x[2 * i + 1] * c;
         }
@@ -95,12 +95,12 @@ __device__ __forceinline__ uint4 rotary_chunk(const DecodeParams& p, const bf16_
         const int i0 = left ? d0 : d0 - half;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-            const float o = (e & 1) ? __uint_as_float(ow[e >> 1] & 0xffff0000u) : __uint_as_float(ow[e >> 1] << 16);
-            const float c = bf16_to_f32(cs[i0 + e]), s = bf16_to_f32(sn[i0 + e]);
+            const float o = (e & 1) ? elem_hi_to_f32(ow[e >> 1]) : elem_lo_to_f32(ow[e >> 1]);
+            const float c = elem_to_f32(cs[i0 + e]), s = elem_to_f32(sn[i0 + e]);
             y[e] = left ? x[e] * c - o * s : x[e] * c + o * s;
         }
     }
-    return make_uint4(pack_bf16x2(y[0], y[1]), pack_bf16x2(y[2], y[3]), pack_bf16x2(y[4], y[5]), pack_bf16x2(y[6], y[7]));
+    return make_uint4(pack_elem2(y[0], y[1]), pack_elem2(y[2], y[3]), pack_elem2(y[4], y[5]), pack_elem2(y[6], y[7]));
 }
 
 constexpr int kVtPitch = kHeadDim + 8;                         // LDS row pitch (elements) of the V tile
@@ -118,7 +118,7 @@ void decode_append_kernel(const DecodeParams p) {
     const int b = static_cast<int>(r / p.seqlen_new);
     const int pos = (p.cache_seqlens ? p.cache_seqlens[b] : 0) + t;             // cache row, left padding included
     if (pos >= p.capacity) return;
-    const bf16_bits* kvec = p.knew + b * p.kn_batch + t * p.kn_row + h * p.kn_head;
+    const elem_bits* kvec = p.knew + b * p.kn_batch + t * p.kn_row + h * p.kn_head;
     const uint4 kv = p.rotary_dim > 0 ? rotary_chunk(p, kvec, chunk, pos) : *reinterpret_cast<const uint4*>(kvec + chunk * 8);
     const uint4 vv = *reinterpret_cast<const uint4*>(p.vnew + b * p.vn_batch + t * p.vn_row + h * p.vn_head + chunk * 8);
     *reinterpret_cast<uint4*>(p.kcache + cache_row_offset(p, b, pos, p.kc_batch, p.kc_row) + h * p.kc_head + chunk * 8) = kv;
@@ -142,7 +142,7 @@ void decode_rotate_q_kernel(const DecodeParams p) {
 template <bool kDirect>
 __global__ __launch_bounds__(64)
 void decode_split_kernel(const DecodeParams p) {
-    __shared__ __attribute__((aligned(16))) bf16_bits vt[kBlockN * kVtPitch];
+    __shared__ __attribute__((aligned(16))) elem_bits vt[kBlockN * kVtPitch];
     const int lane = threadIdx.x;
     const int n = lane & 15, g = lane >> 4;
     const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
@@ -173,13 +173,13 @@ void decode_split_kernel(const DecodeParams p) {
     int count = total - begin;
     if (count > per) count = per;
 
-    bf16x8 qf[4];
+    elem8 qf[4];
     {
-        const bf16_bits* qp = p.rotary_dim > 0
+        const elem_bits* qp = p.rotary_dim > 0
             ? p.q_rot + (static_cast<int64_t>(b) * p.num_heads_k * 16 + 16 * h + n) * kHeadDim + 8 * g
             : p.q + b * p.q_batch + (16 * h + n) * p.q_head + 8 * g;
 #pragma unroll
-        for (int c = 0; c < 4; ++c) qf[c] = *reinterpret_cast<const bf16x8*>(qp + 32 * c);
+        for (int c = 0; c < 4; ++c) qf[c] = *reinterpret_cast<const elem8*>(qp + 32 * c);
     }
     float m = -INFINITY, l = 0.f;
     floatx4 o[8];
@@ -191,17 +191,17 @@ void decode_split_kernel(const DecodeParams p) {
     for (int it = 0; it < count && j >= 0; ++it) {
         const int key0 = j * kBlockN;
         // a block never straddles two pages (page_size is a multiple of 64 and paged caches have no left padding)
-        const bf16_bits* kbase = p.kcache + cache_row_offset(p, b, lp + key0, p.kc_batch, p.kc_row) + h * p.kc_head;
-        const bf16_bits* vbase = p.vcache + cache_row_offset(p, b, lp + key0, p.vc_batch, p.vc_row) + h * p.vc_head;
+        const elem_bits* kbase = p.kcache + cache_row_offset(p, b, lp + key0, p.kc_batch, p.kc_row) + h * p.kc_head;
+        const elem_bits* vbase = p.vcache + cache_row_offset(p, b, lp + key0, p.vc_batch, p.vc_row) + h * p.vc_head;
         // K rows as A operands; rows past the end are clamped to a valid row and masked below
-        bf16x8 kreg[16];
+        elem8 kreg[16];
 #pragma unroll
         for (int kt = 0; kt < 4; ++kt) {
             int key = key0 + 16 * kt + n;
             key = key < L ? key : L - 1;
-            const bf16_bits* src = kbase + static_cast<int64_t>(key - key0) * p.kc_row + 8 * g;
+            const elem_bits* src = kbase + static_cast<int64_t>(key - key0) * p.kc_row + 8 * g;
 #pragma unroll
-            for (int c = 0; c < 4; ++c) kreg[kt * 4 + c] = *reinterpret_cast<const bf16x8*>(src + 32 * c);
+            for (int c = 0; c < 4; ++c) kreg[kt * 4 + c] = *reinterpret_cast<const elem8*>(src + 32 * c);
         }
         // V tile -> LDS, row-major
         uint4 vreg[16];
@@ -218,7 +218,7 @@ void decode_split_kernel(const DecodeParams p) {
             s[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int c = 0; c < 4; ++c)
-                s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[kt * 4 + c], qf[c], s[kt], 0, 0, 0);
+                s[kt] = IV2_MFMA(kreg[kt * 4 + c], qf[c], s[kt], 0, 0, 0);
         }
 #pragma unroll
         for (int u = 0; u < 16; ++u) {
@@ -255,13 +255,13 @@ void decode_split_kernel(const DecodeParams p) {
         m = m_new;
 #pragma unroll
         for (int dt = 0; dt < 8; ++dt) o[dt] *= alpha;
-        bf16x8 pf[2];
+        elem8 pf[2];
 #pragma unroll
         for (int cc = 0; cc < 2; ++cc)
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                pf[cc][e] = static_cast<__bf16>(s[2 * cc][e]);
-                pf[cc][4 + e] = static_cast<__bf16>(s[2 * cc + 1][e]);
+                pf[cc][e] = static_cast<elem_t>(s[2 * cc][e]);
+                pf[cc][4 + e] = static_cast<elem_t>(s[2 * cc + 1][e]);
             }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __builtin_amdgcn_s_barrier();                          // single-wavefront workgroup: orders the LDS tile
@@ -279,9 +279,9 @@ void decode_split_kernel(const DecodeParams p) {
                                  (static_cast<uint32_t>(vt[(key + 1) * kVtPitch + d]) << 16);
                 }
                 const uint4 raw = make_uint4(w[0], w[1], w[2], w[3]);
-                bf16x8 vf;
+                elem8 vf;
                 __builtin_memcpy(&vf, &raw, 16);
-                o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[cc], o[dt], 0, 0, 0);
+                o[dt] = IV2_MFMA(vf, pf[cc], o[dt], 0, 0, 0);
             }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __builtin_amdgcn_s_barrier();                          // tile consumed before the next block overwrites it
@@ -293,12 +293,12 @@ void decode_split_kernel(const DecodeParams p) {
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
     const float lse = l_tot > 0.f ? m * 0.69314718055994530942f + logf(l_tot) : (kDirect ? INFINITY : -INFINITY);
     if (kDirect) {
-        bf16_bits* op = p.out + b * p.o_batch + (16 * h + n) * p.o_head + 4 * g;
+        elem_bits* op = p.out + b * p.o_batch + (16 * h + n) * p.o_head + 4 * g;
 #pragma unroll
         for (int dt = 0; dt < 8; ++dt) {
             uint2 w;
-            w.x = pack_bf16x2(o[dt][0] * inv, o[dt][1] * inv);
-            w.y = pack_bf16x2(o[dt][2] * inv, o[dt][3] * inv);
+            w.x = pack_elem2(o[dt][0] * inv, o[dt][1] * inv);
+            w.y = pack_elem2(o[dt][2] * inv, o[dt][3] * inv);
             *reinterpret_cast<uint2*>(op + 16 * dt) = w;
         }
         if (g == 0) p.lse[static_cast<int64_t>(b) * p.num_heads_k * 16 + 16 * h + n] = lse;
@@ -338,19 +338,20 @@ void decode_combine_kernel(const DecodeParams p) {
     }
     const float inv = wsum > 0.f ? 1.f / wsum : 0.f;
     uint4 outv;
-    outv.x = pack_bf16x2(acc[0] * inv, acc[1] * inv);
-    outv.y = pack_bf16x2(acc[2] * inv, acc[3] * inv);
-    outv.z = pack_bf16x2(acc[4] * inv, acc[5] * inv);
-    outv.w = pack_bf16x2(acc[6] * inv, acc[7] * inv);
+    outv.x = pack_elem2(acc[0] * inv, acc[1] * inv);
+    outv.y = pack_elem2(acc[2] * inv, acc[3] * inv);
+    outv.z = pack_elem2(acc[4] * inv, acc[5] * inv);
+    outv.w = pack_elem2(acc[6] * inv, acc[7] * inv);
     *reinterpret_cast<uint4*>(p.out + b * p.o_batch + (16 * h + head) * p.o_head + d0) = outv;
     if ((tid & 15) == 0)
         p.lse[static_cast<int64_t>(b) * p.num_heads_k * 16 + 16 * h + head] = wsum > 0.f ? mx + logf(wsum) : INFINITY;
 }
 
-}  // namespace infllmv2
+}  // namespace IV2_NS
 
-using namespace infllmv2;
+using namespace IV2_NS;
 
+#ifndef IV2_F16        // element-type independent: defined once
 extern "C" int infllmv2_fwd_kvcache_num_splits(int batch, int num_heads_k, int requested) {
     if (requested > 0) return requested > 64 ? 64 : requested;
     // aim at ~4 single-wavefront workgroups per CU on a 256-CU device
@@ -360,17 +361,20 @@ extern "C" int infllmv2_fwd_kvcache_num_splits(int batch, int num_heads_k, int r
     if (s > 16) s = 16;
     return s;
 }
+#endif
 
 static size_t decode_partials_bytes(int batch, int num_heads_k, int num_splits) {
     if (num_splits <= 1) return 0;
     return static_cast<size_t>(batch) * num_heads_k * num_splits * 16 * (kHeadDim + 1) * sizeof(float);
 }
 
+#ifndef IV2_F16        // both element types are 2 bytes wide: defined once
 extern "C" size_t infllmv2_fwd_kvcache_workspace_bytes(int batch, int num_heads_k, int num_splits) {
     // per-split partial results, then room for the query turned by the rotary embedding
     return decode_partials_bytes(batch, num_heads_k, num_splits) +
-           static_cast<size_t>(batch) * num_heads_k * 16 * kHeadDim * sizeof(bf16_bits);
+           static_cast<size_t>(batch) * num_heads_k * 16 * kHeadDim * sizeof(elem_bits);
 }
+#endif
 
 static int fwd_kvcache_impl(void* stream, const void* q, void* kcache, void* vcache, const void* k_new,
                                     const void* v_new, const int32_t* cache_seqlens, void* out, float* softmax_lse,
@@ -418,12 +422,12 @@ static int fwd_kvcache_impl(void* stream, const void* q, void* kcache, void* vca
         IV2_CHECK(kcache_strides[s] % 8 == 0 && vcache_strides[s] % 8 == 0, "fwd_kvcache: cache strides must be multiples of 8 elements");
 
     DecodeParams p{};
-    p.q = static_cast<const bf16_bits*>(q);
-    p.kcache = static_cast<bf16_bits*>(kcache);
-    p.vcache = static_cast<bf16_bits*>(vcache);
-    p.knew = static_cast<const bf16_bits*>(k_new);
-    p.vnew = static_cast<const bf16_bits*>(v_new);
-    p.out = static_cast<bf16_bits*>(out);
+    p.q = static_cast<const elem_bits*>(q);
+    p.kcache = static_cast<elem_bits*>(kcache);
+    p.vcache = static_cast<elem_bits*>(vcache);
+    p.knew = static_cast<const elem_bits*>(k_new);
+    p.vnew = static_cast<const elem_bits*>(v_new);
+    p.out = static_cast<elem_bits*>(out);
     p.lse = softmax_lse;
     p.cache_seqlens = cache_seqlens;
     p.mask = blockmask;
@@ -437,9 +441,9 @@ static int fwd_kvcache_impl(void* stream, const void* q, void* kcache, void* vca
     p.scale_log2 = softmax_scale * 1.44269504088896340736f;
     p.cache_batch_idx = cache_batch_idx; p.leftpad = cache_leftpad;
     p.block_table = block_table; p.bt_batch = block_table_batch_stride; p.page_size = block_table ? page_block_size : 1;
-    p.rot_cos = static_cast<const bf16_bits*>(rotary_cos); p.rot_sin = static_cast<const bf16_bits*>(rotary_sin);
+    p.rot_cos = static_cast<const elem_bits*>(rotary_cos); p.rot_sin = static_cast<const elem_bits*>(rotary_sin);
     p.rotary_dim = rotary_cos ? rotary_dim : 0; p.rotary_interleaved = rotary_interleaved;
-    p.q_rot = reinterpret_cast<bf16_bits*>(static_cast<unsigned char*>(workspace) + decode_partials_bytes(batch, num_heads_k, num_splits));
+    p.q_rot = reinterpret_cast<elem_bits*>(static_cast<unsigned char*>(workspace) + decode_partials_bytes(batch, num_heads_k, num_splits));
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (k_new != nullptr) {
         IV2_CHECK(reinterpret_cast<uintptr_t>(k_new) % 16 == 0 && reinterpret_cast<uintptr_t>(v_new) % 16 == 0,
@@ -473,7 +477,7 @@ static int fwd_kvcache_impl(void* stream, const void* q, void* kcache, void* vca
     return 0;
 }
 
-extern "C" int infllmv2_fwd_kvcache(void* stream, const void* q, void* kcache, void* vcache, const void* k_new,
+extern "C" int IV2_ENTRY(infllmv2_fwd_kvcache)(void* stream, const void* q, void* kcache, void* vcache, const void* k_new,
                                     const void* v_new, const int32_t* cache_seqlens, void* out, float* softmax_lse,
                                     const uint64_t* blockmask, void* workspace, size_t workspace_bytes, int batch,
                                     int seqlen_q, int num_heads, int num_heads_k, int head_dim, int cache_capacity,
@@ -492,6 +496,7 @@ extern "C" int infllmv2_fwd_kvcache(void* stream, const void* q, void* kcache, v
                             rotary_interleaved);
 }
 
+#ifndef IV2_F16        // one such entry point in the library: bfloat16 only
 // ---- decode for callers that cannot allocate ---------------------------------------------------------------------
 //
 // The split partials and the turned query live in a device array that belongs to the library's code object: every GPU
@@ -549,3 +554,4 @@ extern "C" int infllmv2_fwd_kvcache_static(void* stream, const void* q, void* kc
                             cache_leftpad, block_table, block_table_batch_stride, page_block_size, rotary_cos, rotary_sin,
                             rotary_dim, rotary_interleaved);
 }
+#endif

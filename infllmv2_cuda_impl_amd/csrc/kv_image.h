@@ -19,7 +19,7 @@
 #pragma once
 #include "common.h"
 
-namespace infllmv2 {
+namespace IV2_NS {
 
 constexpr int kImageElems = kBlockN * kHeadDim;            // 8192 bf16 = 16 KiB per image
 
@@ -39,4 +39,4 @@ int launch_pack(hipStream_t st, const void* k, const void* v, const int32_t* cu_
                 size_t workspace_bytes, int batch, int64_t total_k, int num_heads_k, int max_seqlen_k,
                 const int64_t* k_strides, const int64_t* v_strides, bool backward_images, void* kt_image = nullptr);
 
-}  // namespace infllmv2
+}  // namespace IV2_NS

@@ -23,13 +23,13 @@
 #include "../../include/infllmv2_hip.h"
 #include <math.h>
 
-namespace infllmv2 {
+namespace IV2_NS {
 
 struct Stage1Params {
-    const bf16_bits* q;
-    const bf16_bits* k;              // fine compressed keys   (sum Lk, Hk, d)
-    const bf16_bits* c;              // coarse compressed keys (sum Lc, Hk, d)
-    bf16_bits* score;                // (Hk, total_q, row_stride); pooled output: (Hk, total_q, pool_len), dense
+    const elem_bits* q;
+    const elem_bits* k;              // fine compressed keys   (sum Lk, Hk, d)
+    const elem_bits* c;              // coarse compressed keys (sum Lc, Hk, d)
+    elem_bits* score;                // (Hk, total_q, row_stride); pooled output: (Hk, total_q, pool_len), dense
     const int* cu_seqlens_q;
     const int* cu_seqlens_k;
     const int* cu_seqlens_c;
@@ -77,7 +77,7 @@ __device__ __forceinline__ void s1_dma16(const void* base, uint32_t lane_off, ui
     asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
                  : : "v"(lane_off), "s"(base), "s"(lds_base) : "memory", "m0");
 }
-__device__ __forceinline__ void issue_tile(const bf16_bits* base, int row_stride, int key0, int L, uint32_t lds_tile,
+__device__ __forceinline__ void issue_tile(const elem_bits* base, int row_stride, int key0, int L, uint32_t lds_tile,
                                            int wave, int n, int g) {
 #pragma unroll
     for (int it = 0; it < 16 / kWavesS1; ++it) {
@@ -151,13 +151,13 @@ void stage1_kernel(const Stage1Params p) {
     const int tiles_f = (wg_vis_f + 63) >> 6;
 
     // Q as the A operand: r = lane % 16 is the head, g the k-group
-    bf16x8 qf[kTokPerWave][4];
+    elem8 qf[kTokPerWave][4];
 #pragma unroll
     for (int t = 0; t < kTokPerWave; ++t) {
         const int i = live[t] ? tok0 + t : Sq - 1;
-        const bf16_bits* qp = p.q + (static_cast<int64_t>(q0) + i) * p.q_tok_stride + h * p.q_kvh_stride + n * p.q_grp_stride + 8 * g;
+        const elem_bits* qp = p.q + (static_cast<int64_t>(q0) + i) * p.q_tok_stride + h * p.q_kvh_stride + n * p.q_grp_stride + 8 * g;
 #pragma unroll
-        for (int c = 0; c < 4; ++c) qf[t][c] = *reinterpret_cast<const bf16x8*>(qp + 32 * c);
+        for (int c = 0; c < 4; ++c) qf[t][c] = *reinterpret_cast<const elem8*>(qp + 32 * c);
     }
 
     // ---------------- pass 1: per-head log-sum-exp over the coarse keys ----------------
@@ -167,8 +167,8 @@ void stage1_kernel(const Stage1Params p) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) { m[t][e] = -INFINITY; l[t][e] = 0.f; }
 
-    const bf16_bits* cbase = p.c + static_cast<int64_t>(c0) * p.c_row_stride + h * p.c_head_stride;
-    const bf16_bits* kbase = p.k + static_cast<int64_t>(k0) * p.k_row_stride + h * p.k_head_stride;
+    const elem_bits* cbase = p.c + static_cast<int64_t>(c0) * p.c_row_stride + h * p.c_head_stride;
+    const elem_bits* kbase = p.k + static_cast<int64_t>(k0) * p.k_row_stride + h * p.k_head_stride;
     const uint32_t lds_tiles = __builtin_amdgcn_readfirstlane(s1_lds_addr(tile));
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
     const int c_stride = static_cast<int>(p.c_row_stride), k_stride = static_cast<int>(p.k_row_stride);
@@ -192,11 +192,11 @@ void stage1_kernel(const Stage1Params p) {
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 const uint4 raw = cur[(kt * 4 + c) * 64 + lane];
-                bf16x8 kf;
+                elem8 kf;
                 __builtin_memcpy(&kf, &raw, 16);
 #pragma unroll
                 for (int t = 0; t < kTokPerWave; ++t)
-                    s[t][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[t][c], kf, s[t][kt], 0, 0, 0);
+                    s[t][kt] = IV2_MFMA(qf[t][c], kf, s[t][kt], 0, 0, 0);
             }
         }
         // only the tile that holds a token's last visible key needs the per-key test
@@ -248,7 +248,7 @@ void stage1_kernel(const Stage1Params p) {
     if (tiles_f > 0) issue_tile(kbase, k_stride, 0, Lk, lds_tiles, wave_u, n, g);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    bf16_bits* out_rows[kTokPerWave];
+    elem_bits* out_rows[kTokPerWave];
     int bq[kTokPerWave];                                       // pooled output: the key block the token itself sits in
     float carry[kTokPerWave];                                  // pooled output: score of the last key of the previous tile
     {
@@ -263,11 +263,11 @@ void stage1_kernel(const Stage1Params p) {
         }
     }
     // value of a pooled entry that no visible key reaches
-    auto pool_rest = [&](int kb, int bq_t, float reached) -> bf16_bits {
+    auto pool_rest = [&](int kb, int bq_t, float reached) -> elem_bits {
         const bool forced = (kb < p.init_blocks) || (bq_t >= kb && bq_t <= kb + p.local_blocks);
         const int first = kb * kKeysPerBlock - 1;              // first key of the window (before clipping at 0)
         const bool empty = (first < 0 ? 0 : first) >= (Lk < p.score_cols ? Lk : p.score_cols);
-        return forced ? bf16_bits{0x7f80} : (empty ? bf16_bits{0xff80} : f32_to_bf16(reached));
+        return forced ? kElemPosInf : (empty ? kElemNegInf : f32_to_elem(reached));
     };
 
     for (int ti = 0; ti < tiles_f; ++ti) {
@@ -282,11 +282,11 @@ void stage1_kernel(const Stage1Params p) {
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 const uint4 raw = cur[(kt * 4 + c) * 64 + lane];
-                bf16x8 kf;
+                elem8 kf;
                 __builtin_memcpy(&kf, &raw, 16);
 #pragma unroll
                 for (int t = 0; t < kTokPerWave; ++t)
-                    s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[t][c], kf, s[t], 0, 0, 0);
+                    s[t] = IV2_MFMA(qf[t][c], kf, s[t], 0, 0, 0);
             }
 #pragma unroll
             for (int t = 0; t < kTokPerWave; ++t) {
@@ -304,7 +304,7 @@ void stage1_kernel(const Stage1Params p) {
             float mine = fold_rows32(fold_rows16(part[t][0], part[t][1]), fold_rows16(part[t][2], part[t][3]));
             mine = (col < vis_f[t]) ? mine : 0.f;              // keys the token may not see score 0
             if (!kPool) {
-                if (live[t] && col < p.score_cols) out_rows[t][col] = f32_to_bf16(mine);
+                if (live[t] && col < p.score_cols) out_rows[t][col] = f32_to_elem(mine);
             } else {
                 // block kb = col / 4 pools keys 4 kb - 1 .. 4 kb + 3: its quad and the last key of the quad before
                 float left = __shfl_up(mine, 1);
@@ -334,9 +334,9 @@ void stage1_kernel(const Stage1Params p) {
     }
 }
 
-}  // namespace infllmv2
+}  // namespace IV2_NS
 
-using namespace infllmv2;
+using namespace IV2_NS;
 
 namespace {
 
@@ -369,10 +369,10 @@ int launch_stage1(const char* who, void* stream, const void* q, const void* k, c
               "%s: compressed-key rows too far apart (row stride x max_seqlen_k must stay below 2^30 elements)", who);
     if (total_q == 0 || max_seqlen_q == 0) return 0;
     Stage1Params p{};
-    p.q = static_cast<const bf16_bits*>(q);
-    p.k = static_cast<const bf16_bits*>(k);
-    p.c = static_cast<const bf16_bits*>(v);
-    p.score = static_cast<bf16_bits*>(out);
+    p.q = static_cast<const elem_bits*>(q);
+    p.k = static_cast<const elem_bits*>(k);
+    p.c = static_cast<const elem_bits*>(v);
+    p.score = static_cast<elem_bits*>(out);
     p.cu_seqlens_q = cu_seqlens_q; p.cu_seqlens_k = cu_seqlens_k; p.cu_seqlens_c = cu_seqlens_v;
     p.q_tok_stride = q_strides[0]; p.q_grp_stride = q_strides[1]; p.q_kvh_stride = q_strides[2];
     p.k_row_stride = k_strides[0]; p.k_head_stride = k_strides[1];
@@ -400,7 +400,7 @@ int launch_stage1(const char* who, void* stream, const void* q, const void* k, c
 
 }  // namespace
 
-extern "C" int infllmv2_varlen_fwd_stage1(void* stream, const void* q, const void* k, const void* v, void* score,
+extern "C" int IV2_ENTRY(infllmv2_varlen_fwd_stage1)(void* stream, const void* q, const void* k, const void* v, void* score,
                                           const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
                                           const int32_t* cu_seqlens_v, int batch, int64_t total_q, int num_heads,
                                           int num_heads_k, int head_dim, int max_seqlen_q, int max_seqlen_k,
@@ -413,7 +413,7 @@ extern "C" int infllmv2_varlen_fwd_stage1(void* stream, const void* q, const voi
                          v_strides, score_head_stride, score_row_stride, softmax_scale, is_causal, nullptr);
 }
 
-extern "C" int infllmv2_varlen_fwd_stage1_pooled(void* stream, const void* q, const void* k, const void* v,
+extern "C" int IV2_ENTRY(infllmv2_varlen_fwd_stage1_pooled)(void* stream, const void* q, const void* k, const void* v,
                                                  void* pooled, const int32_t* cu_seqlens_q,
                                                  const int32_t* cu_seqlens_k, const int32_t* cu_seqlens_v,
                                                  const int32_t* cache_lens, int cache_len, int batch,

@@ -25,13 +25,13 @@
 #include "../../include/infllmv2_hip.h"
 #include <math.h>
 
-namespace infllmv2 {
+namespace IV2_NS {
 
 struct S1DecodeParams {
-    const bf16_bits* q;
-    const bf16_bits* k;              // fine compressed keys
-    const bf16_bits* c;              // coarse compressed keys (the key set of the log-sum-exp)
-    bf16_bits* out;
+    const elem_bits* q;
+    const elem_bits* k;              // fine compressed keys
+    const elem_bits* c;              // coarse compressed keys (the key set of the log-sum-exp)
+    elem_bits* out;
     float* partial;                  // (batch, Hk, splits_c, 32): log2-domain max of the 16 heads, then their sums
     const int* cu_seqlens_q;         // null: sequence b's query is row b
     const int* cu_seqlens_k;         // packed keys: rows [cu[b], cu[b+1]); null: cache layout, k_lens[b] rows at b * k_batch
@@ -62,8 +62,8 @@ __device__ __forceinline__ int s1d_visible(int s, int L, bool causal) {
 
 struct S1DecodeSeq {
     int q_row, Sq, Lk, Lc;
-    const bf16_bits* kbase;
-    const bf16_bits* cbase;
+    const elem_bits* kbase;
+    const elem_bits* cbase;
 };
 
 __device__ __forceinline__ S1DecodeSeq s1d_sequence(const S1DecodeParams& p, int b, int h) {
@@ -82,22 +82,22 @@ __device__ __forceinline__ S1DecodeSeq s1d_sequence(const S1DecodeParams& p, int
 
 // 64 keys x 128 d as MFMA B operands: register kt*4 + c of lane (n, g) = K[key0 + 16 kt + n][32 c + 8 g ..].
 // Rows past the last key read the last key (finite values that every consumer masks).
-__device__ __forceinline__ void s1d_load_tile(bf16x8 (&t)[16], const bf16_bits* base, int64_t row_stride, int key0,
+__device__ __forceinline__ void s1d_load_tile(elem8 (&t)[16], const elem_bits* base, int64_t row_stride, int key0,
                                               int L, int n, int g) {
 #pragma unroll
     for (int kt = 0; kt < 4; ++kt) {
         int row = key0 + 16 * kt + n;
         row = row < L ? row : L - 1;
-        const bf16_bits* src = base + row * row_stride + 8 * g;
+        const elem_bits* src = base + row * row_stride + 8 * g;
 #pragma unroll
-        for (int c = 0; c < 4; ++c) t[kt * 4 + c] = *reinterpret_cast<const bf16x8*>(src + 32 * c);
+        for (int c = 0; c < 4; ++c) t[kt * 4 + c] = *reinterpret_cast<const elem8*>(src + 32 * c);
     }
 }
 
-__device__ __forceinline__ void s1d_load_q(bf16x8 (&qf)[4], const S1DecodeParams& p, const S1DecodeSeq& s, int h, int n, int g) {
-    const bf16_bits* qp = p.q + static_cast<int64_t>(s.q_row) * p.q_tok_stride + h * p.q_kvh_stride + n * p.q_grp_stride + 8 * g;
+__device__ __forceinline__ void s1d_load_q(elem8 (&qf)[4], const S1DecodeParams& p, const S1DecodeSeq& s, int h, int n, int g) {
+    const elem_bits* qp = p.q + static_cast<int64_t>(s.q_row) * p.q_tok_stride + h * p.q_kvh_stride + n * p.q_grp_stride + 8 * g;
 #pragma unroll
-    for (int c = 0; c < 4; ++c) qf[c] = *reinterpret_cast<const bf16x8*>(qp + 32 * c);
+    for (int c = 0; c < 4; ++c) qf[c] = *reinterpret_cast<const elem8*>(qp + 32 * c);
 }
 
 // run [t0, t1) of `tiles` tiles that split `split` of `splits` works on
@@ -120,19 +120,19 @@ void stage1_decode_lse_kernel(const S1DecodeParams p) {
     int t0, t1;
     s1d_run((vis_c + 63) >> 6, p.splits_c, split, t0, t1);
 
-    bf16x8 qf[4];
+    elem8 qf[4];
     s1d_load_q(qf, p, sq, h, n, g);
     float m[4], l[4];                                          // head 4g + e over the keys == n (mod 16) of the run
 #pragma unroll
     for (int e = 0; e < 4; ++e) { m[e] = -INFINITY; l[e] = 0.f; }
 
-    auto consume = [&](const bf16x8 (&t)[16], int ti) {
+    auto consume = [&](const elem8 (&t)[16], int ti) {
         floatx4 s[4];
 #pragma unroll
         for (int kt = 0; kt < 4; ++kt) {
             s[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int c = 0; c < 4; ++c) s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[c], t[kt * 4 + c], s[kt], 0, 0, 0);
+            for (int c = 0; c < 4; ++c) s[kt] = IV2_MFMA(qf[c], t[kt * 4 + c], s[kt], 0, 0, 0);
         }
         const bool cut = (ti + 1) * 64 > vis_c;
 #pragma unroll
@@ -155,7 +155,7 @@ void stage1_decode_lse_kernel(const S1DecodeParams p) {
         }
     };
 
-    bf16x8 ta[16], tb[16];
+    elem8 ta[16], tb[16];
     if (t0 < t1) s1d_load_tile(ta, sq.cbase, p.c_row_stride, t0 * 64, sq.Lc, n, g);
     if (t0 + 1 < t1) s1d_load_tile(tb, sq.cbase, p.c_row_stride, (t0 + 1) * 64, sq.Lc, n, g);
     for (int ti = t0; ti < t1; ti += 2) {
@@ -218,10 +218,10 @@ void stage1_decode_score_kernel(const S1DecodeParams p) {
     const bool owns_tail = tiles == 0 ? split == 0 : (t0 < t1 && t1 == tiles);
     if (t0 >= t1 && !owns_tail) return;
 
-    bf16x8 qf[4];
+    elem8 qf[4];
     s1d_load_q(qf, p, sq, h, n, g);
     // the first two tiles are requested before anything waits on memory
-    bf16x8 ta[16], tb[16];
+    elem8 ta[16], tb[16];
     if (t0 < t1) s1d_load_tile(ta, sq.kbase, p.k_row_stride, t0 * 64, sq.Lk, n, g);
     if (t0 + 1 < t1) s1d_load_tile(tb, sq.kbase, p.k_row_stride, (t0 + 1) * 64, sq.Lk, n, g);
     // log-sum-exp of head 4g + e: the partials of the coarse runs merged in run order
@@ -242,20 +242,20 @@ void stage1_decode_score_kernel(const S1DecodeParams p) {
         }
     }
     const int64_t out_row = static_cast<int64_t>(h) * p.out_head_stride + static_cast<int64_t>(sq.q_row) * p.out_row_stride;
-    bf16_bits* out = p.out + out_row;
+    elem_bits* out = p.out + out_row;
     const int bq = kPool ? ((p.cache_lens ? p.cache_lens[b] : p.cache_len) / kBlockN) : 0;   // the query's own key block
     const int Lk_cols = sq.Lk < p.cols ? sq.Lk : p.cols;
-    auto pool_rest = [&](int kb, float reached) -> bf16_bits {
+    auto pool_rest = [&](int kb, float reached) -> elem_bits {
         const bool forced = (kb < p.init_blocks) || (bq >= kb && bq <= kb + p.local_blocks);
         const int first = kb * 4 - 1;
         const bool empty = (first < 0 ? 0 : first) >= Lk_cols;
-        return forced ? bf16_bits{0x7f80} : (empty ? bf16_bits{0xff80} : f32_to_bf16(reached));
+        return forced ? kElemPosInf : (empty ? kElemNegInf : f32_to_elem(reached));
     };
     // one 16-key group: this lane's four heads summed for key 16 kt + n of the tile
-    auto group_part = [&](const bf16x8* t4) -> float {
+    auto group_part = [&](const elem8* t4) -> float {
         floatx4 s = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int c = 0; c < 4; ++c) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[c], t4[c], s, 0, 0, 0);
+        for (int c = 0; c < 4; ++c) s = IV2_MFMA(qf[c], t4[c], s, 0, 0, 0);
         float sum = 0.f;
 #pragma unroll
         for (int e = 0; e < 4; ++e) sum += __builtin_amdgcn_exp2f(s[e] * p.scale_log2 - lse2[e]);
@@ -264,18 +264,18 @@ void stage1_decode_score_kernel(const S1DecodeParams p) {
 
     float carry = 0.f;                                         // score of the last key before the current tile
     if (kPool && t0 > 0 && t0 < t1) {
-        bf16x8 t4[4];
+        elem8 t4[4];
         const int row = t0 * 64 - 16 + n;                      // keys of the last group of tile t0 - 1: all exist
-        const bf16_bits* src = sq.kbase + row * p.k_row_stride + 8 * g;
+        const elem_bits* src = sq.kbase + row * p.k_row_stride + 8 * g;
 #pragma unroll
-        for (int c = 0; c < 4; ++c) t4[c] = *reinterpret_cast<const bf16x8*>(src + 32 * c);
+        for (int c = 0; c < 4; ++c) t4[c] = *reinterpret_cast<const elem8*>(src + 32 * c);
         const float part3 = group_part(t4);
         float prev = s1d_fold_rows32(s1d_fold_rows16(0.f, 0.f), s1d_fold_rows16(0.f, part3));
         prev = (t0 * 64 - 64 + lane < vis_f) ? prev : 0.f;
         carry = __shfl(prev, 63);
     }
 
-    auto consume = [&](const bf16x8 (&t)[16], int ti) {
+    auto consume = [&](const elem8 (&t)[16], int ti) {
         float part[4];
 #pragma unroll
         for (int kt = 0; kt < 4; ++kt) part[kt] = group_part(&t[kt * 4]);
@@ -283,7 +283,7 @@ void stage1_decode_score_kernel(const S1DecodeParams p) {
         float mine = s1d_fold_rows32(s1d_fold_rows16(part[0], part[1]), s1d_fold_rows16(part[2], part[3]));
         mine = (col < vis_f) ? mine : 0.f;
         if (!kPool) {
-            if (col < p.cols) out[col] = f32_to_bf16(mine);
+            if (col < p.cols) out[col] = f32_to_elem(mine);
         } else {
             float left = __shfl_up(mine, 1);
             if (lane == 0) left = carry;
@@ -314,9 +314,9 @@ void stage1_decode_score_kernel(const S1DecodeParams p) {
     }
 }
 
-}  // namespace infllmv2
+}  // namespace IV2_NS
 
-using namespace infllmv2;
+using namespace IV2_NS;
 
 namespace {
 
@@ -338,13 +338,15 @@ void s1d_splits(int batch, int num_heads_k, int max_keys, int max_coarse, int& s
 
 }  // namespace
 
+#ifndef IV2_F16        // element-type independent: defined once
 extern "C" size_t infllmv2_stage1_decode_workspace_bytes(int batch, int num_heads_k, int max_seqlen_k, int max_seqlen_v) {
     int sf, sc;
     s1d_splits(batch, num_heads_k, max_seqlen_k, max_seqlen_v, sf, sc);
     return static_cast<size_t>(batch > 0 ? batch : 0) * (num_heads_k > 0 ? num_heads_k : 0) * sc * 32 * sizeof(float);
 }
+#endif
 
-extern "C" int infllmv2_stage1_decode(void* stream, const void* q, const void* k, const void* v, void* out,
+extern "C" int IV2_ENTRY(infllmv2_stage1_decode)(void* stream, const void* q, const void* k, const void* v, void* out,
                                       const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, const int32_t* k_lens,
                                       const int32_t* cu_seqlens_v, const int32_t* v_lens, void* workspace,
                                       size_t workspace_bytes, int batch, int num_heads, int num_heads_k, int head_dim,
@@ -381,10 +383,10 @@ extern "C" int infllmv2_stage1_decode(void* stream, const void* q, const void* k
     IV2_CHECK(workspace != nullptr && reinterpret_cast<uintptr_t>(workspace) % 16 == 0 &&
               workspace_bytes >= infllmv2_stage1_decode_workspace_bytes(batch, num_heads_k, max_seqlen_k, max_seqlen_v),
               "%s: workspace missing, misaligned or too small", who);
-    p.q = static_cast<const bf16_bits*>(q);
-    p.k = static_cast<const bf16_bits*>(k);
-    p.c = static_cast<const bf16_bits*>(v);
-    p.out = static_cast<bf16_bits*>(out);
+    p.q = static_cast<const elem_bits*>(q);
+    p.k = static_cast<const elem_bits*>(k);
+    p.c = static_cast<const elem_bits*>(v);
+    p.out = static_cast<elem_bits*>(out);
     p.partial = static_cast<float*>(workspace);
     p.cu_seqlens_q = cu_seqlens_q;
     p.cu_seqlens_k = cu_seqlens_k; p.k_lens = k_lens;

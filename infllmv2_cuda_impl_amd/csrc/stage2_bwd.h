@@ -2,24 +2,24 @@
 #pragma once
 #include "common.h"
 
-namespace infllmv2 {
+namespace IV2_NS {
 
 constexpr float kLog2e = 1.44269504088896340736f;
 
 struct BwdParams {
-    const bf16_bits* q;
-    const bf16_bits* dout;
-    const bf16_bits* out;
-    bf16_bits* dq;
+    const elem_bits* q;
+    const elem_bits* dout;
+    const elem_bits* out;
+    elem_bits* dq;
     const float* lse;
     float* dsum;                    // (Hk, total_q * 16): D of head 16h+g of token t at [h][16 t + g]
     float* rowstat;                 // (Hk, total_q, 32): LSE * log2(e) of the 16 heads, then D of the 16 heads
-    const bf16_bits* kimg;          // K, K-image order
-    const bf16_bits* vimg_r;        // V, K-image order
+    const elem_bits* kimg;          // K, K-image order
+    const elem_bits* vimg_r;        // V, K-image order
     float* dk_acc;                  // (total_k, Hk, 128) fp32
     float* dv_acc;
-    bf16_bits* dk;
-    bf16_bits* dv;
+    elem_bits* dk;
+    elem_bits* dv;
     const uint64_t* fwd_mask;       // (Hk, total_q, n64_fwd) or null
     const uint64_t* bwd_mask;       // (Hk, k_blocks, n64_bwd) or null
     const int* cu_seqlens_q;
@@ -41,8 +41,8 @@ struct BwdParams {
     // dS hand-off: the column kernel stores the dS^T tile (64 keys x 16 heads, bf16, 2 KiB) of every (token, block)
     // pair it forms, and dQ is computed from those tiles and K alone instead of recomputing S and dP from K and V.
     // The tile of the r-th selected block of a token's mask row is slot (kv head, token, r); null: no hand-off.
-    bf16_bits* ds_buf;              // (Hk, total_q, max_sel + 1, 64, 16); slot max_sel of a row takes misdirected stores
-    const bf16_bits* ktimg;         // K in V-image order (keys contracted): the A operand of dQ^T = K^T dS^T
+    elem_bits* ds_buf;              // (Hk, total_q, max_sel + 1, 64, 16); slot max_sel of a row takes misdirected stores
+    const elem_bits* ktimg;         // K in V-image order (keys contracted): the A operand of dQ^T = K^T dS^T
     const uint4* rankinfo;          // (Hk, total_q, n64_fwd): {mask word lo, hi, set bits in the row's earlier words, 0}
     int max_sel;                    // upper bound of set bits per mask row
 };
@@ -58,4 +58,4 @@ int launch_bwd_dq_handoff(hipStream_t st, const BwdParams& p, int batch, int max
 int launch_bwd_dkdv_reduce(hipStream_t st, const BwdParams& p, int batch);
 constexpr int kDkdvSlice = 512;     // query tokens per dK/dV work item (slices are cut on the packed token axis)
 
-}  // namespace infllmv2
+}  // namespace IV2_NS

@@ -24,7 +24,7 @@
 #include <math.h>
 #include <stdlib.h>
 
-namespace infllmv2 {
+namespace IV2_NS {
 
 // ---------------------------------------------------------------------------------------------
 // preprocessing: D = rowsum(dO * O) (compute_dot_do_o, flash_bwd_preprocess_kernel.h:56-137) and, per token,
@@ -44,8 +44,8 @@ void bwd_prep_kernel(const BwdParams p) {
     float acc = 0.f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        acc += bf16_to_f32(static_cast<bf16_bits>(dw[i] & 0xffff)) * bf16_to_f32(static_cast<bf16_bits>(ow[i] & 0xffff));
-        acc += bf16_to_f32(static_cast<bf16_bits>(dw[i] >> 16)) * bf16_to_f32(static_cast<bf16_bits>(ow[i] >> 16));
+        acc += elem_to_f32(static_cast<elem_bits>(dw[i] & 0xffff)) * elem_to_f32(static_cast<elem_bits>(ow[i] & 0xffff));
+        acc += elem_to_f32(static_cast<elem_bits>(dw[i] >> 16)) * elem_to_f32(static_cast<elem_bits>(ow[i] >> 16));
     }
 #pragma unroll
     for (int off = 1; off < 16; off <<= 1) acc += __shfl_xor(acc, off);
@@ -77,8 +77,8 @@ void bwd_convert_dkdv_kernel(const BwdParams p) {
     const float4 a = *reinterpret_cast<const float4*>(p.dk_acc + rh * kHeadDim + d4 * 4);
     const float4 c = *reinterpret_cast<const float4*>(p.dv_acc + rh * kHeadDim + d4 * 4);
     uint2 ka, va;
-    ka.x = pack_bf16x2(a.x, a.y); ka.y = pack_bf16x2(a.z, a.w);
-    va.x = pack_bf16x2(c.x, c.y); va.y = pack_bf16x2(c.z, c.w);
+    ka.x = pack_elem2(a.x, a.y); ka.y = pack_elem2(a.z, a.w);
+    va.x = pack_elem2(c.x, c.y); va.y = pack_elem2(c.z, c.w);
     *reinterpret_cast<uint2*>(p.dk + row * p.dk_row + h * p.dk_head + d4 * 4) = ka;
     *reinterpret_cast<uint2*>(p.dv + row * p.dv_row + h * p.dv_head + d4 * 4) = va;
 }
@@ -131,10 +131,11 @@ static BwdLayout bwd_layout(int batch, int64_t total_q, int64_t total_k, int num
     return L;
 }
 
-}  // namespace infllmv2
+}  // namespace IV2_NS
 
-using namespace infllmv2;
+using namespace IV2_NS;
 
+#ifndef IV2_F16        // both element types are 2 bytes wide: defined once
 extern "C" size_t infllmv2_varlen_bwd_workspace_bytes(int batch, int64_t total_q, int64_t total_k, int num_heads_k,
                                                       int max_seqlen_k) {
     return bwd_layout(batch, total_q, total_k, num_heads_k, max_seqlen_k).total;
@@ -152,8 +153,9 @@ extern "C" size_t infllmv2_varlen_bwd_workspace_bytes_ex(int batch, int64_t tota
                                    n_uint64_per_row > 0 ? max_selected_blocks : 0, n_uint64_per_row);
     return deterministic ? L.det_total : L.total;
 }
+#endif
 
-extern "C" int infllmv2_varlen_bwd(void* stream, const void* dout, const void* q, const void* k, const void* v,
+extern "C" int IV2_ENTRY(infllmv2_varlen_bwd)(void* stream, const void* dout, const void* q, const void* k, const void* v,
                                    const void* out, const float* softmax_lse, void* dq, void* dk, void* dv,
                                    const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
                                    const uint64_t* fwd_blockmask, void* workspace, size_t workspace_bytes, int batch,
@@ -192,21 +194,21 @@ extern "C" int infllmv2_varlen_bwd(void* stream, const void* dout, const void* q
     unsigned char* ws = static_cast<unsigned char*>(workspace);
 
     BwdParams p{};
-    p.q = static_cast<const bf16_bits*>(q);
-    p.dout = static_cast<const bf16_bits*>(dout);
-    p.out = static_cast<const bf16_bits*>(out);
-    p.dq = static_cast<bf16_bits*>(dq);
+    p.q = static_cast<const elem_bits*>(q);
+    p.dout = static_cast<const elem_bits*>(dout);
+    p.out = static_cast<const elem_bits*>(out);
+    p.dq = static_cast<elem_bits*>(dq);
     p.lse = softmax_lse;
     p.dsum = reinterpret_cast<float*>(ws + L.dsum);
     p.rowstat = reinterpret_cast<float*>(ws + L.rowstat);
     const int64_t n_slots = image_slots(total_k, batch);
     const int64_t img_elems = n_slots * num_heads_k * kImageElems;
-    p.kimg = reinterpret_cast<const bf16_bits*>(ws + L.images);
+    p.kimg = reinterpret_cast<const elem_bits*>(ws + L.images);
     p.vimg_r = p.kimg + img_elems;
     p.dk_acc = reinterpret_cast<float*>(ws + L.dk_acc);
     p.dv_acc = reinterpret_cast<float*>(ws + L.dv_acc);
-    p.dk = static_cast<bf16_bits*>(dk);
-    p.dv = static_cast<bf16_bits*>(dv);
+    p.dk = static_cast<elem_bits*>(dk);
+    p.dv = static_cast<elem_bits*>(dv);
     p.fwd_mask = fwd_blockmask;
     p.cu_seqlens_q = cu_seqlens_q; p.cu_seqlens_k = cu_seqlens_k;
     p.q_tok = q_strides[0]; p.q_grp = q_strides[1]; p.q_kvh = q_strides[2];
@@ -256,8 +258,8 @@ extern "C" int infllmv2_varlen_bwd(void* stream, const void* dout, const void* q
         if (handoff) {
             // the column kernel runs first and leaves the dS^T tile of every pair for the dQ kernel
             p.rankinfo = reinterpret_cast<const uint4*>(ws + L.rankinfo);
-            p.ds_buf = reinterpret_cast<bf16_bits*>(ws + L.ds_buf);
-            p.ktimg = reinterpret_cast<const bf16_bits*>(ws + L.ktimg);
+            p.ds_buf = reinterpret_cast<elem_bits*>(ws + L.ds_buf);
+            p.ktimg = reinterpret_cast<const elem_bits*>(ws + L.ktimg);
             p.max_sel = max_selected_blocks;
             const int64_t rows = static_cast<int64_t>(num_heads_k) * total_q;
             hipLaunchKernelGGL(bwd_rankinfo_kernel, dim3(static_cast<unsigned>((rows + 255) / 256)), dim3(256), 0, st,

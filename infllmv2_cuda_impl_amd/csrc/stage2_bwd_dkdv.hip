@@ -26,7 +26,7 @@
 #include "stage2_bwd.h"
 #include <math.h>
 
-namespace infllmv2 {
+namespace IV2_NS {
 
 constexpr int kColSlice = kDkdvSlice;                          // query tokens per work item
 constexpr int kGroupSlices = 4;                                // slices that pool their light members
@@ -60,16 +60,16 @@ __device__ __forceinline__ void dma4(const void* base, uint32_t lane_off, uint32
 // Written as one asm block because the compiler cannot see that these are MFMAs: an MFMA must not read a VGPR in
 // the two issue slots after a VALU instruction wrote it, so the block opens with the wait states itself and
 // contains nothing but MFMAs; only MFMAs touch these accumulators inside the main loop.
-__device__ __forceinline__ void mfma_dtile(floatx4 (&acc)[4], const bf16x8& a, const bf16x8 (&b)[4]) {
+__device__ __forceinline__ void mfma_dtile(floatx4 (&acc)[4], const elem8& a, const elem8 (&b)[4]) {
     int4v ai, bi[4];
     __builtin_memcpy(&ai, &a, 16);
 #pragma unroll
     for (int kt = 0; kt < 4; ++kt) __builtin_memcpy(&bi[kt], &b[kt], 16);
     asm("s_nop 1\n\t"
-        "v_mfma_f32_16x16x32_bf16 %0, %4, %5, %0\n\t"
-        "v_mfma_f32_16x16x32_bf16 %1, %4, %6, %1\n\t"
-        "v_mfma_f32_16x16x32_bf16 %2, %4, %7, %2\n\t"
-        "v_mfma_f32_16x16x32_bf16 %3, %4, %8, %3"
+        IV2_MFMA_ASM " %0, %4, %5, %0\n\t"
+        IV2_MFMA_ASM " %1, %4, %6, %1\n\t"
+        IV2_MFMA_ASM " %2, %4, %7, %2\n\t"
+        IV2_MFMA_ASM " %3, %4, %8, %3"
         : "+a"(acc[0]), "+a"(acc[1]), "+a"(acc[2]), "+a"(acc[3])
         : "v"(ai), "v"(bi[0]), "v"(bi[1]), "v"(bi[2]), "v"(bi[3]));
 }
@@ -164,15 +164,15 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
     __syncthreads();
 
     // ---- K and V of the block: B operands, resident in registers ----
-    bf16x8 kreg[4][4], vreg[4][4];
+    elem8 kreg[4][4], vreg[4][4];
     {
         const int64_t img = (static_cast<int64_t>(h) * p.n_slots + image_slot0(p.cu_seqlens_k, b) + j) * kImageElems + lane * 8;
 #pragma unroll
         for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
-                kreg[kt][c] = *reinterpret_cast<const bf16x8*>(p.kimg + img + (kt * 4 + c) * 512);
-                vreg[kt][c] = *reinterpret_cast<const bf16x8*>(p.vimg_r + img + (kt * 4 + c) * 512);
+                kreg[kt][c] = *reinterpret_cast<const elem8*>(p.kimg + img + (kt * 4 + c) * 512);
+                vreg[kt][c] = *reinterpret_cast<const elem8*>(p.vimg_r + img + (kt * 4 + c) * 512);
             }
     }
     floatx4 dKt[8][4], dVt[8][4];                              // [d tile][key tile]: lane (n, g) holds [16 dt + 4 g + e][16 kt + n]
@@ -213,8 +213,8 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
     const uint32_t q_lane = static_cast<uint32_t>((dma_head * p.q_grp + 8 * dma_piece) * 2);   // byte offsets inside one token and KV head
     const uint32_t do_lane = static_cast<uint32_t>((dma_head * p.do_grp + 8 * dma_piece) * 2);
     const uint32_t stat_lane = static_cast<uint32_t>((lane & 31) * 4);
-    const bf16_bits* q_head = p.q + static_cast<int64_t>(h) * p.q_kvh;
-    const bf16_bits* do_head = p.dout + static_cast<int64_t>(h) * p.do_kvh;
+    const elem_bits* q_head = p.q + static_cast<int64_t>(h) * p.q_kvh;
+    const elem_bits* do_head = p.dout + static_cast<int64_t>(h) * p.do_kvh;
     const float* stat_head = p.rowstat + static_cast<int64_t>(h) * p.total_q * 32;
     const bool handoff = p.ds_buf != nullptr;                  // uniform over the launch
     const uint32_t rank_lane = static_cast<uint32_t>((lane & 3) * 4);
@@ -316,8 +316,8 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
         const float lse_b[4] = {lb.x, lb.y, lb.z, lb.w};
         const bool edge = (lim_a < kBlockN - 1) || (lim_b < kBlockN - 1);
         // hand-off: where the dS^T tiles of this pair go (rank of block j among the set bits of each token's mask row)
-        bf16_bits* ds_a = nullptr;
-        bf16_bits* ds_b = nullptr;
+        elem_bits* ds_a = nullptr;
+        elem_bits* ds_b = nullptr;
         if (handoff) {
             const uint4 ra = *reinterpret_cast<const uint4*>(st + 16896);
             const uint4 rb = *reinterpret_cast<const uint4*>(st + 16896 + 256);
@@ -341,7 +341,7 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
         //   C  dV^T += dO^T P                  while the VALU forms dS = P (dP - D) (bf16)
         //   D  dK^T += Q^T dS
         const uint4* frag = reinterpret_cast<const uint4*>(st) + frag_unit;      // tile t, chunk c at frag[t * 256 + c * 64]
-        bf16x8 pfr[4], dsfr[4];                                // per key tile: [token a heads 4g..4g+3 | token b heads 4g..4g+3]
+        elem8 pfr[4], dsfr[4];                                // per key tile: [token a heads 4g..4g+3 | token b heads 4g..4g+3]
         floatx4 sa[4], sb[4], dpa[4], dpb[4];
         // the dP accumulators start at -D, so that dS = P (dP - D) is one multiplication per element
         const floatx4 negD_a = {-Da.x, -Da.y, -Da.z, -Da.w}, negD_b = {-Db.x, -Db.y, -Db.z, -Db.w};
@@ -356,13 +356,13 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 if (c < 3) { fr[(c + 1) & 1][0] = frag[(c + 1) * 64]; fr[(c + 1) & 1][1] = frag[256 + (c + 1) * 64]; }
-                bf16x8 qa, qb;
+                elem8 qa, qb;
                 __builtin_memcpy(&qa, &fr[c & 1][0], 16);
                 __builtin_memcpy(&qb, &fr[c & 1][1], 16);
 #pragma unroll
                 for (int kt = 0; kt < 4; ++kt) {
-                    sa[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa, kreg[kt][c], sa[kt], 0, 0, 0);
-                    sb[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qb, kreg[kt][c], sb[kt], 0, 0, 0);
+                    sa[kt] = IV2_MFMA(qa, kreg[kt][c], sa[kt], 0, 0, 0);
+                    sb[kt] = IV2_MFMA(qb, kreg[kt][c], sb[kt], 0, 0, 0);
                 }
             }
         }
@@ -373,13 +373,13 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 if (c < 3) { fr[(c + 1) & 1][0] = frag[512 + (c + 1) * 64]; fr[(c + 1) & 1][1] = frag[768 + (c + 1) * 64]; }
-                bf16x8 doa, dob;
+                elem8 doa, dob;
                 __builtin_memcpy(&doa, &fr[c & 1][0], 16);
                 __builtin_memcpy(&dob, &fr[c & 1][1], 16);
 #pragma unroll
                 for (int kt = 0; kt < 4; ++kt) {
-                    dpa[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(doa, vreg[kt][c], dpa[kt], 0, 0, 0);
-                    dpb[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(dob, vreg[kt][c], dpb[kt], 0, 0, 0);
+                    dpa[kt] = IV2_MFMA(doa, vreg[kt][c], dpa[kt], 0, 0, 0);
+                    dpb[kt] = IV2_MFMA(dob, vreg[kt][c], dpb[kt], 0, 0, 0);
                 }
                 {   // P of key tile c, kept in fp32 in place of S
                     const int kt = c;
@@ -389,8 +389,8 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
                         float xb = __builtin_amdgcn_exp2f(sb[kt][e] * p.scale_log2 - lse_b[e]);
                         sa[kt][e] = xa;
                         sb[kt][e] = xb;
-                        pfr[kt][e] = static_cast<__bf16>(xa);
-                        pfr[kt][4 + e] = static_cast<__bf16>(xb);
+                        pfr[kt][e] = static_cast<elem_t>(xa);
+                        pfr[kt][4 + e] = static_cast<elem_t>(xb);
                     }
                 }
             }
@@ -405,8 +405,8 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
                 for (int e = 0; e < 4; ++e) {
                     sa[kt][e] = off_a ? 0.f : sa[kt][e];
                     sb[kt][e] = off_b ? 0.f : sb[kt][e];
-                    pfr[kt][e] = static_cast<__bf16>(sa[kt][e]);
-                    pfr[kt][4 + e] = static_cast<__bf16>(sb[kt][e]);
+                    pfr[kt][e] = static_cast<elem_t>(sa[kt][e]);
+                    pfr[kt][4 + e] = static_cast<elem_t>(sb[kt][e]);
                 }
             }
         }
@@ -420,7 +420,7 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
 #pragma unroll
             for (int dt = 0; dt < 8; ++dt) {
                 if (dt < 7) { t_a[(dt + 1) & 1] = lds_read_tr(tr_at(8192, dt + 1)); t_b[(dt + 1) & 1] = lds_read_tr(tr_at(12288, dt + 1)); }
-                bf16x8 ad;
+                elem8 ad;
                 __builtin_memcpy(&ad, &t_a[dt & 1], 8);
                 __builtin_memcpy(reinterpret_cast<unsigned char*>(&ad) + 8, &t_b[dt & 1], 8);
                 mfma_dtile(dVt[dt], ad, pfr);
@@ -428,8 +428,8 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
                     const int kt = dt >> 1, e0 = (dt & 1) * 2;
 #pragma unroll
                     for (int e = e0; e < e0 + 2; ++e) {
-                        dsfr[kt][e] = static_cast<__bf16>(sa[kt][e] * dpa[kt][e]);
-                        dsfr[kt][4 + e] = static_cast<__bf16>(sb[kt][e] * dpb[kt][e]);
+                        dsfr[kt][e] = static_cast<elem_t>(sa[kt][e] * dpa[kt][e]);
+                        dsfr[kt][4 + e] = static_cast<elem_t>(sb[kt][e] * dpb[kt][e]);
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);
@@ -454,7 +454,7 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
 #pragma unroll
             for (int dt = 0; dt < 8; ++dt) {
                 if (dt < 7) { t_a[(dt + 1) & 1] = lds_read_tr(tr_at(0, dt + 1)); t_b[(dt + 1) & 1] = lds_read_tr(tr_at(4096, dt + 1)); }
-                bf16x8 aq;
+                elem8 aq;
                 __builtin_memcpy(&aq, &t_a[dt & 1], 8);
                 __builtin_memcpy(reinterpret_cast<unsigned char*>(&aq) + 8, &t_b[dt & 1], 8);
                 mfma_dtile(dKt[dt], aq, dsfr);
@@ -565,4 +565,4 @@ int launch_bwd_dkdv_wave(hipStream_t st, const BwdParams& p, int batch, int max_
     return 0;
 }
 
-}  // namespace infllmv2
+}  // namespace IV2_NS

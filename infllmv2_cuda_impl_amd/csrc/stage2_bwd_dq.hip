@@ -18,7 +18,7 @@
 #include "stage2_bwd.h"
 #include <math.h>
 
-namespace infllmv2 {
+namespace IV2_NS {
 
 constexpr int kDqTokens = 8;
 constexpr int kDqChunk = 16;                                   // token groups per XCD chunk
@@ -60,14 +60,14 @@ __device__ __forceinline__ short4q dq_read_tr(const unsigned char* ptr) {
 // dS^T of one block as the B operand of dQ^T = K^T dS^T, from the S^T and dP^T accumulators
 // dS^T of one block as the B operand of dQ^T += K^T dS^T.  The dP accumulators were started at -D, so dp holds dP - D.
 // lim: last in-block key index the token may see (>= 63 for a whole block, which is the common case).
-__device__ __forceinline__ void ds_tile(const floatx4 (&s)[4], const floatx4 (&dp)[4], bf16x8 (&dsf)[2], int lim, int g,
+__device__ __forceinline__ void ds_tile(const floatx4 (&s)[4], const floatx4 (&dp)[4], elem8 (&dsf)[2], int lim, int g,
                                         float scale_log2, float lse2) {
     if (lim >= kBlockN - 1) {                                  // uniform per wavefront
 #pragma unroll
         for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
             for (int e = 0; e < 4; ++e)
-                dsf[kt >> 1][(kt & 1) * 4 + e] = static_cast<__bf16>(__builtin_amdgcn_exp2f(s[kt][e] * scale_log2 - lse2) * dp[kt][e]);
+                dsf[kt >> 1][(kt & 1) * 4 + e] = static_cast<elem_t>(__builtin_amdgcn_exp2f(s[kt][e] * scale_log2 - lse2) * dp[kt][e]);
     } else {
 #pragma unroll
         for (int kt = 0; kt < 4; ++kt)
@@ -75,7 +75,7 @@ __device__ __forceinline__ void ds_tile(const floatx4 (&s)[4], const floatx4 (&d
             for (int e = 0; e < 4; ++e) {
                 float pv = __builtin_amdgcn_exp2f(s[kt][e] * scale_log2 - lse2);
                 if (16 * kt + 4 * g + e > lim) pv = 0.f;
-                dsf[kt >> 1][(kt & 1) * 4 + e] = static_cast<__bf16>(pv * dp[kt][e]);
+                dsf[kt >> 1][(kt & 1) * 4 + e] = static_cast<elem_t>(pv * dp[kt][e]);
             }
     }
 }
@@ -144,14 +144,14 @@ void bwd_dq_hybrid_kernel(const BwdParams p, const DqExtra x) {
     for (int w = lane; w < nw; w += 64) own[w] &= ~com[w];
 
     // ---- this token's operands ----
-    bf16x8 qf[4], dof[4];
+    elem8 qf[4], dof[4];
     {
-        const bf16_bits* qp = p.q + tok * p.q_tok + h * p.q_kvh + n * p.q_grp + 8 * g;
-        const bf16_bits* dp = p.dout + tok * p.do_tok + h * p.do_kvh + n * p.do_grp + 8 * g;
+        const elem_bits* qp = p.q + tok * p.q_tok + h * p.q_kvh + n * p.q_grp + 8 * g;
+        const elem_bits* dp = p.dout + tok * p.do_tok + h * p.do_kvh + n * p.do_grp + 8 * g;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            qf[c] = *reinterpret_cast<const bf16x8*>(qp + 32 * c);
-            dof[c] = *reinterpret_cast<const bf16x8*>(dp + 32 * c);
+            qf[c] = *reinterpret_cast<const elem8*>(qp + 32 * c);
+            dof[c] = *reinterpret_cast<const elem8*>(dp + 32 * c);
         }
     }
     float lse2 = p.lse[h * p.lse_kvh + tok * p.lse_tok + n * p.lse_grp] * kLog2e;
@@ -197,12 +197,12 @@ void bwd_dq_hybrid_kernel(const BwdParams p, const DqExtra x) {
     const int64_t img0 = slot0 * kImageElems + lane * 8;
     uint4* mine = reinterpret_cast<uint4*>(smem_raw + 2 * kDqTileBytes + wave * 8192) + lane;     // 32 keys of K: 8 fragments
     const unsigned char* mine_tr = smem_raw + 2 * kDqTileBytes + wave * 8192 + tr_lane;
-    bf16x8 kreg[16], vreg[16];
+    elem8 kreg[16], vreg[16];
     int jp = live ? next_own() : -1;
     if (jp >= 0) {
-        const bf16_bits* ksrc = p.kimg + img0 + static_cast<int64_t>(jp) * kImageElems;
+        const elem_bits* ksrc = p.kimg + img0 + static_cast<int64_t>(jp) * kImageElems;
 #pragma unroll
-        for (int f = 0; f < 16; ++f) kreg[f] = *reinterpret_cast<const bf16x8*>(ksrc + f * 512);
+        for (int f = 0; f < 16; ++f) kreg[f] = *reinterpret_cast<const elem8*>(ksrc + f * 512);
     }
     // All ordinary loads so far land before the first LDS-DMA.  From here on the compiler's wait counts know nothing
     // of the DMA loads; they stay correct because loads complete in order, and the waits written by hand below
@@ -243,7 +243,7 @@ void bwd_dq_hybrid_kernel(const BwdParams p, const DqExtra x) {
                 for (int c = 0; c < 4; ++c)
 #pragma unroll
                     for (int kt = 0; kt < 4; ++kt)
-                        s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg[kt * 4 + c], qf[c], s[kt], 0, 0, 0);
+                        s[kt] = IV2_MFMA(vreg[kt * 4 + c], qf[c], s[kt], 0, 0, 0);
 #pragma unroll
                 for (int f = 0; f < 16; ++f) {
                     const uint4 raw = vb[f * 64];
@@ -253,8 +253,8 @@ void bwd_dq_hybrid_kernel(const BwdParams p, const DqExtra x) {
                 for (int c = 0; c < 4; ++c)
 #pragma unroll
                     for (int kt = 0; kt < 4; ++kt)
-                        dp[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg[kt * 4 + c], dof[c], dp[kt], 0, 0, 0);
-                bf16x8 dsf[2];
+                        dp[kt] = IV2_MFMA(vreg[kt * 4 + c], dof[c], dp[kt], 0, 0, 0);
+                elem8 dsf[2];
                 ds_tile(s, dp, dsf, (j0 == last_blk) ? last_key - j0 * kBlockN : kBlockN - 1, g, p.scale_log2, lse2);
                 const unsigned char* ktile = reinterpret_cast<const unsigned char*>(ring + tile * 2048) + tr_lane;
 #pragma unroll
@@ -264,10 +264,10 @@ void bwd_dq_hybrid_kernel(const BwdParams p, const DqExtra x) {
                         // K image unit (kt2, c, g', r') sits at ((kt2 * 4 + c) * 64 + g' * 16 + r') * 16 bytes
                         const unsigned char* at = ktile + ((2 * cc) * 4 + (dt >> 1)) * 1024 + (dt & 1) * 512;
                         const short4q lo = dq_read_tr(at), hi = dq_read_tr(at + 4096);
-                        bf16x8 kt_f;
+                        elem8 kt_f;
                         __builtin_memcpy(&kt_f, &lo, 8);
                         __builtin_memcpy(reinterpret_cast<unsigned char*>(&kt_f) + 8, &hi, 8);
-                        dq[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kt_f, dsf[cc], dq[dt], 0, 0, 0);
+                        dq[dt] = IV2_MFMA(kt_f, dsf[cc], dq[dt], 0, 0, 0);
                     }
             }
             j0 = j1;
@@ -276,9 +276,9 @@ void bwd_dq_hybrid_kernel(const BwdParams p, const DqExtra x) {
         k_ahead = false;
         if (jp >= 0) {                                         // per wavefront
             {
-                const bf16_bits* vsrc = p.vimg_r + img0 + static_cast<int64_t>(jp) * kImageElems;
+                const elem_bits* vsrc = p.vimg_r + img0 + static_cast<int64_t>(jp) * kImageElems;
 #pragma unroll
-                for (int f = 0; f < 16; ++f) vreg[f] = *reinterpret_cast<const bf16x8*>(vsrc + f * 512);
+                for (int f = 0; f < 16; ++f) vreg[f] = *reinterpret_cast<const elem8*>(vsrc + f * 512);
             }
             floatx4 s[4], dp[4];
 #pragma unroll
@@ -290,7 +290,7 @@ void bwd_dq_hybrid_kernel(const BwdParams p, const DqExtra x) {
             for (int c = 0; c < 4; ++c)
 #pragma unroll
                 for (int kt = 0; kt < 4; ++kt)
-                    s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[kt * 4 + c], qf[c], s[kt], 0, 0, 0);
+                    s[kt] = IV2_MFMA(kreg[kt * 4 + c], qf[c], s[kt], 0, 0, 0);
 #pragma unroll
             for (int f = 0; f < 8; ++f) {                      // keys 0..31 of K -> private tile
                 uint4 raw;
@@ -301,8 +301,8 @@ void bwd_dq_hybrid_kernel(const BwdParams p, const DqExtra x) {
             for (int c = 0; c < 4; ++c)
 #pragma unroll
                 for (int kt = 0; kt < 4; ++kt)
-                    dp[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg[kt * 4 + c], dof[c], dp[kt], 0, 0, 0);
-            bf16x8 dsf[2];
+                    dp[kt] = IV2_MFMA(vreg[kt * 4 + c], dof[c], dp[kt], 0, 0, 0);
+            elem8 dsf[2];
             ds_tile(s, dp, dsf, (jp == last_blk) ? last_key - jp * kBlockN : kBlockN - 1, g, p.scale_log2, lse2);
 #pragma unroll
             for (int cc = 0; cc < 2; ++cc) {
@@ -318,19 +318,19 @@ void bwd_dq_hybrid_kernel(const BwdParams p, const DqExtra x) {
                 for (int dt = 0; dt < 8; ++dt) {
                     const unsigned char* at = mine_tr + (dt >> 1) * 1024 + (dt & 1) * 512;
                     const short4q lo = dq_read_tr(at), hi = dq_read_tr(at + 4096);
-                    bf16x8 kt_f;
+                    elem8 kt_f;
                     __builtin_memcpy(&kt_f, &lo, 8);
                     __builtin_memcpy(reinterpret_cast<unsigned char*>(&kt_f) + 8, &hi, 8);
-                    dq[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kt_f, dsf[cc], dq[dt], 0, 0, 0);
+                    dq[dt] = IV2_MFMA(kt_f, dsf[cc], dq[dt], 0, 0, 0);
                 }
             }
             // the K fragments of the next own block go out last: they are the only ordinary loads in flight when the
             // next turn waits for its DMA
             const int jn = next_own();
             if (jn >= 0) {
-                const bf16_bits* ksrc = p.kimg + img0 + static_cast<int64_t>(jn) * kImageElems;
+                const elem_bits* ksrc = p.kimg + img0 + static_cast<int64_t>(jn) * kImageElems;
 #pragma unroll
-                for (int f = 0; f < 16; ++f) kreg[f] = *reinterpret_cast<const bf16x8*>(ksrc + f * 512);
+                for (int f = 0; f < 16; ++f) kreg[f] = *reinterpret_cast<const elem8*>(ksrc + f * 512);
                 k_ahead = true;
             }
             jp = jn;
@@ -338,12 +338,12 @@ void bwd_dq_hybrid_kernel(const BwdParams p, const DqExtra x) {
     }
     if (!live) return;
 
-    bf16_bits* op = p.dq + tok * p.dq_tok + h * p.dq_kvh + n * p.dq_grp + 4 * g;
+    elem_bits* op = p.dq + tok * p.dq_tok + h * p.dq_kvh + n * p.dq_grp + 4 * g;
 #pragma unroll
     for (int dt = 0; dt < 8; ++dt) {
         uint2 wv;
-        wv.x = pack_bf16x2(dq[dt][0] * p.scale, dq[dt][1] * p.scale);
-        wv.y = pack_bf16x2(dq[dt][2] * p.scale, dq[dt][3] * p.scale);
+        wv.x = pack_elem2(dq[dt][0] * p.scale, dq[dt][1] * p.scale);
+        wv.y = pack_elem2(dq[dt][2] * p.scale, dq[dt][3] * p.scale);
         *reinterpret_cast<uint2*>(op + 16 * dt) = wv;
     }
 }
@@ -369,4 +369,4 @@ int launch_bwd_dq_hybrid(hipStream_t st, const BwdParams& p, int batch, int max_
     return 0;
 }
 
-}  // namespace infllmv2
+}  // namespace IV2_NS

@@ -23,7 +23,7 @@
 #include "stage2_bwd.h"
 #include <math.h>
 
-namespace infllmv2 {
+namespace IV2_NS {
 
 constexpr int kHoTokens = 8;
 constexpr int kHoChunk = 16;                                   // token groups per XCD chunk
@@ -154,7 +154,7 @@ void bwd_dq_handoff_kernel(const BwdParams p, const HoExtra x) {
     auto issue_k = [&](int jj, int tile) { ho_dma_copy_2k(ring_src + static_cast<int64_t>(jj) * 1024, ring_dst + tile * 16384); };
     unsigned char* ds_tiles = smem_raw + kHoRingBytes + wave * 8192;               // [common | own][turn parity] x 2 KiB
     const uint32_t ds_lds = __builtin_amdgcn_readfirstlane(ho_lds_address(ds_tiles));
-    const bf16_bits* ds_row = p.ds_buf + (static_cast<int64_t>(h) * p.total_q + tok) * (p.max_sel + 1) * (kBlockN * 16) + lane * 8;
+    const elem_bits* ds_row = p.ds_buf + (static_cast<int64_t>(h) * p.total_q + tok) * (p.max_sel + 1) * (kBlockN * 16) + lane * 8;
     // rank of block j in this token's row; blocks past the announced bound were stored in the row's spare slot
     auto rank_of = [&](int j) -> int {
         const int w = j >> 6;
@@ -192,7 +192,7 @@ void bwd_dq_handoff_kernel(const BwdParams p, const HoExtra x) {
     // before their first use.  Nothing may touch dst between here and the wait at the top of the next turn.
     const unsigned char* kt_bytes = reinterpret_cast<const unsigned char*>(p.ktimg) + slot0 * (kImageElems * 2);
     const uint32_t lane16 = lane * 16;
-    auto load_k = [&](bf16x8 (&dst)[16], int j) {
+    auto load_k = [&](elem8 (&dst)[16], int j) {
         const unsigned char* blk = kt_bytes + static_cast<int64_t>(j) * (kImageElems * 2);         // uniform
 #pragma unroll
         for (int qd = 0; qd < 4; ++qd) {
@@ -207,7 +207,7 @@ void bwd_dq_handoff_kernel(const BwdParams p, const HoExtra x) {
         }
     };
     // B operands of the two 32-key chunks from a dS^T tile in LDS
-    auto read_ds = [&](const unsigned char* tile, bf16x8 (&dsf)[2]) {
+    auto read_ds = [&](const unsigned char* tile, elem8 (&dsf)[2]) {
 #pragma unroll
         for (int cc = 0; cc < 2; ++cc) {
             const short4h lo = ho_read_tr(tile + ds_lane + cc * 1024), hi = ho_read_tr(tile + ds_lane + cc * 1024 + 512);
@@ -218,7 +218,7 @@ void bwd_dq_handoff_kernel(const BwdParams p, const HoExtra x) {
 
     // ---- prologue: what the first two turns need, oldest request first ----
     // c0/c1/c2: the common blocks of this turn, the next and the one after; o0/o1/o2: the same for the own blocks
-    bf16x8 ka[16], kb[16];
+    elem8 ka[16], kb[16];
     int c0 = next_common();
     int c1 = c0 >= 0 ? next_common() : -1;
     int o0 = live ? next_own() : -1;
@@ -231,7 +231,7 @@ void bwd_dq_handoff_kernel(const BwdParams p, const HoExtra x) {
     if (o1 >= 0) issue_ds(o1, 1, 1);
     int tile = 0, par = 0;
     // one turn; the K fragments of the next own block are loaded into the buffer the last turn used
-    auto turn = [&](bf16x8 (&kcur)[16], bf16x8 (&knxt)[16]) {
+    auto turn = [&](elem8 (&kcur)[16], elem8 (&knxt)[16]) {
         // This turn's K (requested during the last turn) and dS tiles (requested the turn before) have landed when
         // only the dS tiles of the next turn, the youngest requests, are still in flight (loads complete in order).
         const int young = ((c1 >= 0 && live) ? 2 : 0) + (o1 >= 0 ? 2 : 0);
@@ -248,7 +248,7 @@ void bwd_dq_handoff_kernel(const BwdParams p, const HoExtra x) {
         if (c1 >= 0) issue_k(c1, tile ^ 1);
         if (o1 >= 0) load_k(knxt, o1);
         if (c0 >= 0 && live) {                                 // the common block
-            bf16x8 dsf[2];
+            elem8 dsf[2];
             read_ds(ds_tiles + par * 2048, dsf);
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the tile is in registers: its buffer takes the tile of
 #pragma unroll                                                  // the turn after next
@@ -260,13 +260,13 @@ void bwd_dq_handoff_kernel(const BwdParams p, const HoExtra x) {
 #pragma unroll
                 for (int cc = 0; cc < 2; ++cc) {
                     const uint4 raw = kt[(dt * 2 + cc) * 64];
-                    bf16x8 kf;
+                    elem8 kf;
                     __builtin_memcpy(&kf, &raw, 16);
-                    dq[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, dsf[cc], dq[dt], 0, 0, 0);
+                    dq[dt] = IV2_MFMA(kf, dsf[cc], dq[dt], 0, 0, 0);
                 }
         }
         if (o0 >= 0) {                                         // the own block
-            bf16x8 dsf[2];
+            elem8 dsf[2];
             read_ds(ds_tiles + (2 + par) * 2048, dsf);
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
@@ -276,7 +276,7 @@ void bwd_dq_handoff_kernel(const BwdParams p, const HoExtra x) {
             for (int dt = 0; dt < 8; ++dt)
 #pragma unroll
                 for (int cc = 0; cc < 2; ++cc)
-                    dq[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kcur[dt * 2 + cc], dsf[cc], dq[dt], 0, 0, 0);
+                    dq[dt] = IV2_MFMA(kcur[dt * 2 + cc], dsf[cc], dq[dt], 0, 0, 0);
         }
         if (c0 >= 0) tile ^= 1;
         par ^= 1;
@@ -290,12 +290,12 @@ void bwd_dq_handoff_kernel(const BwdParams p, const HoExtra x) {
     }
     if (!live) return;
 
-    bf16_bits* op = p.dq + tok * p.dq_tok + h * p.dq_kvh + n * p.dq_grp + 4 * g;
+    elem_bits* op = p.dq + tok * p.dq_tok + h * p.dq_kvh + n * p.dq_grp + 4 * g;
 #pragma unroll
     for (int dt = 0; dt < 8; ++dt) {
         uint2 wv;
-        wv.x = pack_bf16x2(dq[dt][0] * p.scale, dq[dt][1] * p.scale);
-        wv.y = pack_bf16x2(dq[dt][2] * p.scale, dq[dt][3] * p.scale);
+        wv.x = pack_elem2(dq[dt][0] * p.scale, dq[dt][1] * p.scale);
+        wv.y = pack_elem2(dq[dt][2] * p.scale, dq[dt][3] * p.scale);
         *reinterpret_cast<uint2*>(op + 16 * dt) = wv;
     }
 }
@@ -321,4 +321,4 @@ int launch_bwd_dq_handoff(hipStream_t st, const BwdParams& p, int batch, int max
     return 0;
 }
 
-}  // namespace infllmv2
+}  // namespace IV2_NS

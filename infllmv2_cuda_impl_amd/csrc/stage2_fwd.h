@@ -2,14 +2,14 @@
 #pragma once
 #include "common.h"
 
-namespace infllmv2 {
+namespace IV2_NS {
 
 struct FwdParams {
-    const bf16_bits* q;
-    bf16_bits* out;
+    const elem_bits* q;
+    elem_bits* out;
     float* lse;
-    const bf16_bits* kimg;
-    const bf16_bits* vimg;
+    const elem_bits* kimg;
+    const elem_bits* vimg;
     const int* cu_seqlens_q;
     const int* cu_seqlens_k;
     const uint64_t* mask;           // (Hk, total_q, n64) or null for dense
@@ -27,4 +27,4 @@ struct FwdParams {
 int launch_stage2_fwd_hybrid(hipStream_t st, const FwdParams& p, int batch, int num_heads_k, int max_seqlen_q,
                              int max_seqlen_k, bool causal);
 
-}  // namespace infllmv2
+}  // namespace IV2_NS

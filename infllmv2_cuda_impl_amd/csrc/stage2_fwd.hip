@@ -21,18 +21,18 @@
 #include <math.h>
 #include <stdlib.h>
 
-namespace infllmv2 {
+namespace IV2_NS {
 
 // ---------------------------------------------------------------------------------------------
 // K/V -> block images
 // ---------------------------------------------------------------------------------------------
 struct PackParams {
-    const bf16_bits* k;
-    const bf16_bits* v;
-    bf16_bits* kimg;                // K in K-image order (operand of a GEMM contracting over d)
-    bf16_bits* vimg;                // forward: V in V-image order (A operand of a GEMM contracting over keys), else null
-    bf16_bits* vimg_r;              // backward: V in K-image order (dP = dO V^T contracts over d), else null
-    bf16_bits* ktimg;               // backward with dS hand-off: K in V-image order (A operand of dQ^T = K^T dS^T), else null
+    const elem_bits* k;
+    const elem_bits* v;
+    elem_bits* kimg;                // K in K-image order (operand of a GEMM contracting over d)
+    elem_bits* vimg;                // forward: V in V-image order (A operand of a GEMM contracting over keys), else null
+    elem_bits* vimg_r;              // backward: V in K-image order (dP = dO V^T contracts over d), else null
+    elem_bits* ktimg;               // backward with dS hand-off: K in V-image order (A operand of dQ^T = K^T dS^T), else null
     const int* cu_seqlens_k;
     int64_t k_row_stride, k_head_stride;
     int64_t v_row_stride, v_head_stride;
@@ -43,15 +43,15 @@ constexpr int kVPad = 8;            // LDS row padding (elements) for the V tran
 
 __global__ __launch_bounds__(256)
 void pack_kv_kernel(const PackParams p) {
-    __shared__ __attribute__((aligned(16))) bf16_bits vt[kBlockN][kHeadDim + kVPad];
+    __shared__ __attribute__((aligned(16))) elem_bits vt[kBlockN][kHeadDim + kVPad];
     const int j = blockIdx.x, b = blockIdx.y, h = blockIdx.z;
     const int k0 = p.cu_seqlens_k[b];
     const int Sk = p.cu_seqlens_k[b + 1] - k0;
     if (static_cast<int64_t>(j) * kBlockN >= Sk) return;
     const int64_t slot = image_slot0(p.cu_seqlens_k, b) + j;
     const int tid = threadIdx.x;
-    const bf16_bits* kb = p.k + (k0 + static_cast<int64_t>(j) * kBlockN) * p.k_row_stride + h * p.k_head_stride;
-    const bf16_bits* vb = p.v + (k0 + static_cast<int64_t>(j) * kBlockN) * p.v_row_stride + h * p.v_head_stride;
+    const elem_bits* kb = p.k + (k0 + static_cast<int64_t>(j) * kBlockN) * p.k_row_stride + h * p.k_head_stride;
+    const elem_bits* vb = p.v + (k0 + static_cast<int64_t>(j) * kBlockN) * p.v_row_stride + h * p.v_head_stride;
     const int64_t img_off = (static_cast<int64_t>(h) * p.n_slots + slot) * kImageElems;
     const int valid = Sk - j * kBlockN;                       // keys of this block inside the sequence
     const uint4 zero = make_uint4(0, 0, 0, 0);
@@ -72,9 +72,9 @@ void pack_kv_kernel(const PackParams p) {
     // images that contract over the keys: V for the forward, K for the dQ kernel of the dS hand-off
 #pragma unroll 1
     for (int which = 0; which < 2; ++which) {
-        bf16_bits* dst = which == 0 ? p.vimg : p.ktimg;
+        elem_bits* dst = which == 0 ? p.vimg : p.ktimg;
         if (dst == nullptr) continue;                         // uniform per workgroup
-        const bf16_bits* src = which == 0 ? vb : kb;
+        const elem_bits* src = which == 0 ? vb : kb;
         const int64_t src_row = which == 0 ? p.v_row_stride : p.k_row_stride;
         __syncthreads();
         for (int u = tid; u < 1024; u += 256) {
@@ -117,10 +117,10 @@ void stage2_fwd_kernel(const FwdParams p) {
     const int64_t tok = static_cast<int64_t>(q0) + i;
     const int n = lane & 15, g = lane >> 4;
 
-    const bf16_bits* qp = p.q + tok * p.q_tok_stride + h * p.q_kvh_stride + n * p.q_grp_stride + 8 * g;
-    bf16x8 qf[4];
+    const elem_bits* qp = p.q + tok * p.q_tok_stride + h * p.q_kvh_stride + n * p.q_grp_stride + 8 * g;
+    elem8 qf[4];
 #pragma unroll
-    for (int c = 0; c < 4; ++c) qf[c] = *reinterpret_cast<const bf16x8*>(qp + 32 * c);
+    for (int c = 0; c < 4; ++c) qf[c] = *reinterpret_cast<const elem8*>(qp + 32 * c);
 
     int last_key = kCausal ? (i + Sk - Sq) : (Sk - 1);          // largest allowed key index
     if (last_key > Sk - 1) last_key = Sk - 1;
@@ -130,26 +130,26 @@ void stage2_fwd_kernel(const FwdParams p) {
     walk.init(p.mask ? p.mask + (static_cast<int64_t>(h) * p.total_q + tok) * p.n64 : nullptr, p.n64, last_blk);
 
     const int64_t img0 = (static_cast<int64_t>(h) * p.n_slots + image_slot0(p.cu_seqlens_k, b)) * kImageElems;
-    const bf16_bits* kimg = p.kimg + img0 + lane * 8;
-    const bf16_bits* vimg = p.vimg + img0 + lane * 8;
+    const elem_bits* kimg = p.kimg + img0 + lane * 8;
+    const elem_bits* vimg = p.vimg + img0 + lane * 8;
 
     float m = -INFINITY, l = 0.f;
     floatx4 o[8];
 #pragma unroll
     for (int dt = 0; dt < 8; ++dt) o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    bf16x8 kreg[16], vreg[16];
+    elem8 kreg[16], vreg[16];
     int j = walk.next();
     if (j >= 0) {
-        const bf16_bits* src = kimg + static_cast<int64_t>(j) * kImageElems;
+        const elem_bits* src = kimg + static_cast<int64_t>(j) * kImageElems;
 #pragma unroll
-        for (int f = 0; f < 16; ++f) kreg[f] = *reinterpret_cast<const bf16x8*>(src + f * 512);
+        for (int f = 0; f < 16; ++f) kreg[f] = *reinterpret_cast<const elem8*>(src + f * 512);
     }
     while (j >= 0) {
         {
-            const bf16_bits* src = vimg + static_cast<int64_t>(j) * kImageElems;
+            const elem_bits* src = vimg + static_cast<int64_t>(j) * kImageElems;
 #pragma unroll
-            for (int f = 0; f < 16; ++f) vreg[f] = *reinterpret_cast<const bf16x8*>(src + f * 512);
+            for (int f = 0; f < 16; ++f) vreg[f] = *reinterpret_cast<const elem8*>(src + f * 512);
         }
         floatx4 s[4];
 #pragma unroll
@@ -157,13 +157,13 @@ void stage2_fwd_kernel(const FwdParams p) {
             s[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int c = 0; c < 4; ++c)
-                s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[kt * 4 + c], qf[c], s[kt], 0, 0, 0);
+                s[kt] = IV2_MFMA(kreg[kt * 4 + c], qf[c], s[kt], 0, 0, 0);
         }
         const int jn = walk.next();
         if (jn >= 0) {
-            const bf16_bits* src = kimg + static_cast<int64_t>(jn) * kImageElems;
+            const elem_bits* src = kimg + static_cast<int64_t>(jn) * kImageElems;
 #pragma unroll
-            for (int f = 0; f < 16; ++f) kreg[f] = *reinterpret_cast<const bf16x8*>(src + f * 512);
+            for (int f = 0; f < 16; ++f) kreg[f] = *reinterpret_cast<const elem8*>(src + f * 512);
         }
         if (j == last_blk) {                                    // only the last allowed block needs element masking
             const int lim = last_key - j * kBlockN;              // keys with in-block index > lim are masked
@@ -195,30 +195,30 @@ void stage2_fwd_kernel(const FwdParams p) {
         m = m_new;
 #pragma unroll
         for (int dt = 0; dt < 8; ++dt) o[dt] *= alpha;
-        bf16x8 pf[2];
+        elem8 pf[2];
 #pragma unroll
         for (int cc = 0; cc < 2; ++cc)
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                pf[cc][e] = static_cast<__bf16>(s[2 * cc][e]);
-                pf[cc][4 + e] = static_cast<__bf16>(s[2 * cc + 1][e]);
+                pf[cc][e] = static_cast<elem_t>(s[2 * cc][e]);
+                pf[cc][4 + e] = static_cast<elem_t>(s[2 * cc + 1][e]);
             }
 #pragma unroll
         for (int dt = 0; dt < 8; ++dt)
 #pragma unroll
             for (int cc = 0; cc < 2; ++cc)
-                o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg[dt * 2 + cc], pf[cc], o[dt], 0, 0, 0);
+                o[dt] = IV2_MFMA(vreg[dt * 2 + cc], pf[cc], o[dt], 0, 0, 0);
         j = jn;
     }
 
     const float l_tot = wave_sum_over_g(l);
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-    bf16_bits* op = p.out + tok * p.o_tok_stride + h * p.o_kvh_stride + n * p.o_grp_stride + 4 * g;
+    elem_bits* op = p.out + tok * p.o_tok_stride + h * p.o_kvh_stride + n * p.o_grp_stride + 4 * g;
 #pragma unroll
     for (int dt = 0; dt < 8; ++dt) {
         uint2 w;
-        w.x = pack_bf16x2(o[dt][0] * inv, o[dt][1] * inv);
-        w.y = pack_bf16x2(o[dt][2] * inv, o[dt][3] * inv);
+        w.x = pack_elem2(o[dt][0] * inv, o[dt][1] * inv);
+        w.y = pack_elem2(o[dt][2] * inv, o[dt][3] * inv);
         *reinterpret_cast<uint2*>(op + 16 * dt) = w;
     }
     if (g == 0) {
@@ -227,15 +227,17 @@ void stage2_fwd_kernel(const FwdParams p) {
     }
 }
 
-}  // namespace infllmv2
+}  // namespace IV2_NS
 
-using namespace infllmv2;
+using namespace IV2_NS;
 
+#ifndef IV2_F16        // both element types are 2 bytes wide: defined once
 extern "C" size_t infllmv2_kv_image_bytes(int64_t total_k, int batch, int num_heads_k) {
-    return static_cast<size_t>(image_slots(total_k, batch)) * num_heads_k * kImageElems * sizeof(bf16_bits) * 2;
+    return static_cast<size_t>(image_slots(total_k, batch)) * num_heads_k * kImageElems * sizeof(elem_bits) * 2;
 }
+#endif
 
-namespace infllmv2 {
+namespace IV2_NS {
 int launch_pack(hipStream_t st, const void* k, const void* v, const int32_t* cu_seqlens_k, void* workspace,
                 size_t workspace_bytes, int batch, int64_t total_k, int num_heads_k, int max_seqlen_k,
                 const int64_t* k_strides, const int64_t* v_strides, bool backward_images, void* kt_image) {
@@ -251,12 +253,12 @@ int launch_pack(hipStream_t st, const void* k, const void* v, const int32_t* cu_
     const int max_blocks = (max_seqlen_k + kBlockN - 1) / kBlockN;
     if (max_blocks == 0 || total_k == 0) return 0;
     PackParams pp{};
-    pp.k = static_cast<const bf16_bits*>(k);
-    pp.v = static_cast<const bf16_bits*>(v);
-    pp.kimg = static_cast<bf16_bits*>(workspace);
-    bf16_bits* second = pp.kimg + n_slots * num_heads_k * kImageElems;
+    pp.k = static_cast<const elem_bits*>(k);
+    pp.v = static_cast<const elem_bits*>(v);
+    pp.kimg = static_cast<elem_bits*>(workspace);
+    elem_bits* second = pp.kimg + n_slots * num_heads_k * kImageElems;
     if (backward_images) pp.vimg_r = second; else pp.vimg = second;
-    pp.ktimg = static_cast<bf16_bits*>(kt_image);
+    pp.ktimg = static_cast<elem_bits*>(kt_image);
     pp.cu_seqlens_k = cu_seqlens_k;
     pp.k_row_stride = k_strides[0]; pp.k_head_stride = k_strides[1];
     pp.v_row_stride = v_strides[0]; pp.v_head_stride = v_strides[1];
@@ -265,8 +267,9 @@ int launch_pack(hipStream_t st, const void* k, const void* v, const int32_t* cu_
     IV2_LAUNCH_CHECK();
     return 0;
 }
-}  // namespace infllmv2
+}  // namespace IV2_NS
 
+#ifndef IV2_F16        // the images are a permutation of 2-byte elements: one entry point serves both element types
 extern "C" int infllmv2_pack_kv(void* stream, const void* k, const void* v, const int32_t* cu_seqlens_k,
                                 void* workspace, size_t workspace_bytes, int batch, int64_t total_k,
                                 int num_heads_k, int head_dim, int max_seqlen_k, const int64_t* k_strides,
@@ -275,8 +278,9 @@ extern "C" int infllmv2_pack_kv(void* stream, const void* k, const void* v, cons
     return launch_pack(static_cast<hipStream_t>(stream), k, v, cu_seqlens_k, workspace, workspace_bytes, batch,
                        total_k, num_heads_k, max_seqlen_k, k_strides, v_strides, false);
 }
+#endif
 
-extern "C" int infllmv2_varlen_fwd(void* stream, const void* q, const void* k, const void* v, void* out,
+extern "C" int IV2_ENTRY(infllmv2_varlen_fwd)(void* stream, const void* q, const void* k, const void* v, void* out,
                                    float* softmax_lse, const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
                                    const uint64_t* blockmask, void* workspace, size_t workspace_bytes,
                                    int kv_prepacked, int batch, int64_t total_q, int64_t total_k, int num_heads,
@@ -307,10 +311,10 @@ extern "C" int infllmv2_varlen_fwd(void* stream, const void* q, const void* k, c
     }
     const int64_t n_slots = image_slots(total_k, batch);
     FwdParams fp{};
-    fp.q = static_cast<const bf16_bits*>(q);
-    fp.out = static_cast<bf16_bits*>(out);
+    fp.q = static_cast<const elem_bits*>(q);
+    fp.out = static_cast<elem_bits*>(out);
     fp.lse = softmax_lse;
-    fp.kimg = static_cast<const bf16_bits*>(workspace);
+    fp.kimg = static_cast<const elem_bits*>(workspace);
     fp.vimg = fp.kimg + n_slots * num_heads_k * kImageElems;
     fp.cu_seqlens_q = cu_seqlens_q; fp.cu_seqlens_k = cu_seqlens_k;
     fp.mask = blockmask;

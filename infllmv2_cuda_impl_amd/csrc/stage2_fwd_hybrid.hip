@@ -28,7 +28,7 @@
 #include "stage2_fwd.h"
 #include <math.h>
 
-namespace infllmv2 {
+namespace IV2_NS {
 
 constexpr int kHybTokens = 8;                                  // tokens (= wavefronts) per workgroup
 constexpr int kHybChunk = 16;                                  // token groups per XCD chunk
@@ -65,7 +65,7 @@ __device__ __forceinline__ uint64_t uniform_u64(uint64_t v) {
 }
 
 // online-softmax update with one 16 x 64 score tile (s: S^T accumulators); returns P as the B operand of P.V
-__device__ __forceinline__ void softmax_step(floatx4 (&s)[4], float& m, float& l, floatx4 (&o)[8], bf16x8 (&pf)[2],
+__device__ __forceinline__ void softmax_step(floatx4 (&s)[4], float& m, float& l, floatx4 (&o)[8], elem8 (&pf)[2],
                                              int lim, int g, float scale_log2) {
     if (lim < kBlockN - 1) {
 #pragma unroll
@@ -102,8 +102,8 @@ __device__ __forceinline__ void softmax_step(floatx4 (&s)[4], float& m, float& l
     for (int cc = 0; cc < 2; ++cc)
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            pf[cc][e] = static_cast<__bf16>(s[2 * cc][e]);
-            pf[cc][4 + e] = static_cast<__bf16>(s[2 * cc + 1][e]);
+            pf[cc][e] = static_cast<elem_t>(s[2 * cc][e]);
+            pf[cc][4 + e] = static_cast<elem_t>(s[2 * cc + 1][e]);
         }
 }
 
@@ -172,11 +172,11 @@ void stage2_fwd_hybrid_kernel(const FwdParams p, const HybridExtra x) {
     for (int w = lane; w < nw; w += 64) own[w] &= ~com[w];
 
     // ---- Q operand ----
-    bf16x8 qf[4];
+    elem8 qf[4];
     {
-        const bf16_bits* qp = p.q + tok * p.q_tok_stride + h * p.q_kvh_stride + n * p.q_grp_stride + 8 * g;
+        const elem_bits* qp = p.q + tok * p.q_tok_stride + h * p.q_kvh_stride + n * p.q_grp_stride + 8 * g;
 #pragma unroll
-        for (int c = 0; c < 4; ++c) qf[c] = *reinterpret_cast<const bf16x8*>(qp + 32 * c);
+        for (int c = 0; c < 4; ++c) qf[c] = *reinterpret_cast<const elem8*>(qp + 32 * c);
     }
     float m = -INFINITY, l = 0.f;
     floatx4 o[8];
@@ -212,14 +212,14 @@ void stage2_fwd_hybrid_kernel(const FwdParams p, const HybridExtra x) {
         obits &= obits - 1ull;
         return ow * 64 + bit;
     };
-    const bf16_bits* kimg = p.kimg + slot0 * kImageElems + lane * 8;
-    const bf16_bits* vimg = p.vimg + slot0 * kImageElems + lane * 8;
-    bf16x8 kreg[16], vreg[16];
+    const elem_bits* kimg = p.kimg + slot0 * kImageElems + lane * 8;
+    const elem_bits* vimg = p.vimg + slot0 * kImageElems + lane * 8;
+    elem8 kreg[16], vreg[16];
     int jp = live ? next_own() : -1;                           // own block of this turn; its K fragments are loaded a turn ahead
     if (jp >= 0) {
-        const bf16_bits* src = kimg + static_cast<int64_t>(jp) * kImageElems;
+        const elem_bits* src = kimg + static_cast<int64_t>(jp) * kImageElems;
 #pragma unroll
-        for (int f = 0; f < 16; ++f) kreg[f] = *reinterpret_cast<const bf16x8*>(src + f * 512);
+        for (int f = 0; f < 16; ++f) kreg[f] = *reinterpret_cast<const elem8*>(src + f * 512);
     }
     // All ordinary loads so far (Q, mask words, first K fragments) land before the first LDS-DMA.  From here on the
     // compiler's wait counts know nothing of the DMA loads; they stay correct because loads complete in order (an
@@ -255,25 +255,25 @@ void stage2_fwd_hybrid_kernel(const FwdParams p, const HybridExtra x) {
         for (int c = 0; c < 4; ++c)
 #pragma unroll
             for (int kt = 0; kt < 4; ++kt)
-                s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg[kt * 4 + c], qf[c], s[kt], 0, 0, 0);
+                s[kt] = IV2_MFMA(vreg[kt * 4 + c], qf[c], s[kt], 0, 0, 0);
 #pragma unroll
         for (int f = 0; f < 16; ++f) {
             const uint4 raw = vb[f * 64];
             __builtin_memcpy(&vreg[f], &raw, 16);
         }
-        bf16x8 pf[2];
+        elem8 pf[2];
         softmax_step(s, m, l, o, pf, (j0 == last_blk) ? last_key - j0 * kBlockN : kBlockN, g, p.scale_log2);
 #pragma unroll
         for (int cc = 0; cc < 2; ++cc)
 #pragma unroll
             for (int dt = 0; dt < 8; ++dt)
-                o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg[dt * 2 + cc], pf[cc], o[dt], 0, 0, 0);
+                o[dt] = IV2_MFMA(vreg[dt * 2 + cc], pf[cc], o[dt], 0, 0, 0);
     };
     auto own_part = [&]() {
         {
-            const bf16_bits* src = vimg + static_cast<int64_t>(jp) * kImageElems;
+            const elem_bits* src = vimg + static_cast<int64_t>(jp) * kImageElems;
 #pragma unroll
-            for (int f = 0; f < 16; ++f) vreg[f] = *reinterpret_cast<const bf16x8*>(src + f * 512);
+            for (int f = 0; f < 16; ++f) vreg[f] = *reinterpret_cast<const elem8*>(src + f * 512);
         }
         floatx4 s[4];
 #pragma unroll
@@ -282,20 +282,20 @@ void stage2_fwd_hybrid_kernel(const FwdParams p, const HybridExtra x) {
         for (int c = 0; c < 4; ++c)
 #pragma unroll
             for (int kt = 0; kt < 4; ++kt)
-                s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[kt * 4 + c], qf[c], s[kt], 0, 0, 0);
-        bf16x8 pf[2];
+                s[kt] = IV2_MFMA(kreg[kt * 4 + c], qf[c], s[kt], 0, 0, 0);
+        elem8 pf[2];
         softmax_step(s, m, l, o, pf, (jp == last_blk) ? last_key - jp * kBlockN : kBlockN, g, p.scale_log2);
 #pragma unroll
         for (int cc = 0; cc < 2; ++cc)
 #pragma unroll
             for (int dt = 0; dt < 8; ++dt)
-                o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg[dt * 2 + cc], pf[cc], o[dt], 0, 0, 0);
+                o[dt] = IV2_MFMA(vreg[dt * 2 + cc], pf[cc], o[dt], 0, 0, 0);
         const int jn = next_own();
         k_ahead = false;
         if (jn >= 0) {                                         // K fragments of the next own block
-            const bf16_bits* src = kimg + static_cast<int64_t>(jn) * kImageElems;
+            const elem_bits* src = kimg + static_cast<int64_t>(jn) * kImageElems;
 #pragma unroll
-            for (int f = 0; f < 16; ++f) kreg[f] = *reinterpret_cast<const bf16x8*>(src + f * 512);
+            for (int f = 0; f < 16; ++f) kreg[f] = *reinterpret_cast<const elem8*>(src + f * 512);
             k_ahead = true;
         }
         jp = jn;
@@ -327,12 +327,12 @@ void stage2_fwd_hybrid_kernel(const FwdParams p, const HybridExtra x) {
     // ---- epilogue ----
     const float l_tot = wave_sum_over_g(l);
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-    bf16_bits* op = p.out + tok * p.o_tok_stride + h * p.o_kvh_stride + n * p.o_grp_stride + 4 * g;
+    elem_bits* op = p.out + tok * p.o_tok_stride + h * p.o_kvh_stride + n * p.o_grp_stride + 4 * g;
 #pragma unroll
     for (int dt = 0; dt < 8; ++dt) {
         uint2 wv;
-        wv.x = pack_bf16x2(o[dt][0] * inv, o[dt][1] * inv);
-        wv.y = pack_bf16x2(o[dt][2] * inv, o[dt][3] * inv);
+        wv.x = pack_elem2(o[dt][0] * inv, o[dt][1] * inv);
+        wv.y = pack_elem2(o[dt][2] * inv, o[dt][3] * inv);
         *reinterpret_cast<uint2*>(op + 16 * dt) = wv;
     }
     if (g == 0) {
@@ -363,4 +363,4 @@ int launch_stage2_fwd_hybrid(hipStream_t st, const FwdParams& p, int batch, int 
     return 0;
 }
 
-}  // namespace infllmv2
+}  // namespace IV2_NS

@@ -37,8 +37,6 @@ def decode_with_kvcache(q, k_cache, v_cache, k_new, v_new, cache_seqlens, softma
         raise RuntimeError("query and key must have the same dtype")
     if v_cache.dtype != q.dtype:
         raise RuntimeError("query and value must have the same dtype")
-    if q.dtype != torch.bfloat16:
-        raise RuntimeError("this build only has bf16 kernels")
     if q.dim() != 4 or k_cache.dim() != 4 or v_cache.dim() != 4:
         raise RuntimeError("q, k_cache, v_cache must have 4 dimensions")
     batch, seqlen_q, Hq, d = q.shape
@@ -134,7 +132,7 @@ def decode_with_kvcache(q, k_cache, v_cache, k_new, v_new, cache_seqlens, softma
     workspace = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=q.device)
     two = lambda t: _lib.i64_array([t.stride(0), t.stride(2)])
     with torch.cuda.device(q.device):
-        _lib.call("infllmv2_fwd_kvcache", stream_ptr(q.device), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+        _lib.call_for(q.dtype, "infllmv2_fwd_kvcache", stream_ptr(q.device), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                   ptr(k_new), ptr(v_new), ptr(cache_seqlens), out.data_ptr(), lse.data_ptr(), ptr(mask),
                   workspace.data_ptr(), workspace.numel(), batch, seqlen_q, Hq, Hk, d, cap, seqlen_new, two(q),
                   _s3(k_cache), _s3(v_cache), _s3(k_new) if k_new is not None else _lib.i64_array([0, 0, 0]),

@@ -93,7 +93,7 @@ class InfLLMv2Attention(torch.nn.Module):
         columns, with every other block dropped.  ``rows``: packed query tokens; ``positions`` int32 (batch): tokens before each
         sequence's first query.  Returns ``(topk_idx, block_mask)`` with ``init_blocks + local_blocks + 1`` index slots."""
         batch = cu_seqlens_q.numel() - 1
-        empty = torch.empty((nheads_k, rows, 0), dtype=torch.bfloat16, device=device)
+        empty = torch.empty((nheads_k, rows, 0), dtype=torch.bfloat16, device=device)  # pooled scores: any 16-bit type
         no_keys = torch.zeros(batch + 1, dtype=torch.int32, device=device)
         pooled = max_pooling_1d_varlen(empty, cu_seqlens_q, no_keys, positions, max_seqlen_q, 0, self.local_blocks,
                                        self.init_blocks, block_size=self.block_size, stride=self.stride,

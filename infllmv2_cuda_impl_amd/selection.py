@@ -55,8 +55,8 @@ def compress_keys(k: torch.Tensor, cu_seqlens_k: torch.Tensor, max_seqlen_k: int
     buffer returned by an earlier call) and ``first_row`` only rows ``>= first_row`` of each sequence are written.
     """
     require_gpu(k, "k")
-    if k.dtype != torch.bfloat16:
-        raise RuntimeError("this build only has bf16 kernels")
+    if k.dtype not in (torch.float16, torch.bfloat16):
+        raise RuntimeError("FlashAttention only support fp16 and bf16 data type")
     if k.dim() != 3 or k.stride(-1) != 1:
         raise RuntimeError("k must have shape (total_k, num_heads_k, head_size) with a contiguous last dimension")
     if cu_seqlens_k.dtype != torch.int32 or not cu_seqlens_k.is_contiguous():
@@ -76,7 +76,7 @@ def compress_keys(k: torch.Tensor, cu_seqlens_k: torch.Tensor, max_seqlen_k: int
         backing = out
     cu_out = torch.empty(batch + 1, dtype=torch.int32, device=k.device)
     with torch.cuda.device(k.device):
-        _lib.call("infllmv2_compress_keys", stream_ptr(k.device), k.data_ptr(), backing.data_ptr(), cu_seqlens_k.data_ptr(),
+        _lib.call_for(k.dtype, "infllmv2_compress_keys", stream_ptr(k.device), k.data_ptr(), backing.data_ptr(), cu_seqlens_k.data_ptr(),
                   cu_out.data_ptr(), batch, max_seqlen_k, Hk, d, k.stride(0), k.stride(1), kernel_size, stride, first_row)
     return out, cu_out
 
@@ -90,8 +90,8 @@ def compress_keys_cache(k_cache: torch.Tensor, new_lens: torch.Tensor, kernel_si
     are written in place.  ``max_new_rows`` bounds the new rows per sequence (default: every row of ``out``; 1 suffices
     for a one-token step).  Returns ``out_lens`` int32 ``(batch,)``: the rows each compressed cache now holds."""
     require_gpu(k_cache, "k_cache")
-    if k_cache.dtype != torch.bfloat16 or out.dtype != torch.bfloat16:
-        raise RuntimeError("this build only has bf16 kernels")
+    if k_cache.dtype not in (torch.float16, torch.bfloat16) or out.dtype != k_cache.dtype:
+        raise RuntimeError("FlashAttention only support fp16 and bf16 data type")
     if k_cache.dim() != 4 or out.dim() != 4 or k_cache.stride(-1) != 1 or out.stride(-1) != 1 or \
             out.shape[0] != k_cache.shape[0] or tuple(out.shape[2:]) != tuple(k_cache.shape[2:]):
         raise RuntimeError("k_cache and out must have shapes (batch, capacity, num_heads_k, head_size) and "
@@ -108,7 +108,7 @@ def compress_keys_cache(k_cache: torch.Tensor, new_lens: torch.Tensor, kernel_si
         out_lens = torch.empty(batch, dtype=torch.int32, device=k_cache.device)
     s3 = lambda t: _lib.i64_array([t.stride(0), t.stride(1), t.stride(2)])
     with torch.cuda.device(k_cache.device):
-        _lib.call("infllmv2_compress_keys_cache", stream_ptr(k_cache.device), k_cache.data_ptr(), out.data_ptr(),
+        _lib.call_for(k_cache.dtype, "infllmv2_compress_keys_cache", stream_ptr(k_cache.device), k_cache.data_ptr(), out.data_ptr(),
                   None if old_lens is None else old_lens.data_ptr(), new_lens.data_ptr(), out_lens.data_ptr(), batch,
                   int(max_new_rows), Hk, d, s3(k_cache), s3(out), kernel_size, stride)
     return out_lens

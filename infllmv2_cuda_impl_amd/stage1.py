@@ -42,7 +42,7 @@ def stage1_scores(q, k, v, cu_seqlens_q, cu_seqlens_k, cu_seqlens_v, max_seqlen_
         raise RuntimeError("v must have shape (total_v, num_heads_k, head_size)")
     k, v = _readable(k), _readable(v)
     row = (max_seqlen_k + row_pad_to - 1) // row_pad_to * row_pad_to
-    buf = torch.empty((Hk, total_q, row), dtype=torch.bfloat16, device=q.device)
+    buf = torch.empty((Hk, total_q, row), dtype=q.dtype, device=q.device)
     if max_seqlen_q == 1 and total_q > 0:
         # decode: one query per sequence, so the parallelism has to come from the keys
         stage1_decode(q, k, v, cu_seqlens_q=cu_seqlens_q, cu_seqlens_k=cu_seqlens_k, cu_seqlens_v=cu_seqlens_v,
@@ -51,7 +51,7 @@ def stage1_scores(q, k, v, cu_seqlens_q, cu_seqlens_k, cu_seqlens_v, max_seqlen_
                       out_row_stride=buf.stride(1))
         return buf if row == max_seqlen_k else buf[:, :, :max_seqlen_k]
     with torch.cuda.device(q.device):
-        _lib.call("infllmv2_varlen_fwd_stage1", stream_ptr(q.device), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+        _lib.call_for(q.dtype, "infllmv2_varlen_fwd_stage1", stream_ptr(q.device), q.data_ptr(), k.data_ptr(), v.data_ptr(),
                   buf.data_ptr(), cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), cu_seqlens_v.data_ptr(), batch,
                   total_q, Hq, Hk, d, max_seqlen_q, max_seqlen_k,
                   _lib.i64_array([q.stride(0), q.stride(1), GROUP * q.stride(1)]),
@@ -78,7 +78,7 @@ def stage1_pooled(q, k, v, cu_seqlens_q, cu_seqlens_k, cu_seqlens_v, max_seqlen_
         raise RuntimeError("v must have shape (total_v, num_heads_k, head_size)")
     k, v = _readable(k), _readable(v)
     per_block = block_size // stride
-    out = torch.empty((Hk, total_q, out_len), dtype=torch.bfloat16, device=q.device)
+    out = torch.empty((Hk, total_q, out_len), dtype=q.dtype, device=q.device)
     if max_seqlen_q == 1 and total_q > 0 and out_len > 0:
         return stage1_decode(q, k, v, cu_seqlens_q=cu_seqlens_q, cu_seqlens_k=cu_seqlens_k, cu_seqlens_v=cu_seqlens_v,
                              max_seqlen_k=max_seqlen_k, max_seqlen_v=_max_rows_bound(v, batch, max_seqlen_k),
@@ -87,7 +87,7 @@ def stage1_pooled(q, k, v, cu_seqlens_q, cu_seqlens_k, cu_seqlens_v, max_seqlen_
                              out_len=out_len, local_blocks=local_blocks, init_blocks=init_blocks,
                              block_size=block_size, stride=stride)
     with torch.cuda.device(q.device):
-        _lib.call("infllmv2_varlen_fwd_stage1_pooled", stream_ptr(q.device), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+        _lib.call_for(q.dtype, "infllmv2_varlen_fwd_stage1_pooled", stream_ptr(q.device), q.data_ptr(), k.data_ptr(), v.data_ptr(),
                   out.data_ptr(), cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), cu_seqlens_v.data_ptr(),
                   cache_lens.data_ptr() if cache_lens is not None else None, int(cache_len), batch, total_q, Hq, Hk, d,
                   max_seqlen_q, max_seqlen_k,
@@ -118,7 +118,7 @@ def stage1_decode(q, k, v, *, cu_seqlens_q=None, cu_seqlens_k=None, k_lens=None,
     per_block = block_size // stride
     p = lambda t: None if t is None else t.data_ptr()
     with torch.cuda.device(q.device):
-        _lib.call("infllmv2_stage1_decode", stream_ptr(q.device), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+        _lib.call_for(q.dtype, "infllmv2_stage1_decode", stream_ptr(q.device), q.data_ptr(), k.data_ptr(), v.data_ptr(),
                   out.data_ptr(), p(cu_seqlens_q), p(cu_seqlens_k), p(k_lens), p(cu_seqlens_v), p(v_lens),
                   workspace.data_ptr(), workspace.numel(), batch, Hq, Hk, d, max_seqlen_k, max_seqlen_v,
                   _lib.i64_array([q.stride(0), q.stride(-2), GROUP * q.stride(-2)]),

@@ -57,6 +57,11 @@ def bf16_round(x: np.ndarray) -> np.ndarray:
     return r.astype(np.uint32).view(np.float32).reshape(x.shape)
 
 
+def f16_round(x: np.ndarray) -> np.ndarray:
+    """Round fp32 to the nearest-even IEEE half and return it as fp32 (numpy's own conversion)."""
+    return np.asarray(x, dtype=np.float32).astype(np.float16).astype(np.float32)
+
+
 def _trunc_div(a: int, b: int) -> int:
     """C++ integer division (rounds toward zero), as the kernels compute it."""
     q = abs(a) // abs(b)
@@ -70,10 +75,11 @@ def compressed_len(seqlen: int, kernel: int, stride: int) -> int:
     return 0 if seqlen < kernel else (seqlen - kernel) // stride + 1
 
 
-def compress_keys(k: np.ndarray, cu_seqlens, kernel: int, stride: int):
+def compress_keys(k: np.ndarray, cu_seqlens, kernel: int, stride: int, rounding=bf16_round):
     """Mean over full windows [stride*j, stride*j + kernel) of every packed sequence.
 
-    k: (total, H, d) fp32.  Returns (k_cmp (sum L, H, d) fp32 rounded to bf16, cu_cmp int32).
+    k: (total, H, d) fp32.  Returns (k_cmp (sum L, H, d) fp32 rounded to the element type (``rounding``: bf16_round or
+    f16_round), cu_cmp int32).
     """
     cu = [int(c) for c in cu_seqlens]
     outs, cu_c = [], [0]
@@ -83,7 +89,7 @@ def compress_keys(k: np.ndarray, cu_seqlens, kernel: int, stride: int):
         if L:
             idx = (np.arange(L)[:, None] * stride + np.arange(kernel)[None, :]).reshape(-1)
             win = seq[idx].reshape(L, kernel, *seq.shape[1:]).astype(np.float32)
-            outs.append(bf16_round(win.mean(axis=1, dtype=np.float32)))
+            outs.append(rounding(win.mean(axis=1, dtype=np.float32)))
         cu_c.append(cu_c[-1] + L)
     if outs:
         kc = np.concatenate(outs, axis=0)
@@ -108,7 +114,7 @@ def stage1_visible(i: int, stride: int, L: int, seqlen_q: int, causal: bool) -> 
 
 def stage1_scores(q, k_cmp, k_coarse, cu_seqlens_q, cu_seqlens_k, cu_seqlens_v,
                   max_seqlen_k: int, softmax_scale: float, causal: bool,
-                  round_output: bool = True) -> np.ndarray:
+                  round_output: bool = True, rounding=bf16_round) -> np.ndarray:
     """Stage-1 group scores (flash_fwd_kernel.h:1203-1744, softmax.h:94-121,198-237).
 
     q (T, Hq, d); k_cmp (sum Lk, Hk, d) fine compressed keys; k_coarse (sum Lc, Hk, d) the key
@@ -154,7 +160,7 @@ def stage1_scores(q, k_cmp, k_coarse, cu_seqlens_q, cu_seqlens_k, cu_seqlens_v,
             p = np.where((vis_c > 0)[:, None], p, 0.0)
             p = np.where(np.isnan(p), 0.0, p)                           # infllmv2_sparse_attention.py:589
             out[h, cu_q[b]:cu_q[b + 1], :Lk] = p.astype(np.float32)
-    return bf16_round(out) if round_output else out
+    return rounding(out) if round_output else out
 
 
 # ----------------------------------------------------------------------------------------
@@ -480,11 +486,12 @@ def decode_forward(q, k_cache, v_cache, cache_seqlens, fwd_mask_words, softmax_s
     return out, lse
 
 
-def rotary_apply(x: np.ndarray, cos: np.ndarray, sin: np.ndarray, pos: int, interleaved: bool) -> np.ndarray:
+def rotary_apply(x: np.ndarray, cos: np.ndarray, sin: np.ndarray, pos: int, interleaved: bool,
+                 rounding=bf16_round) -> np.ndarray:
     """Rotary embedding of the rows of ``x`` (..., d) at position ``pos`` (csrc/flash_attn/src/rotary.h:19-82
     interleaved, :84-150 contiguous): only the first ``rotary_dim = 2 * cos.shape[1]`` columns turn.
     interleaved: pairs (2i, 2i+1); contiguous: pairs (i, i + rotary_dim/2);
-    (a, b) -> (a cos_i - b sin_i, a sin_i + b cos_i), fp32 arithmetic, result rounded to bf16."""
+    (a, b) -> (a cos_i - b sin_i, a sin_i + b cos_i), fp32 arithmetic, result rounded to the element type."""
     x = np.asarray(x, dtype=np.float32).copy()
     half = cos.shape[1]
     c = np.asarray(cos[pos], dtype=np.float32)
@@ -497,12 +504,12 @@ def rotary_apply(x: np.ndarray, cos: np.ndarray, sin: np.ndarray, pos: int, inte
         a, b = x[..., :half].copy(), x[..., half:2 * half].copy()
         x[..., :half] = a * c - b * s_
         x[..., half:2 * half] = a * s_ + b * c
-    return bf16_round(x)
+    return rounding(x)
 
 
 def decode_forward_ext(q, k_cache, v_cache, cache_seqlens, fwd_mask_words, softmax_scale: float, k_new=None,
                        v_new=None, cache_batch_idx=None, cache_leftpad=None, block_table=None, rotary_cos=None,
-                       rotary_sin=None, rotary_interleaved=True, dtype=np.float64):
+                       rotary_sin=None, rotary_interleaved=True, dtype=np.float64, rounding=bf16_round):
     """mha_fwd_kvcache with its remaining options (flash_api.cpp:1549-1843, flash_fwd_kernel.h:606-1199):
     * cache_batch_idx (b): sequence b lives in cache row cache_batch_idx[b];
     * cache_leftpad (b): the sequence's keys are cache rows [leftpad, cache_seqlens) (block_info.h:23-25, 41-43);
@@ -537,8 +544,8 @@ def decode_forward_ext(q, k_cache, v_cache, cache_seqlens, fwd_mask_words, softm
             ci, ri = rows(b, end, end + n)
             kn = np.asarray(k_new[b], dtype=np.float32)
             if rotary_cos is not None:
-                kn = np.stack([rotary_apply(kn[t], rotary_cos, rotary_sin, end + t, rotary_interleaved) for t in range(n)])
-                qb = rotary_apply(qb, rotary_cos, rotary_sin, end, rotary_interleaved)
+                kn = np.stack([rotary_apply(kn[t], rotary_cos, rotary_sin, end + t, rotary_interleaved, rounding) for t in range(n)])
+                qb = rotary_apply(qb, rotary_cos, rotary_sin, end, rotary_interleaved, rounding)
             k_cache[ci, ri] = kn
             v_cache[ci, ri] = v_new[b]
             end += n
