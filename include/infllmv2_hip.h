@@ -220,9 +220,10 @@ size_t infllmv2_kv_image_bytes(int64_t total_k, int batch, int num_heads_k);
 
 /* csrc/entry.cu:14,210 `varlen_fwd` = mha_varlen_fwd (csrc/flash_attn/flash_api.cpp:519-782) on
  * the sparse path (blockmask given) and on the dense path (blockmask null).
- * bf16, head_dim 128, num_heads == 16 * num_heads_k.
+ * bf16, head_dim 128, num_heads == g * num_heads_k with g = 16 (the reference build) or 1, 2, 4, 8; the same holds
+ * for every entry point that takes num_heads and num_heads_k.
  * q/out: element strides {token, head-in-group, kv-head}; the caller's (T, Hq, d) tensor is
- *   {Hq*d, d, 16*d}; the reference's re-laid-out (T*16, Hk, d) tensor is {16*Hk*d, Hk*d, d}.
+ *   {Hq*d, d, g*d}; the reference's re-laid-out (T*16, Hk, d) tensor is {16*Hk*d, Hk*d, d}.
  * k/v: (total_k, Hk, d), strides {row, head}.  softmax_lse strides {token, head-in-group, kv-head};
  *   the reference's (Hk, T*16) layout (flash_api.cpp:665) is {16, 1, T*16}.
  * blockmask (Hk, total_q, n_uint64_per_row): block indices local to each sequence, rows by packed

@@ -15,7 +15,17 @@ from . import _lib
 from ._util import ptr, require_gpu, stream_ptr
 from .masks import topk_to_uint64, transpose_blockmask
 
-GROUP = 16          # query heads per KV head the kernels are built for (flash_api.cpp:941)
+GROUP = 16          # query heads per KV head the reference build is hard-wired to (flash_api.cpp:941)
+GROUPS = (1, 2, 4, 8, 16)     # group sizes served: smaller ones run on the same 16-row tiles
+
+
+def group_size(num_heads: int, num_heads_k: int) -> int:
+    """Query heads per KV head, checked against what the kernels serve."""
+    if num_heads_k <= 0 or num_heads % num_heads_k != 0:
+        raise RuntimeError("Number of heads in key/value must divide number of heads in query")
+    if num_heads // num_heads_k not in GROUPS:
+        raise RuntimeError("this build requires 1, 2, 4, 8 or 16 query heads per key/value head")
+    return num_heads // num_heads_k
 BLOCK_N = 64        # key-block size of the sparse mask (infllmv2_sparse_attention.py:93)
 
 
@@ -101,14 +111,13 @@ def _check_qkv(q, k, v, cu_seqlens_q, cu_seqlens_k, same_kv_len=True):
         raise RuntimeError("cu_seqlens_k must have shape (batch_size + 1)")
     if head_size != 128:
         raise RuntimeError("this build only supports head dimension 128")
-    if q.shape[1] != GROUP * k.shape[1]:
-        raise RuntimeError("this build requires 16 query heads per key/value head")
+    group_size(q.shape[1], k.shape[1])
     return batch
 
 
-def _natural_strides(t: torch.Tensor):
+def _natural_strides(t: torch.Tensor, group: int = GROUP):
     """{token, head-in-group, kv-head} element strides of a (T, Hq, d) tensor."""
-    return _lib.i64_array([t.stride(0), t.stride(1), GROUP * t.stride(1)])
+    return _lib.i64_array([t.stride(0), t.stride(1), group * t.stride(1)])
 
 
 def _sparse_forward(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, softmax_scale, causal,
@@ -118,12 +127,13 @@ def _sparse_forward(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqle
     total_q, Hq, d = q.shape
     total_k, Hk = k.shape[0], k.shape[1]
     out = torch.empty_like(q)
+    grp = Hq // Hk
     if lse_expanded:
-        lse = torch.empty((Hk, total_q * GROUP), dtype=torch.float32, device=q.device)       # flash_api.cpp:665
-        lse_strides = _lib.i64_array([GROUP, 1, total_q * GROUP])
+        lse = torch.empty((Hk, total_q * grp), dtype=torch.float32, device=q.device)         # flash_api.cpp:665
+        lse_strides = _lib.i64_array([grp, 1, total_q * grp])
     else:
         lse = torch.empty((Hq, total_q), dtype=torch.float32, device=q.device)
-        lse_strides = _lib.i64_array([1, total_q, GROUP * total_q])
+        lse_strides = _lib.i64_array([1, total_q, grp * total_q])
     ws_bytes = _lib.lib.infllmv2_kv_image_bytes(total_k, batch, Hk)
     workspace = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=q.device)
     n64 = 0 if fwd_mask is None else fwd_mask.shape[-1]
@@ -131,8 +141,8 @@ def _sparse_forward(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqle
         _lib.call_for(q.dtype, "infllmv2_varlen_fwd", stream_ptr(q.device), q.data_ptr(), k.data_ptr(), v.data_ptr(),
                   out.data_ptr(), lse.data_ptr(), cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), ptr(fwd_mask),
                   workspace.data_ptr(), workspace.numel(), 0, batch, total_q, total_k, Hq, Hk, d, max_seqlen_q,
-                  max_seqlen_k, _natural_strides(q), _lib.i64_array([k.stride(0), k.stride(1)]),
-                  _lib.i64_array([v.stride(0), v.stride(1)]), _natural_strides(out), lse_strides, n64,
+                  max_seqlen_k, _natural_strides(q, grp), _lib.i64_array([k.stride(0), k.stride(1)]),
+                  _lib.i64_array([v.stride(0), v.stride(1)]), _natural_strides(out, grp), lse_strides, n64,
                   float(softmax_scale), int(bool(causal)))
     return out, lse
 
@@ -199,14 +209,15 @@ def infllmv2_attn_varlen_func(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q,
                               topk_idx=None, block_mask=None):
     """Block-sparse (or, with ``topk_idx=None``, dense) attention over packed variable-length sequences.
 
-    q ``(total_q, nheads, 128)``, k/v ``(total_k, nheads_k, 128)`` bf16 with ``nheads == 16*nheads_k``;
+    q ``(total_q, nheads, 128)``, k/v ``(total_k, nheads_k, 128)`` bf16 or fp16 with ``nheads == g*nheads_k``, g in 1, 2, 4, 8, 16
+    (16 is what the reference build serves and what the kernels' tiles are laid out for);
     ``cu_seqlens_q/k`` int32 ``(batch+1,)``.  ``topk_idx`` int32 ``(nheads_k, total_q, k)`` lists, per KV head
     and packed query token, the 64-key blocks (indices local to the token's sequence, ``-1`` = unused) the
-    token attends to; all 16 query heads of a group share the row.  ``causal=True`` aligns the causal mask to
+    token attends to; all query heads of a group share the row.  ``causal=True`` aligns the causal mask to
     the bottom-right corner; a query with no visible key yields zeros.  Differentiable w.r.t. q, k, v.
 
     Returns ``out (total_q, nheads, 128)``; with ``return_attn_probs`` the tuple ``(out, softmax_lse, S_dmask)``
-    where ``softmax_lse`` is fp32 ``(nheads_k, total_q*16)`` with column ``t*16 + g`` on the sparse path
+    where ``softmax_lse`` is fp32 ``(nheads_k, total_q*g)`` with column ``t*g + head-in-group`` on the sparse path
     (``(nheads, total_q)`` on the dense path) and ``S_dmask`` is empty.  dropout, softcap, ALiBi, sliding
     windows and paged KV are rejected exactly as the reference build rejects them.
     ``block_mask`` (not in the reference's signature) is the packed form of the same selection, int64
@@ -226,7 +237,7 @@ def infllmv2_attn_stage1(q, k, v, cu_seqlens_q, cu_seqlens_k, cu_seqlens_v, max_
     q ``(total_q, nheads, 128)``; k ``(sum Lk, nheads_k, 128)`` the stride-16 compressed keys; v
     ``(sum Lc, nheads_k, 128)`` the key set the log-sum-exp is taken over (the stride-64 compressed keys, or
     ``k`` itself for an exact softmax); ``cu_seqlens_{q,k,v}`` int32.  Returns bf16
-    ``(nheads_k, total_q, max_seqlen_k)``: for every token and KV head the sum over the 16 grouped heads of
+    ``(nheads_k, total_q, max_seqlen_k)``: for every token and KV head the sum over the grouped heads of
     ``exp(scale*q.k_j - lse)`` on the keys the token may see, 0 elsewhere.
     """
     from .stage1 import stage1_scores
@@ -310,8 +321,9 @@ def infllmv2_attn_stage1_kvcache(q, k_fine_cache, k_coarse_cache, fine_lens, coa
             k_coarse_cache.shape[0] != batch:
         raise RuntimeError("compressed-key caches must have shape (batch_size, rows, num_heads_k, head_size)")
     Hk = k_fine_cache.shape[2]
-    if d != 128 or Hq != GROUP * Hk or tuple(k_coarse_cache.shape[2:]) != (Hk, d) or k_fine_cache.shape[3] != d:
-        raise RuntimeError("this build requires head dimension 128 and 16 query heads per key/value head")
+    group_size(Hq, Hk)
+    if d != 128 or tuple(k_coarse_cache.shape[2:]) != (Hk, d) or k_fine_cache.shape[3] != d:
+        raise RuntimeError("this build requires head dimension 128")
     for name, t in (("fine_lens", fine_lens), ("coarse_lens", coarse_lens), ("cache_seqlens", cache_seqlens)):
         if t.dtype != torch.int32 or tuple(t.shape) != (batch,) or not t.is_contiguous():
             raise RuntimeError(f"{name} must be a contiguous int32 tensor of shape (batch_size)")

@@ -31,8 +31,8 @@ def _handoff_limit() -> int:
     return int(os.environ.get("INFLLMV2_BWD_HANDOFF_MAX_BYTES", HANDOFF_MAX_BYTES))
 
 
-def _nat(t):
-    return _lib.i64_array([t.stride(0), t.stride(1), GROUP * t.stride(1)])
+def _nat(t, group=GROUP):
+    return _lib.i64_array([t.stride(0), t.stride(1), group * t.stride(1)])
 
 
 def sparse_backward(dout, q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, softmax_scale,
@@ -50,10 +50,11 @@ def sparse_backward(dout, q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, max_seq
     total_q, Hq, d = q.shape
     total_k, Hk = k.shape[0], k.shape[1]
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    grp = Hq // Hk
     if lse_expanded:
-        lse_strides = _lib.i64_array([GROUP, 1, total_q * GROUP])
+        lse_strides = _lib.i64_array([grp, 1, total_q * grp])
     else:
-        lse_strides = _lib.i64_array([1, total_q, GROUP * total_q])
+        lse_strides = _lib.i64_array([1, total_q, grp * total_q])
     n64 = 0 if fwd_mask is None else fwd_mask.shape[-1]
     if fwd_mask is None or Hk * total_q * (max_selected + 1) * 2048 > _handoff_limit():
         max_selected = 0
@@ -74,6 +75,6 @@ def sparse_backward(dout, q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, max_seq
                   v.data_ptr(), out.data_ptr(), lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
                   cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), ptr(fwd_mask), workspace.data_ptr(),
                   workspace.numel(), batch, total_q, total_k, Hq, Hk, d, max_seqlen_q, max_seqlen_k,
-                  _nat(q), kv(k), kv(v), _nat(out), _nat(dout), _nat(dq), kv(dk), kv(dv), lse_strides, n64,
+                  _nat(q, grp), kv(k), kv(v), _nat(out, grp), _nat(dout, grp), _nat(dq, grp), kv(dk), kv(dv), lse_strides, n64,
                   float(softmax_scale), int(bool(causal)), int(bool(deterministic)), int(max_selected))
     return dq, dk, dv

@@ -30,7 +30,7 @@ namespace IV2_NS {
 
 constexpr int kWave = 64;          // CDNA wavefront width
 constexpr int kHeadDim = 128;      // only head size the reference build instantiates (static_switch.h:79-89)
-constexpr int kGroup = 16;         // query heads per KV head (flash_api.cpp:941)
+constexpr int kGroup = 16;         // query heads per KV head the MFMA tiles are laid out for (flash_api.cpp:941)
 constexpr int kBlockN = 64;        // key-block size of the sparse mask (flash_api.cpp:706-710)
 
 #ifdef IV2_F16
@@ -42,6 +42,14 @@ typedef __attribute__((__vector_size__(8 * sizeof(elem_t)))) elem_t elem8;     /
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 typedef uint16_t bf16_bits;
 typedef uint16_t elem_bits;                                  // an element as it lies in memory
+
+// Group sizes served: the reference build is hard-wired to 16 heads per KV head; smaller powers of two run on the same
+// 16-row tiles with the spare rows repeating the last head (their results are never stored and never accumulated).
+inline bool valid_group(int num_heads, int num_heads_k) {
+    if (num_heads_k <= 0 || num_heads <= 0 || num_heads % num_heads_k != 0) return false;
+    const int grp = num_heads / num_heads_k;
+    return grp == 1 || grp == 2 || grp == 4 || grp == 8 || grp == 16;
+}
 
 #define IV2_CHECK(cond, ...)                         \
     do {                                             \

@@ -40,6 +40,7 @@ struct DecodeParams {
     int64_t kc_batch, kc_row, kc_head, vc_batch, vc_row, vc_head;
     int64_t kn_batch, kn_row, kn_head, vn_batch, vn_row, vn_head;
     int batch, num_heads_k, capacity, seqlen_new, n64, splits;
+    int group;                      // query heads per KV head, 1..16
     float scale_log2;
     // where a sequence's rows lie (flash_api.cpp:1593-1611, 1762-1771, 1800-1808)
     const int* cache_batch_idx;     // sequence b uses cache row cache_batch_idx[b]; null: b
@@ -130,7 +131,7 @@ void decode_append_kernel(const DecodeParams p) {
 __global__ __launch_bounds__(256)
 void decode_rotate_q_kernel(const DecodeParams p) {
     const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-    const int heads = p.num_heads_k * 16;
+    const int heads = p.num_heads_k * p.group;
     if (idx >= static_cast<int64_t>(p.batch) * heads * 16) return;
     const int chunk = static_cast<int>(idx & 15);
     const int head = static_cast<int>((idx >> 4) % heads), b = static_cast<int>((idx >> 4) / heads);
@@ -175,9 +176,10 @@ void decode_split_kernel(const DecodeParams p) {
 
     elem8 qf[4];
     {
+        const int qh = p.group * h + (n < p.group ? n : p.group - 1);      // rows beyond the group repeat its last head
         const elem_bits* qp = p.rotary_dim > 0
-            ? p.q_rot + (static_cast<int64_t>(b) * p.num_heads_k * 16 + 16 * h + n) * kHeadDim + 8 * g
-            : p.q + b * p.q_batch + (16 * h + n) * p.q_head + 8 * g;
+            ? p.q_rot + (static_cast<int64_t>(b) * p.num_heads_k * p.group + qh) * kHeadDim + 8 * g
+            : p.q + b * p.q_batch + qh * p.q_head + 8 * g;
 #pragma unroll
         for (int c = 0; c < 4; ++c) qf[c] = *reinterpret_cast<const elem8*>(qp + 32 * c);
     }
@@ -293,7 +295,8 @@ void decode_split_kernel(const DecodeParams p) {
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
     const float lse = l_tot > 0.f ? m * 0.69314718055994530942f + logf(l_tot) : (kDirect ? INFINITY : -INFINITY);
     if (kDirect) {
-        elem_bits* op = p.out + b * p.o_batch + (16 * h + n) * p.o_head + 4 * g;
+        if (n >= p.group) return;
+        elem_bits* op = p.out + b * p.o_batch + (p.group * h + n) * p.o_head + 4 * g;
 #pragma unroll
         for (int dt = 0; dt < 8; ++dt) {
             uint2 w;
@@ -301,7 +304,7 @@ void decode_split_kernel(const DecodeParams p) {
             w.y = pack_elem2(o[dt][2] * inv, o[dt][3] * inv);
             *reinterpret_cast<uint2*>(op + 16 * dt) = w;
         }
-        if (g == 0) p.lse[static_cast<int64_t>(b) * p.num_heads_k * 16 + 16 * h + n] = lse;
+        if (g == 0) p.lse[static_cast<int64_t>(b) * p.num_heads_k * p.group + p.group * h + n] = lse;
     } else {
         const int64_t slot = (static_cast<int64_t>(b) * p.num_heads_k + h) * p.splits + split;
         float* op = p.o_part + (slot * 16 + n) * kHeadDim + 4 * g;
@@ -318,6 +321,7 @@ void decode_combine_kernel(const DecodeParams p) {
     const int h = blockIdx.x, b = blockIdx.y;
     const int tid = threadIdx.x;
     const int head = tid >> 4, d0 = (tid & 15) * 8;
+    if (head >= p.group) return;                               // partial rows that only filled the MFMA tile
     const int64_t slot0 = (static_cast<int64_t>(b) * p.num_heads_k + h) * p.splits;
     float mx = -INFINITY;
     for (int s = 0; s < p.splits; ++s) mx = fmaxf(mx, p.lse_part[(slot0 + s) * 16 + head]);
@@ -342,9 +346,9 @@ void decode_combine_kernel(const DecodeParams p) {
     outv.y = pack_elem2(acc[2] * inv, acc[3] * inv);
     outv.z = pack_elem2(acc[4] * inv, acc[5] * inv);
     outv.w = pack_elem2(acc[6] * inv, acc[7] * inv);
-    *reinterpret_cast<uint4*>(p.out + b * p.o_batch + (16 * h + head) * p.o_head + d0) = outv;
+    *reinterpret_cast<uint4*>(p.out + b * p.o_batch + (p.group * h + head) * p.o_head + d0) = outv;
     if ((tid & 15) == 0)
-        p.lse[static_cast<int64_t>(b) * p.num_heads_k * 16 + 16 * h + head] = wsum > 0.f ? mx + logf(wsum) : INFINITY;
+        p.lse[static_cast<int64_t>(b) * p.num_heads_k * p.group + p.group * h + head] = wsum > 0.f ? mx + logf(wsum) : INFINITY;
 }
 
 }  // namespace IV2_NS
@@ -389,8 +393,8 @@ static int fwd_kvcache_impl(void* stream, const void* q, void* kcache, void* vca
                                     const void* rotary_sin, int rotary_dim, int rotary_interleaved) {
     IV2_CHECK(head_dim == kHeadDim, "fwd_kvcache: this build only supports head_dim 128 (got %d)", head_dim);
     IV2_CHECK(seqlen_q == 1, "fwd_kvcache: this build only supports one query token per sequence (got %d)", seqlen_q);
-    IV2_CHECK(num_heads_k > 0 && num_heads == num_heads_k * kGroup,
-              "fwd_kvcache: requires num_heads == 16 * num_heads_k (got %d and %d)", num_heads, num_heads_k);
+    IV2_CHECK(valid_group(num_heads, num_heads_k),
+              "fwd_kvcache: requires num_heads == g * num_heads_k with g in {1, 2, 4, 8, 16} (got %d and %d)", num_heads, num_heads_k);
     IV2_CHECK(batch > 0 && cache_capacity > 0, "fwd_kvcache: batch size and cache capacity must be positive");
     IV2_CHECK(batch <= 65535 && num_heads_k <= 65535, "fwd_kvcache: batch and num_heads_k must not exceed 65535");
     IV2_CHECK(q && kcache && vcache && out && softmax_lse, "fwd_kvcache: null pointer");
@@ -436,6 +440,7 @@ static int fwd_kvcache_impl(void* stream, const void* q, void* kcache, void* vca
     p.kc_batch = kcache_strides[0]; p.kc_row = kcache_strides[1]; p.kc_head = kcache_strides[2];
     p.vc_batch = vcache_strides[0]; p.vc_row = vcache_strides[1]; p.vc_head = vcache_strides[2];
     p.batch = batch; p.num_heads_k = num_heads_k; p.capacity = cache_capacity;
+    p.group = num_heads / num_heads_k;
     p.seqlen_new = k_new ? seqlen_new : 0;
     p.n64 = n_uint64_per_row; p.splits = num_splits;
     p.scale_log2 = softmax_scale * 1.44269504088896340736f;

@@ -39,6 +39,7 @@ struct Stage1Params {
     int score_cols;                  // columns to define in every row (max_seqlen_k)
     float scale_log2;
     int causal;
+    int group;                       // query heads per KV head, 1..16: MFMA rows >= group repeat head group - 1 and add nothing
     // pooled output only
     const int* cache_lens;           // per sequence, or null: cache_len for all
     int cache_len;
@@ -155,7 +156,7 @@ void stage1_kernel(const Stage1Params p) {
 #pragma unroll
     for (int t = 0; t < kTokPerWave; ++t) {
         const int i = live[t] ? tok0 + t : Sq - 1;
-        const elem_bits* qp = p.q + (static_cast<int64_t>(q0) + i) * p.q_tok_stride + h * p.q_kvh_stride + n * p.q_grp_stride + 8 * g;
+        const elem_bits* qp = p.q + (static_cast<int64_t>(q0) + i) * p.q_tok_stride + h * p.q_kvh_stride + (n < p.group ? n : p.group - 1) * p.q_grp_stride + 8 * g;
 #pragma unroll
         for (int c = 0; c < 4; ++c) qf[t][c] = *reinterpret_cast<const elem8*>(qp + 32 * c);
     }
@@ -242,6 +243,7 @@ void stage1_kernel(const Stage1Params p) {
                 mm = mn;
             }
             lse2[t][e] = mm + __builtin_amdgcn_logf(ll);        // v_log_f32 is log2
+            if (4 * g + e >= p.group) lse2[t][e] = INFINITY;    // a row that only fills the tile: exp2(x - inf) = 0 in the head sum
         }
 
     // ---------------- pass 2: scores over the fine keys ----------------
@@ -352,8 +354,8 @@ int launch_stage1(const char* who, void* stream, const void* q, const void* k, c
                   int64_t out_head_stride, int64_t out_row_stride, float softmax_scale, int is_causal,
                   const Stage1Pool* pool) {
     IV2_CHECK(head_dim == kHeadDim, "%s: this build only supports head_dim 128 (got %d)", who, head_dim);
-    IV2_CHECK(num_heads_k > 0 && num_heads == num_heads_k * kGroup,
-              "%s: requires num_heads == 16 * num_heads_k (got %d and %d)", who, num_heads, num_heads_k);
+    IV2_CHECK(valid_group(num_heads, num_heads_k),
+              "%s: requires num_heads == g * num_heads_k with g in {1, 2, 4, 8, 16} (got %d and %d)", who, num_heads, num_heads_k);
     IV2_CHECK(batch > 0 && total_q >= 0 && max_seqlen_q >= 0 && max_seqlen_k >= 0, "%s: bad sizes", who);
     IV2_CHECK(q && k && v && out && cu_seqlens_q && cu_seqlens_k && cu_seqlens_v, "%s: null pointer", who);
     IV2_CHECK(num_heads_k <= 65535 && batch <= 65535, "%s: batch and num_heads_k must not exceed 65535", who);
@@ -379,6 +381,7 @@ int launch_stage1(const char* who, void* stream, const void* q, const void* k, c
     p.c_row_stride = v_strides[0]; p.c_head_stride = v_strides[1];
     p.score_head_stride = out_head_stride; p.score_row_stride = out_row_stride;
     p.score_cols = max_seqlen_k;
+    p.group = num_heads / num_heads_k;
     p.scale_log2 = softmax_scale * 1.44269504088896340736f;
     p.causal = is_causal;
     if (pool) {

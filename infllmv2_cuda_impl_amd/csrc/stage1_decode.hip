@@ -45,6 +45,7 @@ struct S1DecodeParams {
     int cols;                        // score columns to define per row (max_seqlen_k)
     float scale_log2;
     int causal;
+    int group;                       // query heads per KV head, 1..16: MFMA rows >= group repeat head group - 1 and add nothing
     int splits_c, splits_f;
     // pooled output
     const int* cache_lens;           // per sequence, or null: cache_len for all
@@ -95,7 +96,7 @@ __device__ __forceinline__ void s1d_load_tile(elem8 (&t)[16], const elem_bits* b
 }
 
 __device__ __forceinline__ void s1d_load_q(elem8 (&qf)[4], const S1DecodeParams& p, const S1DecodeSeq& s, int h, int n, int g) {
-    const elem_bits* qp = p.q + static_cast<int64_t>(s.q_row) * p.q_tok_stride + h * p.q_kvh_stride + n * p.q_grp_stride + 8 * g;
+    const elem_bits* qp = p.q + static_cast<int64_t>(s.q_row) * p.q_tok_stride + h * p.q_kvh_stride + (n < p.group ? n : p.group - 1) * p.q_grp_stride + 8 * g;
 #pragma unroll
     for (int c = 0; c < 4; ++c) qf[c] = *reinterpret_cast<const elem8*>(qp + 32 * c);
 }
@@ -239,6 +240,7 @@ void stage1_decode_score_kernel(const S1DecodeParams p) {
                 mm = mn;
             }
             lse2[e] = mm + __builtin_amdgcn_logf(ll);            // v_log_f32 is log2
+            if (4 * g + e >= p.group) lse2[e] = INFINITY;        // a row that only fills the tile adds exp2(x - inf) = 0
         }
     }
     const int64_t out_row = static_cast<int64_t>(h) * p.out_head_stride + static_cast<int64_t>(sq.q_row) * p.out_row_stride;
@@ -357,8 +359,8 @@ extern "C" int IV2_ENTRY(infllmv2_stage1_decode)(void* stream, const void* q, co
                                       int padding, int block_size, int local_blocks, int init_blocks) {
     const char* who = "stage1_decode";
     IV2_CHECK(head_dim == kHeadDim, "%s: this build only supports head_dim 128 (got %d)", who, head_dim);
-    IV2_CHECK(num_heads_k > 0 && num_heads == num_heads_k * kGroup,
-              "%s: requires num_heads == 16 * num_heads_k (got %d and %d)", who, num_heads, num_heads_k);
+    IV2_CHECK(valid_group(num_heads, num_heads_k),
+              "%s: requires num_heads == g * num_heads_k with g in {1, 2, 4, 8, 16} (got %d and %d)", who, num_heads, num_heads_k);
     IV2_CHECK(batch > 0 && max_seqlen_k >= 0 && max_seqlen_v >= 0, "%s: bad sizes", who);
     IV2_CHECK(num_heads_k <= 65535 && batch <= 65535, "%s: batch and num_heads_k must not exceed 65535", who);
     IV2_CHECK(q && k && v && out, "%s: null pointer", who);
@@ -396,6 +398,7 @@ extern "C" int IV2_ENTRY(infllmv2_stage1_decode)(void* stream, const void* q, co
     p.c_batch_stride = v_strides[0]; p.c_row_stride = v_strides[1]; p.c_head_stride = v_strides[2];
     p.out_head_stride = out_head_stride; p.out_row_stride = out_row_stride;
     p.cols = max_seqlen_k;
+    p.group = num_heads / num_heads_k;
     p.scale_log2 = softmax_scale * 1.44269504088896340736f;
     p.causal = is_causal;
     p.cache_lens = cache_lens; p.cache_len = cache_len; p.pool_len = out_len;

@@ -32,6 +32,7 @@ struct BwdParams {
     int64_t dk_row, dk_head, dv_row, dv_head;
     int64_t n_slots, total_q, total_k;
     int n64_fwd, n64_bwd, k_blocks, num_heads_k;
+    int group;                      // query heads per KV head, 1..16: rows >= group repeat head group - 1 with LSE = +inf (P = dS = 0)
     float scale_log2, scale;
     // deterministic dK/dV: every (block, 512-token slice) work item stores its two tiles in a slot of its own and a
     // second kernel adds the slots of a block in slice order (no atomics); null: fp32 atomics into dk_acc / dv_acc

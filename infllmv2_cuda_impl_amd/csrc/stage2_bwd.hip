@@ -37,8 +37,10 @@ void bwd_prep_kernel(const BwdParams p) {
     const int h = blockIdx.y;
     const int tid = threadIdx.x;
     const int row = tid >> 4, part = tid & 15;
-    const uint4 dv = *reinterpret_cast<const uint4*>(p.dout + tok * p.do_tok + h * p.do_kvh + row * p.do_grp + part * 8);
-    const uint4 ov = *reinterpret_cast<const uint4*>(p.out + tok * p.o_tok + h * p.o_kvh + row * p.o_grp + part * 8);
+    const bool spare = row >= p.group;                         // a row that only fills the 16-row tiles of the other kernels
+    const int rowc = spare ? p.group - 1 : row;
+    const uint4 dv = *reinterpret_cast<const uint4*>(p.dout + tok * p.do_tok + h * p.do_kvh + rowc * p.do_grp + part * 8);
+    const uint4 ov = *reinterpret_cast<const uint4*>(p.out + tok * p.o_tok + h * p.o_kvh + rowc * p.o_grp + part * 8);
     const uint32_t dw[4] = {dv.x, dv.y, dv.z, dv.w};
     const uint32_t ow[4] = {ov.x, ov.y, ov.z, ov.w};
     float acc = 0.f;
@@ -50,10 +52,11 @@ void bwd_prep_kernel(const BwdParams p) {
 #pragma unroll
     for (int off = 1; off < 16; off <<= 1) acc += __shfl_xor(acc, off);
     if (part == 0) {
-        p.dsum[static_cast<int64_t>(h) * p.total_q * 16 + tok * 16 + row] = acc;
+        // spare rows get LSE = +inf and D = 0: their P = exp2(x - inf) and dS = P (dP - D) vanish in every kernel
+        p.dsum[static_cast<int64_t>(h) * p.total_q * 16 + tok * 16 + row] = spare ? 0.f : acc;
         float* rs = p.rowstat + (static_cast<int64_t>(h) * p.total_q + tok) * 32;
-        rs[row] = p.lse[h * p.lse_kvh + tok * p.lse_tok + row * p.lse_grp] * kLog2e;
-        rs[16 + row] = acc;
+        rs[row] = spare ? INFINITY : p.lse[h * p.lse_kvh + tok * p.lse_tok + row * p.lse_grp] * kLog2e;
+        rs[16 + row] = spare ? 0.f : acc;
     }
 }
 
@@ -166,8 +169,8 @@ extern "C" int IV2_ENTRY(infllmv2_varlen_bwd)(void* stream, const void* dout, co
                                    const int64_t* dv_strides, const int64_t* lse_strides, int n_uint64_per_row,
                                    float softmax_scale, int is_causal, int deterministic, int max_selected_blocks) {
     IV2_CHECK(head_dim == kHeadDim, "varlen_bwd: this build only supports head_dim 128 (got %d)", head_dim);
-    IV2_CHECK(num_heads_k > 0 && num_heads == num_heads_k * kGroup,
-              "varlen_bwd: requires num_heads == 16 * num_heads_k (got %d and %d)", num_heads, num_heads_k);
+    IV2_CHECK(valid_group(num_heads, num_heads_k),
+              "varlen_bwd: requires num_heads == g * num_heads_k with g in {1, 2, 4, 8, 16} (got %d and %d)", num_heads, num_heads_k);
     IV2_CHECK(batch > 0 && total_q >= 0 && total_k >= 0 && max_seqlen_q >= 0 && max_seqlen_k >= 0, "varlen_bwd: bad sizes");
     IV2_CHECK(dout && q && k && v && out && softmax_lse && dq && dk && dv && cu_seqlens_q && cu_seqlens_k && workspace,
               "varlen_bwd: null pointer");
@@ -211,6 +214,7 @@ extern "C" int IV2_ENTRY(infllmv2_varlen_bwd)(void* stream, const void* dout, co
     p.dv = static_cast<elem_bits*>(dv);
     p.fwd_mask = fwd_blockmask;
     p.cu_seqlens_q = cu_seqlens_q; p.cu_seqlens_k = cu_seqlens_k;
+    p.group = num_heads / num_heads_k;
     p.q_tok = q_strides[0]; p.q_grp = q_strides[1]; p.q_kvh = q_strides[2];
     p.do_tok = do_strides[0]; p.do_grp = do_strides[1]; p.do_kvh = do_strides[2];
     p.o_tok = o_strides[0]; p.o_grp = o_strides[1]; p.o_kvh = o_strides[2];

@@ -209,7 +209,8 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
     // Which 16 bytes a lane fetches: the four lanes of a quad take the four 16-byte pieces of one head's 64-byte
     // chunk, so a quad is one contiguous 64-byte request.  LDS unit l = 4 * head + j of a chunk then holds piece
     // (j + head / 4) % 4: the rotation makes the operand reads below bank-conflict free.
-    const int dma_head = lane >> 2, dma_piece = ((lane & 3) + (lane >> 4)) & 3;
+    const int dma_piece = ((lane & 3) + (lane >> 4)) & 3;
+    const int dma_head = (lane >> 2) < p.group ? (lane >> 2) : p.group - 1;    // rows beyond the group repeat its last head: their LSE is +inf
     const uint32_t q_lane = static_cast<uint32_t>((dma_head * p.q_grp + 8 * dma_piece) * 2);   // byte offsets inside one token and KV head
     const uint32_t do_lane = static_cast<uint32_t>((dma_head * p.do_grp + 8 * dma_piece) * 2);
     const uint32_t stat_lane = static_cast<uint32_t>((lane & 31) * 4);

@@ -146,16 +146,18 @@ void bwd_dq_hybrid_kernel(const BwdParams p, const DqExtra x) {
     // ---- this token's operands ----
     elem8 qf[4], dof[4];
     {
-        const elem_bits* qp = p.q + tok * p.q_tok + h * p.q_kvh + n * p.q_grp + 8 * g;
-        const elem_bits* dp = p.dout + tok * p.do_tok + h * p.do_kvh + n * p.do_grp + 8 * g;
+        const int nq = n < p.group ? n : p.group - 1;          // rows beyond the group repeat its last head; their LSE is +inf
+        const elem_bits* qp = p.q + tok * p.q_tok + h * p.q_kvh + nq * p.q_grp + 8 * g;
+        const elem_bits* dp = p.dout + tok * p.do_tok + h * p.do_kvh + nq * p.do_grp + 8 * g;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             qf[c] = *reinterpret_cast<const elem8*>(qp + 32 * c);
             dof[c] = *reinterpret_cast<const elem8*>(dp + 32 * c);
         }
     }
-    float lse2 = p.lse[h * p.lse_kvh + tok * p.lse_tok + n * p.lse_grp] * kLog2e;
-    float dsum = p.dsum[static_cast<int64_t>(h) * p.total_q * 16 + tok * 16 + n];
+    const float* rs = p.rowstat + (static_cast<int64_t>(h) * p.total_q + tok) * 32;    // [LSE * log2(e) x 16 | D x 16]
+    float lse2 = rs[n];
+    float dsum = rs[16 + n];
     const floatx4 neg_dsum = {-dsum, -dsum, -dsum, -dsum};     // the dP accumulators start here: dS = P (dP - D) is then one product
     floatx4 dq[8];
 #pragma unroll
@@ -336,7 +338,7 @@ void bwd_dq_hybrid_kernel(const BwdParams p, const DqExtra x) {
             jp = jn;
         }
     }
-    if (!live) return;
+    if (!live || n >= p.group) return;
 
     elem_bits* op = p.dq + tok * p.dq_tok + h * p.dq_kvh + n * p.dq_grp + 4 * g;
 #pragma unroll

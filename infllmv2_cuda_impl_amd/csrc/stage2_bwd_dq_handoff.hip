@@ -288,7 +288,7 @@ void bwd_dq_handoff_kernel(const BwdParams p, const HoExtra x) {
         if (c0 < 0 && o0 < 0) break;
         turn(kb, ka);
     }
-    if (!live) return;
+    if (!live || n >= p.group) return;
 
     elem_bits* op = p.dq + tok * p.dq_tok + h * p.dq_kvh + n * p.dq_grp + 4 * g;
 #pragma unroll

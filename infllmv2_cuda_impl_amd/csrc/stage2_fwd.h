@@ -19,6 +19,7 @@ struct FwdParams {
     int64_t n_slots;
     int64_t total_q;
     int n64;
+    int group;                      // query heads per KV head, 1..16: MFMA rows >= group repeat head group - 1 and are never stored
     float scale_log2;               // softmax_scale * log2(e)
 };
 

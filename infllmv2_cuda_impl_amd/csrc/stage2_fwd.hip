@@ -117,7 +117,8 @@ void stage2_fwd_kernel(const FwdParams p) {
     const int64_t tok = static_cast<int64_t>(q0) + i;
     const int n = lane & 15, g = lane >> 4;
 
-    const elem_bits* qp = p.q + tok * p.q_tok_stride + h * p.q_kvh_stride + n * p.q_grp_stride + 8 * g;
+    const int nq = n < p.group ? n : p.group - 1;               // rows beyond the group repeat its last head and are never stored
+    const elem_bits* qp = p.q + tok * p.q_tok_stride + h * p.q_kvh_stride + nq * p.q_grp_stride + 8 * g;
     elem8 qf[4];
 #pragma unroll
     for (int c = 0; c < 4; ++c) qf[c] = *reinterpret_cast<const elem8*>(qp + 32 * c);
@@ -213,6 +214,7 @@ void stage2_fwd_kernel(const FwdParams p) {
 
     const float l_tot = wave_sum_over_g(l);
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    if (n >= p.group) return;
     elem_bits* op = p.out + tok * p.o_tok_stride + h * p.o_kvh_stride + n * p.o_grp_stride + 4 * g;
 #pragma unroll
     for (int dt = 0; dt < 8; ++dt) {
@@ -289,8 +291,8 @@ extern "C" int IV2_ENTRY(infllmv2_varlen_fwd)(void* stream, const void* q, const
                                    const int64_t* o_strides, const int64_t* lse_strides,
                                    int n_uint64_per_row, float softmax_scale, int is_causal) {
     IV2_CHECK(head_dim == kHeadDim, "varlen_fwd: this build only supports head_dim 128 (got %d)", head_dim);
-    IV2_CHECK(num_heads_k > 0 && num_heads == num_heads_k * kGroup,
-              "varlen_fwd: requires num_heads == 16 * num_heads_k (got %d and %d)", num_heads, num_heads_k);
+    IV2_CHECK(valid_group(num_heads, num_heads_k),
+              "varlen_fwd: requires num_heads == g * num_heads_k with g in {1, 2, 4, 8, 16} (got %d and %d)", num_heads, num_heads_k);
     IV2_CHECK(batch > 0 && total_q >= 0 && total_k >= 0 && max_seqlen_q >= 0 && max_seqlen_k >= 0, "varlen_fwd: bad sizes");
     IV2_CHECK(q && out && softmax_lse && cu_seqlens_q && cu_seqlens_k && workspace, "varlen_fwd: null pointer");
     IV2_CHECK(num_heads_k <= 65535 && batch <= 65535, "varlen_fwd: batch and num_heads_k must not exceed 65535");
@@ -323,6 +325,7 @@ extern "C" int IV2_ENTRY(infllmv2_varlen_fwd)(void* stream, const void* q, const
     fp.lse_tok_stride = lse_strides[0]; fp.lse_grp_stride = lse_strides[1]; fp.lse_kvh_stride = lse_strides[2];
     fp.n_slots = n_slots;
     fp.total_q = total_q;
+    fp.group = num_heads / num_heads_k;
     fp.n64 = n_uint64_per_row;
     fp.scale_log2 = softmax_scale * 1.44269504088896340736f;
     static const bool per_token = [] {                         // diagnostic switch: the one-wavefront-per-token kernel

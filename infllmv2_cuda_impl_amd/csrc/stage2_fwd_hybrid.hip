@@ -174,7 +174,8 @@ void stage2_fwd_hybrid_kernel(const FwdParams p, const HybridExtra x) {
     // ---- Q operand ----
     elem8 qf[4];
     {
-        const elem_bits* qp = p.q + tok * p.q_tok_stride + h * p.q_kvh_stride + n * p.q_grp_stride + 8 * g;
+        const int nq = n < p.group ? n : p.group - 1;
+        const elem_bits* qp = p.q + tok * p.q_tok_stride + h * p.q_kvh_stride + nq * p.q_grp_stride + 8 * g;
 #pragma unroll
         for (int c = 0; c < 4; ++c) qf[c] = *reinterpret_cast<const elem8*>(qp + 32 * c);
     }
@@ -327,6 +328,7 @@ void stage2_fwd_hybrid_kernel(const FwdParams p, const HybridExtra x) {
     // ---- epilogue ----
     const float l_tot = wave_sum_over_g(l);
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    if (n >= p.group) return;                                  // rows that only fill the MFMA tile
     elem_bits* op = p.out + tok * p.o_tok_stride + h * p.o_kvh_stride + n * p.o_grp_stride + 4 * g;
 #pragma unroll
     for (int dt = 0; dt < 8; ++dt) {

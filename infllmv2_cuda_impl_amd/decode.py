@@ -68,8 +68,8 @@ def decode_with_kvcache(q, k_cache, v_cache, k_new, v_new, cache_seqlens, softma
         raise RuntimeError("this build only supports head dimension 128")
     if Hq % Hk != 0:
         raise RuntimeError("Number of heads in key/value must divide number of heads in query")
-    if Hq != GROUP * Hk:
-        raise RuntimeError("this build requires 16 query heads per key/value head")
+    if Hq // Hk not in (1, 2, 4, 8, 16):
+        raise RuntimeError("this build requires 1, 2, 4, 8 or 16 query heads per key/value head")
     if seqlen_q != 1:
         raise RuntimeError("this build only supports seqlen_q == 1 in infllmv2_attn_with_kvcache")
     if paged:

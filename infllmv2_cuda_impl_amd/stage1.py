@@ -54,7 +54,7 @@ def stage1_scores(q, k, v, cu_seqlens_q, cu_seqlens_k, cu_seqlens_v, max_seqlen_
         _lib.call_for(q.dtype, "infllmv2_varlen_fwd_stage1", stream_ptr(q.device), q.data_ptr(), k.data_ptr(), v.data_ptr(),
                   buf.data_ptr(), cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), cu_seqlens_v.data_ptr(), batch,
                   total_q, Hq, Hk, d, max_seqlen_q, max_seqlen_k,
-                  _lib.i64_array([q.stride(0), q.stride(1), GROUP * q.stride(1)]),
+                  _lib.i64_array([q.stride(0), q.stride(1), (Hq // Hk) * q.stride(1)]),
                   _lib.i64_array([k.stride(0), k.stride(1)]), _lib.i64_array([v.stride(0), v.stride(1)]),
                   buf.stride(0), buf.stride(1), float(softmax_scale), int(bool(causal)))
     return buf if row == max_seqlen_k else buf[:, :, :max_seqlen_k]
@@ -91,7 +91,7 @@ def stage1_pooled(q, k, v, cu_seqlens_q, cu_seqlens_k, cu_seqlens_v, max_seqlen_
                   out.data_ptr(), cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), cu_seqlens_v.data_ptr(),
                   cache_lens.data_ptr() if cache_lens is not None else None, int(cache_len), batch, total_q, Hq, Hk, d,
                   max_seqlen_q, max_seqlen_k,
-                  _lib.i64_array([q.stride(0), q.stride(1), GROUP * q.stride(1)]),
+                  _lib.i64_array([q.stride(0), q.stride(1), (Hq // Hk) * q.stride(1)]),
                   _lib.i64_array([k.stride(0), k.stride(1)]), _lib.i64_array([v.stride(0), v.stride(1)]),
                   out_len, float(softmax_scale), int(bool(causal)), per_block + 1, per_block, 1, block_size,
                   local_blocks, init_blocks)
@@ -121,7 +121,7 @@ def stage1_decode(q, k, v, *, cu_seqlens_q=None, cu_seqlens_k=None, k_lens=None,
         _lib.call_for(q.dtype, "infllmv2_stage1_decode", stream_ptr(q.device), q.data_ptr(), k.data_ptr(), v.data_ptr(),
                   out.data_ptr(), p(cu_seqlens_q), p(cu_seqlens_k), p(k_lens), p(cu_seqlens_v), p(v_lens),
                   workspace.data_ptr(), workspace.numel(), batch, Hq, Hk, d, max_seqlen_k, max_seqlen_v,
-                  _lib.i64_array([q.stride(0), q.stride(-2), GROUP * q.stride(-2)]),
+                  _lib.i64_array([q.stride(0), q.stride(-2), (Hq // Hk) * q.stride(-2)]),
                   key_strides(k, cu_seqlens_k is not None), key_strides(v, cu_seqlens_v is not None),
                   out_head_stride, out_row_stride, float(softmax_scale), int(bool(causal)), int(bool(pooled)),
                   p(cache_lens), int(cache_len), int(out_len), per_block + 1, per_block, 1, block_size,

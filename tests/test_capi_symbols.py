@@ -58,7 +58,7 @@ def test_new_entry_points_validate_before_launch():
     assert rc != 0 and "head_dim 128" in _err(lib)
     rc = lib.infllmv2_varlen_fwd_stage1(None, fake, fake, fake, fake, fake, fake, fake, 1, 128, 24, 2, 128, 128, 7,
                                         i64([4096, 128, 2048]), i64([256, 128]), i64([256, 128]), 896, 7, 0.088, 1)
-    assert rc != 0 and "16 * num_heads_k" in _err(lib)
+    assert rc != 0 and "g * num_heads_k" in _err(lib)
     rc = lib.infllmv2_varlen_fwd_stage1(None, fake + 2, fake, fake, fake, fake, fake, fake, 1, 128, 32, 2, 128, 128, 7,
                                         i64([4096, 128, 2048]), i64([256, 128]), i64([256, 128]), 896, 7, 0.088, 1)
     assert rc != 0 and "16-byte aligned" in _err(lib)
