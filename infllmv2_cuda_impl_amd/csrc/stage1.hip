@@ -103,6 +103,24 @@ __device__ __forceinline__ float fold_rows32(float x, float y) {
     const u2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(y), false, false);
     return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
+// value of lane (n + k) % 16 of the same 16-lane row (DPP row_ror:k)
+template <int kRot>
+__device__ __forceinline__ float dpp_row_ror(float x) {
+    return __uint_as_float(__builtin_amdgcn_mov_dpp(__float_as_uint(x), 0x120 + kRot, 0xF, 0xF, false));
+}
+// maximum / sum over the 16 lanes of a row, left in every lane: rotations by 8, 4, 2, 1 each double the covered set
+__device__ __forceinline__ float row16_max(float x) {
+    x = fmaxf(x, dpp_row_ror<8>(x));
+    x = fmaxf(x, dpp_row_ror<4>(x));
+    x = fmaxf(x, dpp_row_ror<2>(x));
+    return fmaxf(x, dpp_row_ror<1>(x));
+}
+__device__ __forceinline__ float row16_sum(float x) {
+    x += dpp_row_ror<8>(x);
+    x += dpp_row_ror<4>(x);
+    x += dpp_row_ror<2>(x);
+    return x + dpp_row_ror<1>(x);
+}
 __device__ __forceinline__ float dpp_quad_xor1(float x) {
     return __uint_as_float(__builtin_amdgcn_mov_dpp(__float_as_uint(x), 0xB1, 0xF, 0xF, false));    // quad_perm:[1,0,3,2]
 }
@@ -202,25 +220,40 @@ void stage1_kernel(const Stage1Params p) {
         }
         // only the tile that holds a token's last visible key needs the per-key test
         const bool cut = (ti + 1) * 64 > min_vis_c;            // uniform per wavefront
+        if (!cut) {
+            // every key of the tile is visible to both tokens: the maximum is finite, no key test, and the scale
+            // rides in the multiply-add that feeds exp2
 #pragma unroll
-        for (int t = 0; t < kTokPerWave; ++t) {
+            for (int t = 0; t < kTokPerWave; ++t) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                float v[4];
+                for (int e = 0; e < 4; ++e) {
+                    const float mx = fmaxf(fmaxf(s[t][0][e], s[t][1][e]), fmaxf(s[t][2][e], s[t][3][e]));
+                    const float m_new = fmaxf(m[t][e], mx * p.scale_log2);
+                    float acc = l[t][e] * __builtin_amdgcn_exp2f(m[t][e] - m_new);
 #pragma unroll
-                for (int kt = 0; kt < 4; ++kt) v[kt] = s[t][kt][e] * p.scale_log2;
-                if (cut) {
-#pragma unroll
-                    for (int kt = 0; kt < 4; ++kt) v[kt] = (ti * 64 + kt * 16 + n < vis_c[t]) ? v[kt] : -INFINITY;
+                    for (int kt = 0; kt < 4; ++kt) acc += __builtin_amdgcn_exp2f(s[t][kt][e] * p.scale_log2 - m_new);
+                    l[t][e] = acc;
+                    m[t][e] = m_new;
                 }
-                const float mx = fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3]));
-                const float m_new = fmaxf(m[t][e], mx);
-                const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-                float acc = l[t][e] * __builtin_amdgcn_exp2f(m[t][e] - m_use);
+            }
+        } else {
 #pragma unroll
-                for (int kt = 0; kt < 4; ++kt) acc += __builtin_amdgcn_exp2f(v[kt] - m_use);
-                l[t][e] = acc;
-                m[t][e] = m_new;
+            for (int t = 0; t < kTokPerWave; ++t) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float v[4];
+#pragma unroll
+                    for (int kt = 0; kt < 4; ++kt)
+                        v[kt] = (ti * 64 + kt * 16 + n < vis_c[t]) ? s[t][kt][e] * p.scale_log2 : -INFINITY;
+                    const float mx = fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3]));
+                    const float m_new = fmaxf(m[t][e], mx);
+                    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+                    float acc = l[t][e] * __builtin_amdgcn_exp2f(m[t][e] - m_use);
+#pragma unroll
+                    for (int kt = 0; kt < 4; ++kt) acc += __builtin_amdgcn_exp2f(v[kt] - m_use);
+                    l[t][e] = acc;
+                    m[t][e] = m_new;
+                }
             }
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");         // this wavefront's share of the next tile has landed
@@ -232,16 +265,10 @@ void stage1_kernel(const Stage1Params p) {
     for (int t = 0; t < kTokPerWave; ++t)
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            float mm = m[t][e], ll = l[t][e];
-#pragma unroll
-            for (int off = 1; off < 16; off <<= 1) {
-                const float mo = __shfl_xor(mm, off);
-                const float lo = __shfl_xor(ll, off);
-                const float mn = fmaxf(mm, mo);
-                const float mu = (mn == -INFINITY) ? 0.f : mn;
-                ll = ll * __builtin_amdgcn_exp2f(mm - mu) + lo * __builtin_amdgcn_exp2f(mo - mu);
-                mm = mn;
-            }
+            // the row's maximum first, then every lane's sum rescaled to it once, then the sum of those
+            const float mm = row16_max(m[t][e]);
+            const float mu = (mm == -INFINITY) ? 0.f : mm;
+            const float ll = row16_sum(l[t][e] * __builtin_amdgcn_exp2f(m[t][e] - mu));
             lse2[t][e] = mm + __builtin_amdgcn_logf(ll);        // v_log_f32 is log2
             if (4 * g + e >= p.group) lse2[t][e] = INFINITY;    // a row that only fills the tile: exp2(x - inf) = 0 in the head sum
         }
