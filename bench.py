@@ -274,7 +274,7 @@ def stream_probes(torch, _lib, dev):
     out = torch.zeros(2 * wgs, dtype=torch.int64, device=dev)
     stream = torch.cuda.current_stream(dev).cuda_stream
     record = {}
-    for mode, name in ((0, "global_load_dwordx4"), (1, "lds_dma_dwordx4"), (2, "ds_read_b128")):
+    for mode, name in ((0, "global_load_dwordx4"), (1, "lds_dma_dwordx4"), (2, "ds_read_b128"), (3, "ds_read_b64_tr_b16")):
         launch = lambda: _lib.call("infllmv2_probe_stream", stream, src.data_ptr(), src.numel() * 4, out.data_ptr(),
                                    wgs, iters, mode)
         ms = min(event_ms(torch, launch, 3) for _ in range(3))

@@ -38,7 +38,7 @@ int infllmv2_check_device(int device);
 
 /* Measurement aid, no counterpart in the reference and not on the attention path: `workgroups` workgroups of eight
  * wavefronts each re-read their own 128 KiB of `src` `iters` times with global_load_dwordx4 (mode 0), LDS-DMA
- * (mode 1) or ds_read_b128 from an LDS copy (mode 2).  out[2 w] = cycle-counter ticks workgroup w took, out[2 w + 1] =
+ * (mode 1), ds_read_b128 from an LDS copy (mode 2) or ds_read_b64_tr_b16 from it (mode 3).  out[2 w] = cycle-counter ticks workgroup w took, out[2 w + 1] =
  * bytes it moved: with one workgroup per CU, bytes over time is what a CU's L1 return path (modes 0, 1) or its LDS
  * (mode 2) delivers, the rates the Stage-2 gather is held against. */
 int infllmv2_probe_stream(void* stream, const void* src, size_t src_bytes, unsigned long long* out, int workgroups,
