@@ -115,6 +115,22 @@ def _check_qkv(q, k, v, cu_seqlens_q, cu_seqlens_k, same_kv_len=True):
     return batch
 
 
+HEAD_DIM = 128      # the head size the kernels are laid out for (static_switch.h:79-89 instantiates the same one)
+
+
+def pad_head_dim(*tensors):
+    """Zero-pads the last dimension of every tensor to 128, as the reference's wrapper pads it to a multiple of 8 before
+    its kernels and slices the result afterwards (infllmv2_sparse_attention.py:299-303, 336, 352-355, 381).  Zeros
+    in q/k leave every dot product unchanged, zeros in v give zero output columns, and the padding is differentiable,
+    so gradients come back at the original width.  Returns the tensors (unchanged objects when already 128 wide)."""
+    d = tensors[0].shape[-1]
+    if d == HEAD_DIM:
+        return tensors
+    if d > HEAD_DIM or d < 1:
+        raise RuntimeError("this build only supports head dimension at most 128")
+    return tuple(torch.nn.functional.pad(t, [0, HEAD_DIM - d]) for t in tensors)
+
+
 def _natural_strides(t: torch.Tensor, group: int = GROUP):
     """{token, head-in-group, kv-head} element strides of a (T, Hq, d) tensor."""
     return _lib.i64_array([t.stride(0), t.stride(1), group * t.stride(1)])
@@ -223,10 +239,22 @@ def infllmv2_attn_varlen_func(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q,
     ``block_mask`` (not in the reference's signature) is the packed form of the same selection, int64
     ``(nheads_k, total_q, ceil(ceil(max_seqlen_k / 64) / 64))`` as ``topk_to_uint64`` / ``topk_blocks(return_mask=True)``
     produce it; when given it is used as is and ``topk_idx`` only bounds the blocks per row for the backward.
+    Head sizes below 128 are served by zero padding (see :func:`pad_head_dim`); ``softmax_scale`` then defaults to
+    the caller's head size ``** -0.5``, as in the reference.
     """
-    return Infllmv2AttnVarlenFunc.apply(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p,
-                                        softmax_scale, causal, window_size, softcap, alibi_slopes, deterministic,
-                                        return_attn_probs, block_table, topk_idx, block_mask)
+    head_size_og = q.shape[-1]
+    if head_size_og != HEAD_DIM and q.dim() == 3 and k.dim() == 3 and v.dim() == 3:
+        if softmax_scale is None:
+            softmax_scale = head_size_og ** (-0.5)
+        q, k, v = pad_head_dim(q, k, v)
+    res = Infllmv2AttnVarlenFunc.apply(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p,
+                                       softmax_scale, causal, window_size, softcap, alibi_slopes, deterministic,
+                                       return_attn_probs, block_table, topk_idx, block_mask)
+    if head_size_og == HEAD_DIM:
+        return res
+    if isinstance(res, tuple):
+        return (res[0][..., :head_size_og],) + tuple(res[1:])
+    return res[..., :head_size_og]
 
 
 def infllmv2_attn_stage1(q, k, v, cu_seqlens_q, cu_seqlens_k, cu_seqlens_v, max_seqlen_q, max_seqlen_k,
@@ -243,6 +271,8 @@ def infllmv2_attn_stage1(q, k, v, cu_seqlens_q, cu_seqlens_k, cu_seqlens_v, max_
     from .stage1 import stage1_scores
     if softmax_scale is None:
         softmax_scale = q.shape[-1] ** (-0.5)
+    if q.shape[-1] != HEAD_DIM and q.dim() == 3 and k.dim() == 3 and v.dim() == 3:
+        q, k, v = pad_head_dim(q, k, v)                        # scores depend on dot products only
     causal = _reject_unsupported(dropout_p, window_size, softcap, alibi_slopes, causal, max_seqlen_k)
     if block_table is not None:
         raise RuntimeError("paged KV (block_table) is not supported by this build")
@@ -270,6 +300,8 @@ def infllmv2_attn_stage1_pooled(q, k, v, cu_seqlens_q, cu_seqlens_k, cu_seqlens_
     from .stage1 import stage1_pooled
     if softmax_scale is None:
         softmax_scale = q.shape[-1] ** (-0.5)
+    if q.shape[-1] != HEAD_DIM and q.dim() == 3 and k.dim() == 3 and v.dim() == 3:
+        q, k, v = pad_head_dim(q, k, v)
     q, k, v = [_dense_last_dim(x) for x in (q, k, v)]
     _check_qkv(q, k, v, cu_seqlens_q, cu_seqlens_k, same_kv_len=False)
     if cu_seqlens_v.dtype != torch.int32:

@@ -130,7 +130,11 @@ def select_blocks(q: torch.Tensor, k: torch.Tensor, cu_seqlens_q: torch.Tensor, 
     ``(topk_idx, block_mask)`` and the mask (as wide as ``max_seqlen_k`` needs) can be handed to
     ``infllmv2_attn_varlen_func(block_mask=...)``.
     """
-    from .attention import infllmv2_attn_stage1_pooled
+    from .attention import infllmv2_attn_stage1_pooled, pad_head_dim, HEAD_DIM
+    if q.shape[-1] != HEAD_DIM:
+        if softmax_scale is None:
+            softmax_scale = q.shape[-1] ** (-0.5)
+        q, k = pad_head_dim(q, k)                              # the mean of zero columns is zero
     kf, cu_f = compress_keys(k, cu_seqlens_k, max_seqlen_k, kernel_size, stride)
     if exact_lse:
         kc, cu_c = kf, cu_f

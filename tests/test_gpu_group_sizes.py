@@ -1,4 +1,5 @@
-"""Group sizes other than 16 (1, 2, 4, 8 query heads per KV head) through every attention entry point.
+"""Group sizes other than 16 (1, 2, 4, 8 query heads per KV head) through every attention entry point, and head
+sizes below 128 through the wrappers that pad them.
 
 The reference's Python is written for any group size (infllmv2_sparse_attention.py:76-88, 546-555) but its native code
 divides by 16 everywhere (flash_api.cpp:706-710, 941, 1397): only 16 runs there.  Here smaller groups run on the same
@@ -179,4 +180,52 @@ def test_unsupported_group_is_rejected(ops):
     q, k, v = rand((64, 6, 128), 20).to(DEV), rand((64, 2, 128), 21).to(DEV), rand((64, 2, 128), 22).to(DEV)
     cu = torch.tensor([0, 64], dtype=torch.int32, device=DEV)
     with pytest.raises(RuntimeError, match="1, 2, 4, 8 or 16"):
+        ops.infllmv2_attn_varlen_func(q, k, v, cu, cu, 64, 64, causal=True)
+
+
+@pytest.mark.parametrize("d", [64, 80, 32])
+def test_head_sizes_below_128_by_zero_padding(ops, d):
+    """The wrapper pads the head dimension with zeros up to the kernels' 128, as the reference's wrapper pads it to a
+    multiple of 8 (infllmv2_sparse_attention.py:299-303, 336, 381): forward, gradients (at the caller's width) and the
+    selection front end against the oracle at the original head size, default scale d ** -0.5."""
+    seqs = [400, 270]
+    T, G, Hk = sum(seqs), 16, 2
+    q, k, v, dout = rand((T, G * Hk, d), 30), rand((T, Hk, d), 31), rand((T, Hk, d), 32), rand((T, G * Hk, d), 33)
+    idx = random_selection(34, Hk, seqs, 4)
+    cu_np = np.cumsum([0] + seqs).astype(np.int32)
+    cu = torch.from_numpy(cu_np).to(DEV)
+    qg, kg, vg = [t.to(DEV).requires_grad_(True) for t in (q, k, v)]
+    out = ops.infllmv2_attn_varlen_func(qg, kg, vg, cu, cu, max(seqs), max(seqs), causal=True, topk_idx=idx.to(DEV))
+    assert tuple(out.shape) == (T, G * Hk, d)
+    out.backward(dout.to(DEV))
+    words = O.topk_to_uint64(idx.numpy(), max(seqs), 64)[0]
+    qn, kn, vn, dn = [bf16_np(t) for t in (q, k, v, dout)]
+    ref_o, _ = O.stage2_forward(qn, kn, vn, cu_np, cu_np, words, d ** -0.5, True)
+    err = np.abs(bf16_np(out).astype(np.float64) - ref_o)
+    assert err.max() <= 2e-2 and err.mean() <= 1e-3, (err.max(), err.mean())
+    dq, dk, dv = O.stage2_backward(qn, kn, vn, dn, cu_np, cu_np, words, d ** -0.5, True)
+    for name, got, ref in (("dq", qg.grad, dq), ("dk", kg.grad, dk), ("dv", vg.grad, dv)):
+        assert tuple(got.shape) == ref.shape
+        s = max(1.0, float(np.abs(ref).max()))
+        e = np.abs(bf16_np(got).astype(np.float64) - ref)
+        assert e.max() <= 2e-2 * s and e.mean() <= 1e-3 * s, (name, e.max(), e.mean(), s)
+    # Stage 1 on compressed keys of the original width
+    kf, cu_f = O.compress_keys(kn, cu_np, 32, 16)
+    kc, cu_c = O.compress_keys(kn, cu_np, 128, 64)
+    Lk = int(max(np.diff(cu_f)))
+    t = lambda x, dt=None: torch.from_numpy(np.ascontiguousarray(x)).to(DEV) if dt is None else torch.from_numpy(np.ascontiguousarray(x)).to(dt).to(DEV)
+    score = ops.infllmv2_attn_stage1(q.to(DEV), t(kf, BF), t(kc, BF), cu, t(cu_f), t(cu_c), max(seqs), Lk, causal=True)
+    ref = O.stage1_scores(qn, kf, kc, cu_np, cu_f, cu_c, Lk, d ** -0.5, True, round_output=False)
+    assert (np.abs(bf16_np(score).astype(np.float64) - ref) <= 2.0 ** -7 * np.abs(ref) + 2e-3).all()
+    # the whole front end picks what top-k of the pooled oracle-side GPU scores gives
+    cache_lens = torch.zeros(2, dtype=torch.int32, device=DEV)
+    sel = ops.select_blocks(q.to(DEV), k.to(DEV), cu, cu, max(seqs), max(seqs), 5, 1, 1, cache_lens=cache_lens)
+    pooled = ops.max_pooling_1d_varlen(score, cu, t(cu_f), cache_lens, max(seqs), Lk, 1, 1)
+    assert torch.equal(sel, ops.topk_blocks(pooled, 5))
+
+
+def test_head_size_above_128_is_rejected(ops):
+    q, k, v = rand((64, 32, 256), 35).to(DEV), rand((64, 2, 256), 36).to(DEV), rand((64, 2, 256), 37).to(DEV)
+    cu = torch.tensor([0, 64], dtype=torch.int32, device=DEV)
+    with pytest.raises(RuntimeError, match="at most 128"):
         ops.infllmv2_attn_varlen_func(q, k, v, cu, cu, 64, 64, causal=True)
