@@ -110,19 +110,10 @@ __device__ __forceinline__ void s1d_run(int tiles, int splits, int split, int& t
     t1 = t1 < tiles ? t1 : tiles;
 }
 
-__global__ __launch_bounds__(64)
-void stage1_decode_lse_kernel(const S1DecodeParams p) {
-    const int lane = threadIdx.x, n = lane & 15, g = lane >> 4;
-    const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
-    const S1DecodeSeq sq = s1d_sequence(p, b, h);
-    if (sq.Sq <= 0) return;
-    const int s1 = (sq.Lk == sq.Lc) ? 16 : 64;                 // flash_fwd_kernel.h:1236-1240
-    const int vis_c = s1d_visible(s1, sq.Lc, p.causal != 0);
-    int t0, t1;
-    s1d_run((vis_c + 63) >> 6, p.splits_c, split, t0, t1);
-
-    elem8 qf[4];
-    s1d_load_q(qf, p, sq, h, n, g);
+// (max, sum) in log2 units of head 4g + e over the coarse tiles [t0, t1) of one sequence and KV head, merged over the
+// 16 key-column lanes: every lane of row g returns the values of its four heads.
+__device__ __forceinline__ void s1d_lse_run(const S1DecodeParams& p, const S1DecodeSeq& sq, const elem8 (&qf)[4], int vis_c,
+                                            int t0, int t1, int n, int g, float (&m_out)[4], float (&l_out)[4]) {
     float m[4], l[4];                                          // head 4g + e over the keys == n (mod 16) of the run
 #pragma unroll
     for (int e = 0; e < 4; ++e) { m[e] = -INFINITY; l[e] = 0.f; }
@@ -168,7 +159,6 @@ void stage1_decode_lse_kernel(const S1DecodeParams p) {
         }
     }
     // merge the 16 key-column lanes of each head
-    float* slot = p.partial + ((static_cast<int64_t>(b) * gridDim.y + h) * p.splits_c + split) * 32;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         float mm = m[e], ll = l[e];
@@ -181,7 +171,46 @@ void stage1_decode_lse_kernel(const S1DecodeParams p) {
             ll = ll * __builtin_amdgcn_exp2f(mm - mu) + lo * __builtin_amdgcn_exp2f(mo - mu);
             mm = mn;
         }
-        if (n == 0) { slot[4 * g + e] = mm; slot[16 + 4 * g + e] = ll; }
+        m_out[e] = mm;
+        l_out[e] = ll;
+    }
+}
+
+// log-sum-exp (log2 units) of head 4g + e from `count` partial records {max x 16, sum x 16} merged in order
+__device__ __forceinline__ void s1d_merge_partials(const float* part, int count, int g, int group, float (&lse2)[4]) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        float mm = -INFINITY, ll = 0.f;
+        for (int s = 0; s < count; ++s) {
+            const float mo = part[s * 32 + 4 * g + e], lo = part[s * 32 + 16 + 4 * g + e];
+            const float mn = fmaxf(mm, mo);
+            const float mu = (mn == -INFINITY) ? 0.f : mn;
+            ll = ll * __builtin_amdgcn_exp2f(mm - mu) + lo * __builtin_amdgcn_exp2f(mo - mu);
+            mm = mn;
+        }
+        lse2[e] = mm + __builtin_amdgcn_logf(ll);                // v_log_f32 is log2
+        if (4 * g + e >= group) lse2[e] = INFINITY;              // a row that only fills the tile adds exp2(x - inf) = 0
+    }
+}
+
+__global__ __launch_bounds__(64)
+void stage1_decode_lse_kernel(const S1DecodeParams p) {
+    const int lane = threadIdx.x, n = lane & 15, g = lane >> 4;
+    const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const S1DecodeSeq sq = s1d_sequence(p, b, h);
+    if (sq.Sq <= 0) return;
+    const int s1 = (sq.Lk == sq.Lc) ? 16 : 64;                 // flash_fwd_kernel.h:1236-1240
+    const int vis_c = s1d_visible(s1, sq.Lc, p.causal != 0);
+    int t0, t1;
+    s1d_run((vis_c + 63) >> 6, p.splits_c, split, t0, t1);
+    elem8 qf[4];
+    s1d_load_q(qf, p, sq, h, n, g);
+    float mm[4], ll[4];
+    s1d_lse_run(p, sq, qf, vis_c, t0, t1, n, g, mm, ll);
+    float* slot = p.partial + ((static_cast<int64_t>(b) * gridDim.y + h) * p.splits_c + split) * 32;
+    if (n == 0) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { slot[4 * g + e] = mm[e]; slot[16 + 4 * g + e] = ll[e]; }
     }
 }
 
@@ -202,47 +231,13 @@ __device__ __forceinline__ float s1d_quad_xor2(float x) {
     return __uint_as_float(__builtin_amdgcn_mov_dpp(__float_as_uint(x), 0x4E, 0xF, 0xF, false));
 }
 
+// Scores (or pooled block scores) of the fine tiles [t0, t1) of one sequence and KV head, by one wavefront; ta / tb
+// hold tiles t0 and t0 + 1 already (requested by the caller before it waited for the log-sum-exp).
 template <bool kPool>
-__global__ __launch_bounds__(64)
-void stage1_decode_score_kernel(const S1DecodeParams p) {
-    const int lane = threadIdx.x, n = lane & 15, g = lane >> 4;
-    const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
-    const S1DecodeSeq sq = s1d_sequence(p, b, h);
-    if (sq.Sq <= 0) return;
-    const int s1 = (sq.Lk == sq.Lc) ? 16 : 64;
-    const int vis_c = s1d_visible(s1, sq.Lc, p.causal != 0);
-    int vis_f = vis_c == 0 ? 0 : s1d_visible(16, sq.Lk, p.causal != 0);  // early exit of flash_fwd_kernel.h:1271-1276
-    if (kPool && vis_f > p.cols) vis_f = p.cols;               // the score row the pooling would have read ends there
-    const int tiles = (vis_f + 63) >> 6;
-    int t0, t1;
-    s1d_run(tiles, p.splits_f, split, t0, t1);
-    const bool owns_tail = tiles == 0 ? split == 0 : (t0 < t1 && t1 == tiles);
-    if (t0 >= t1 && !owns_tail) return;
-
-    elem8 qf[4];
-    s1d_load_q(qf, p, sq, h, n, g);
-    // the first two tiles are requested before anything waits on memory
-    elem8 ta[16], tb[16];
-    if (t0 < t1) s1d_load_tile(ta, sq.kbase, p.k_row_stride, t0 * 64, sq.Lk, n, g);
-    if (t0 + 1 < t1) s1d_load_tile(tb, sq.kbase, p.k_row_stride, (t0 + 1) * 64, sq.Lk, n, g);
-    // log-sum-exp of head 4g + e: the partials of the coarse runs merged in run order
-    float lse2[4];
-    {
-        const float* part = p.partial + (static_cast<int64_t>(b) * gridDim.y + h) * p.splits_c * 32;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            float mm = -INFINITY, ll = 0.f;
-            for (int s = 0; s < p.splits_c; ++s) {
-                const float mo = part[s * 32 + 4 * g + e], lo = part[s * 32 + 16 + 4 * g + e];
-                const float mn = fmaxf(mm, mo);
-                const float mu = (mn == -INFINITY) ? 0.f : mn;
-                ll = ll * __builtin_amdgcn_exp2f(mm - mu) + lo * __builtin_amdgcn_exp2f(mo - mu);
-                mm = mn;
-            }
-            lse2[e] = mm + __builtin_amdgcn_logf(ll);            // v_log_f32 is log2
-            if (4 * g + e >= p.group) lse2[e] = INFINITY;        // a row that only fills the tile adds exp2(x - inf) = 0
-        }
-    }
+__device__ __forceinline__ void s1d_score_run(const S1DecodeParams& p, const S1DecodeSeq& sq, const elem8 (&qf)[4],
+                                              const float (&lse2)[4], elem8 (&ta)[16], elem8 (&tb)[16], int vis_f,
+                                              int tiles, int t0, int t1, bool owns_tail, int b, int h, int lane) {
+    const int n = lane & 15, g = lane >> 4;
     const int64_t out_row = static_cast<int64_t>(h) * p.out_head_stride + static_cast<int64_t>(sq.q_row) * p.out_row_stride;
     elem_bits* out = p.out + out_row;
     const int bq = kPool ? ((p.cache_lens ? p.cache_lens[b] : p.cache_len) / kBlockN) : 0;   // the query's own key block
@@ -314,6 +309,87 @@ void stage1_decode_score_kernel(const S1DecodeParams p) {
             for (int kb = tiles * 16 + lane; kb < p.pool_len; kb += 64) out[kb] = pool_rest(kb, kb == tiles * 16 ? carry : 0.f);
         }
     }
+}
+
+// visible fine keys and tiles of a sequence (0 when no coarse key is visible: early exit of flash_fwd_kernel.h:1271-1276)
+template <bool kPool>
+__device__ __forceinline__ void s1d_fine_extent(const S1DecodeParams& p, const S1DecodeSeq& sq, int& vis_c, int& vis_f, int& tiles) {
+    const int s1 = (sq.Lk == sq.Lc) ? 16 : 64;                 // flash_fwd_kernel.h:1236-1240
+    vis_c = s1d_visible(s1, sq.Lc, p.causal != 0);
+    vis_f = vis_c == 0 ? 0 : s1d_visible(16, sq.Lk, p.causal != 0);
+    if (kPool && vis_f > p.cols) vis_f = p.cols;               // the score row the pooling would have read ends there
+    tiles = (vis_f + 63) >> 6;
+}
+
+template <bool kPool>
+__global__ __launch_bounds__(64)
+void stage1_decode_score_kernel(const S1DecodeParams p) {
+    const int lane = threadIdx.x, n = lane & 15, g = lane >> 4;
+    const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const S1DecodeSeq sq = s1d_sequence(p, b, h);
+    if (sq.Sq <= 0) return;
+    int vis_c, vis_f, tiles;
+    s1d_fine_extent<kPool>(p, sq, vis_c, vis_f, tiles);
+    int t0, t1;
+    s1d_run(tiles, p.splits_f, split, t0, t1);
+    const bool owns_tail = tiles == 0 ? split == 0 : (t0 < t1 && t1 == tiles);
+    if (t0 >= t1 && !owns_tail) return;
+
+    elem8 qf[4];
+    s1d_load_q(qf, p, sq, h, n, g);
+    // the first two tiles are requested before anything waits on memory
+    elem8 ta[16], tb[16];
+    if (t0 < t1) s1d_load_tile(ta, sq.kbase, p.k_row_stride, t0 * 64, sq.Lk, n, g);
+    if (t0 + 1 < t1) s1d_load_tile(tb, sq.kbase, p.k_row_stride, (t0 + 1) * 64, sq.Lk, n, g);
+    // log-sum-exp of head 4g + e: the partials of the coarse runs merged in run order
+    float lse2[4];
+    s1d_merge_partials(p.partial + (static_cast<int64_t>(b) * gridDim.y + h) * p.splits_c * 32, p.splits_c, g, p.group, lse2);
+    s1d_score_run<kPool>(p, sq, qf, lse2, ta, tb, vis_f, tiles, t0, t1, owns_tail, b, h, lane);
+}
+
+// Both passes in one launch, for batches with enough (sequence, KV head) pairs to fill the device without splitting a
+// pair over more than a few workgroups: a workgroup of 8 wavefronts splits ALL coarse tiles of its pair among its
+// wavefronts, merges their (max, sum) records through LDS, and then scores its part of the fine tiles, one run per
+// wavefront.  With `parts` workgroups per pair the coarse keys are read `parts` times (the repeats come from L2), which
+// is why this form is only used for parts <= 4; it saves the second launch and the trip of the records through memory.
+constexpr int kS1dFusedWaves = 8;
+template <bool kPool>
+__global__ __launch_bounds__(64 * kS1dFusedWaves)
+void stage1_decode_fused_kernel(const S1DecodeParams p) {
+    __shared__ float records[kS1dFusedWaves * 32];
+    const int lane = threadIdx.x & 63, n = lane & 15, g = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
+    const int part = blockIdx.x, parts = gridDim.x, h = blockIdx.y, b = blockIdx.z;
+    const S1DecodeSeq sq = s1d_sequence(p, b, h);
+    if (sq.Sq <= 0) return;                                    // uniform per workgroup
+    int vis_c, vis_f, tiles;
+    s1d_fine_extent<kPool>(p, sq, vis_c, vis_f, tiles);
+    const int split = part * kS1dFusedWaves + wave, splits = parts * kS1dFusedWaves;
+    int t0, t1;
+    s1d_run(tiles, splits, split, t0, t1);
+    const bool owns_tail = tiles == 0 ? split == 0 : (t0 < t1 && t1 == tiles);
+
+    elem8 qf[4];
+    s1d_load_q(qf, p, sq, h, n, g);
+    {
+        int c0, c1;
+        s1d_run((vis_c + 63) >> 6, kS1dFusedWaves, wave, c0, c1);
+        float mm[4], ll[4];
+        s1d_lse_run(p, sq, qf, vis_c, c0, c1, n, g, mm, ll);
+        if (n == 0) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { records[wave * 32 + 4 * g + e] = mm[e]; records[wave * 32 + 16 + 4 * g + e] = ll[e]; }
+        }
+    }
+    // the first two fine tiles are on their way while the records are exchanged
+    elem8 ta[16], tb[16];
+    if (t0 < t1) s1d_load_tile(ta, sq.kbase, p.k_row_stride, t0 * 64, sq.Lk, n, g);
+    if (t0 + 1 < t1) s1d_load_tile(tb, sq.kbase, p.k_row_stride, (t0 + 1) * 64, sq.Lk, n, g);
+    __syncthreads();
+    if (t0 >= t1 && !owns_tail) return;                        // per wavefront, after the only barrier
+    float lse2[4];
+    s1d_merge_partials(records, kS1dFusedWaves, g, p.group, lse2);
+    s1d_score_run<kPool>(p, sq, qf, lse2, ta, tb, vis_f, tiles, t0, t1, owns_tail, b, h, lane);
 }
 
 }  // namespace IV2_NS
@@ -404,6 +480,21 @@ extern "C" int IV2_ENTRY(infllmv2_stage1_decode)(void* stream, const void* q, co
     p.cache_lens = cache_lens; p.cache_len = cache_len; p.pool_len = out_len;
     p.local_blocks = local_blocks; p.init_blocks = init_blocks;
     hipStream_t st = static_cast<hipStream_t>(stream);
+    // enough pairs to fill the device with at most 4 workgroups of 8 wavefronts per pair: both passes in one launch
+    const int pairs = batch * num_heads_k;
+    if (pairs >= 64) {
+        int parts = (256 + pairs - 1) / pairs;
+        const int tiles_max = (max_seqlen_k + 63) / 64;
+        const int cap = (tiles_max + 2 * kS1dFusedWaves - 1) / (2 * kS1dFusedWaves);    // no run shorter than two tiles of the longest sequence
+        if (parts > cap) parts = cap;
+        if (parts > 4) parts = 4;
+        if (parts < 1) parts = 1;
+        const dim3 fgrid(parts, num_heads_k, batch);
+        if (pooled) hipLaunchKernelGGL(stage1_decode_fused_kernel<true>, fgrid, dim3(64 * kS1dFusedWaves), 0, st, p);
+        else hipLaunchKernelGGL(stage1_decode_fused_kernel<false>, fgrid, dim3(64 * kS1dFusedWaves), 0, st, p);
+        IV2_LAUNCH_CHECK();
+        return 0;
+    }
     hipLaunchKernelGGL(stage1_decode_lse_kernel, dim3(p.splits_c, num_heads_k, batch), dim3(64), 0, st, p);
     IV2_LAUNCH_CHECK();
     const dim3 grid(p.splits_f, num_heads_k, batch);
