@@ -50,7 +50,7 @@ struct BwdParams {
 
 // dQ, 8 consecutive tokens per workgroup sharing their common blocks through LDS: stage2_bwd_dq.hip
 int launch_bwd_dq_hybrid(hipStream_t st, const BwdParams& p, int batch, int max_seqlen_q, bool causal);
-// dK/dV, one wavefront per (64-key block, 512-token slice): stage2_bwd_dkdv.hip
+// dK/dV, two wavefronts (32 keys each) per (64-key block, 512-token slice): stage2_bwd_dkdv.hip
 int launch_bwd_dkdv_wave(hipStream_t st, const BwdParams& p, int batch, int max_seqlen_q, bool causal);
 
 // dQ from the dS tiles handed over by the column kernel: stage2_bwd_dq_handoff.hip

@@ -1,26 +1,29 @@
-// Stage-2 backward, dK / dV (gfx950): one wavefront per (64-key block, 512-token slice).
+// Stage-2 backward, dK / dV (gfx950): two wavefronts per (64-key block, 512-token slice), each owning 32 of the keys.
 //
 // Mathematics as in compute_dq_dk_dv_1colblock (csrc/flash_attn/src/flash_bwd_kernel.h:498-794):
 // P = exp(scale S - LSE), dV += P^T dO, dS = P (dP - D), dK += scale dS^T Q, the 16 grouped heads
 // of a token accumulating into their KV head.
 //
-// Why one wavefront owns a whole key block.  Per (token, block) pair the query side is only 16
-// rows (the grouped heads), so every MFMA needs a fresh 1 KiB query-side operand unless that
-// operand is reused across key tiles.  Here the block's K and V (B operands of S = Q K^T and
-// dP = dO V^T, 128 registers) stay in VGPRs for the whole slice, the 64 x 128 dK^T and dV^T
-// tiles are the wavefront's 256 accumulation registers (AGPRs), and each query-side operand
-// fetched from LDS feeds four MFMAs.  No workgroup barrier and no cross-wavefront reduction is
-// left; the CU runs four such wavefronts, one per SIMD.
+// Why the key block stays put.  Per (token, block) pair the query side is only 16 rows (the grouped
+// heads), so every MFMA needs a fresh 1 KiB query-side operand unless that operand is reused across
+// key tiles.  Here a wavefront keeps its 32 keys of K and V (B operands of S = Q K^T and
+// dP = dO V^T, 64 registers) in VGPRs for the whole slice, its 32 x 128 dK^T and dV^T tiles are
+// 128 accumulation registers (AGPRs), and each query-side operand fetched from LDS feeds two MFMAs.
+// With 256 registers per wavefront a SIMD holds two of them (one wavefront owning all 64 keys needs
+// all 512 registers and then has nobody to fill its issue gaps: measured 6 % slower); the price is
+// that the two wavefronts of a block read every query-side fragment once each, which makes the LDS
+// pipe the busiest unit of the kernel.
 //
 // Query-side data path.  q and dout of a token pair are gathered straight from the caller's
 // tensors into a two-stage LDS ring by LDS-DMA loads issued one pair ahead (no registers, no
-// transposed copies in memory): the ring holds them as A-operand fragments of the first two
-// GEMMs, and the transposed operands of dV^T = dO^T P and dK^T = Q^T dS are read from the same
-// bytes with ds_read_b64_tr_b16.  Two tokens fill the 32-deep contraction of those GEMMs, and
-// the S / dS accumulator registers are, converted to bf16, their B operands.
+// transposed copies in memory; wavefront 0 fetches q, wavefront 1 dout, one workgroup barrier per
+// pair): the ring holds them as A-operand fragments of the first two GEMMs, and the transposed
+// operands of dV^T = dO^T P and dK^T = Q^T dS are read from the same bytes with ds_read_b64_tr_b16.
+// Two tokens fill the 32-deep contraction of those GEMMs, and the S / dS accumulator registers are,
+// converted to bf16, their B operands.
 //
-// The slice ends with one fp32 atomic flush of the two 64 x 128 tiles (transposed through the
-// ring's LDS so that every atomic instruction covers 256 contiguous bytes).
+// The slice ends with one fp32 atomic flush of the two tiles (transposed through the ring's LDS so
+// that every atomic instruction covers 256 contiguous bytes).
 #include "common.h"
 #include "kv_image.h"
 #include "stage2_bwd.h"
@@ -35,6 +38,7 @@ constexpr int kHeavyPairs = 128;                               // a slice with f
 constexpr int kStage = 16384 + 512 + 512;                      // q a|b, dout a|b (4 KiB each), the pair's 64 row scalars, its two rank records
 constexpr int kWaveLds = 2 * kStage;                           // = 64 rows x 132 floats: also the flush tile
 constexpr int kFlushPitch = 132;                               // floats per key row of the flush tile
+constexpr int kWaveTiles = 2;                                  // 16-key tiles per wavefront: a wavefront owns 32 of the block's 64 keys
 
 typedef short short4v __attribute__((ext_vector_type(4)));
 typedef int int4v __attribute__((ext_vector_type(4)));
@@ -56,22 +60,20 @@ __device__ __forceinline__ void dma4(const void* base, uint32_t lane_off, uint32
     asm volatile("s_add_i32 m0, %2, %3\n\tglobal_load_lds_dword %0, %1"
                  : : "v"(lane_off), "s"(base), "s"(lds_base), "n"(kLds) : "memory", "m0", "scc");
 }
-// One d tile of one of the second GEMMs: acc[kt] += a * b[kt] for the four key tiles, accumulators in AGPRs.
+// One d tile of one of the second GEMMs: acc[kt] += a * b[kt] for the wavefront's two key tiles, accumulators in AGPRs.
 // Written as one asm block because the compiler cannot see that these are MFMAs: an MFMA must not read a VGPR in
 // the two issue slots after a VALU instruction wrote it, so the block opens with the wait states itself and
 // contains nothing but MFMAs; only MFMAs touch these accumulators inside the main loop.
-__device__ __forceinline__ void mfma_dtile(floatx4 (&acc)[4], const elem8& a, const elem8 (&b)[4]) {
-    int4v ai, bi[4];
+__device__ __forceinline__ void mfma_dtile(floatx4 (&acc)[kWaveTiles], const elem8& a, const elem8 (&b)[kWaveTiles]) {
+    int4v ai, bi[kWaveTiles];
     __builtin_memcpy(&ai, &a, 16);
 #pragma unroll
-    for (int kt = 0; kt < 4; ++kt) __builtin_memcpy(&bi[kt], &b[kt], 16);
+    for (int kt = 0; kt < kWaveTiles; ++kt) __builtin_memcpy(&bi[kt], &b[kt], 16);
     asm("s_nop 1\n\t"
-        IV2_MFMA_ASM " %0, %4, %5, %0\n\t"
-        IV2_MFMA_ASM " %1, %4, %6, %1\n\t"
-        IV2_MFMA_ASM " %2, %4, %7, %2\n\t"
-        IV2_MFMA_ASM " %3, %4, %8, %3"
-        : "+a"(acc[0]), "+a"(acc[1]), "+a"(acc[2]), "+a"(acc[3])
-        : "v"(ai), "v"(bi[0]), "v"(bi[1]), "v"(bi[2]), "v"(bi[3]));
+        IV2_MFMA_ASM " %0, %2, %3, %0\n\t"
+        IV2_MFMA_ASM " %1, %2, %4, %1"
+        : "+a"(acc[0]), "+a"(acc[1])
+        : "v"(ai), "v"(bi[0]), "v"(bi[1]));
 }
 // 16 lanes x 4 halfwords, transposed: lane (16 g + r) receives element r % 4 of the rows supplied by lanes
 // 16 g + r / 4 + {0, 4, 8, 12}.
@@ -79,11 +81,12 @@ __device__ __forceinline__ short4v lds_read_tr(const unsigned char* ptr) {
     return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v*)(ptr));
 }
 
-template <bool kCausal>
-__global__ __launch_bounds__(64)
+template <bool kCausal, bool kHandoff>
+__global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void bwd_dkdv_wave_kernel(const BwdParams p) {
     extern __shared__ __attribute__((aligned(16))) unsigned char ring[];
-    const int lane = threadIdx.x;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));   // which half of the block's keys
     const int n = lane & 15, g = lane >> 4;
     const int b = blockIdx.y, h = blockIdx.z;
     const int q0 = p.cu_seqlens_q[b];
@@ -164,22 +167,23 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
     __syncthreads();
 
     // ---- K and V of the block: B operands, resident in registers ----
-    elem8 kreg[4][4], vreg[4][4];
+    elem8 kreg[kWaveTiles][4], vreg[kWaveTiles][4];
     {
-        const int64_t img = (static_cast<int64_t>(h) * p.n_slots + image_slot0(p.cu_seqlens_k, b) + j) * kImageElems + lane * 8;
+        const int64_t img = (static_cast<int64_t>(h) * p.n_slots + image_slot0(p.cu_seqlens_k, b) + j) * kImageElems +
+                            wave * (kWaveTiles * 4 * 512) + lane * 8;
 #pragma unroll
-        for (int kt = 0; kt < 4; ++kt)
+        for (int kt = 0; kt < kWaveTiles; ++kt)
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 kreg[kt][c] = *reinterpret_cast<const elem8*>(p.kimg + img + (kt * 4 + c) * 512);
                 vreg[kt][c] = *reinterpret_cast<const elem8*>(p.vimg_r + img + (kt * 4 + c) * 512);
             }
     }
-    floatx4 dKt[8][4], dVt[8][4];                              // [d tile][key tile]: lane (n, g) holds [16 dt + 4 g + e][16 kt + n]
+    floatx4 dKt[8][kWaveTiles], dVt[8][kWaveTiles];            // [d tile][key tile]: lane (n, g) holds [16 dt + 4 g + e][32 wave + 16 kt + n]
 #pragma unroll
     for (int dt = 0; dt < 8; ++dt)
 #pragma unroll
-        for (int kt = 0; kt < 4; ++kt) {
+        for (int kt = 0; kt < kWaveTiles; ++kt) {
             dKt[dt][kt] = floatx4{0.f, 0.f, 0.f, 0.f};
             dVt[dt][kt] = floatx4{0.f, 0.f, 0.f, 0.f};
         }
@@ -211,13 +215,14 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
     // (j + head / 4) % 4: the rotation makes the operand reads below bank-conflict free.
     const int dma_piece = ((lane & 3) + (lane >> 4)) & 3;
     const int dma_head = (lane >> 2) < p.group ? (lane >> 2) : p.group - 1;    // rows beyond the group repeat its last head: their LSE is +inf
-    const uint32_t q_lane = static_cast<uint32_t>((dma_head * p.q_grp + 8 * dma_piece) * 2);   // byte offsets inside one token and KV head
-    const uint32_t do_lane = static_cast<uint32_t>((dma_head * p.do_grp + 8 * dma_piece) * 2);
+    // byte offsets inside one token and KV head; wavefront 0 fetches q, wavefront 1 dout
+    const uint32_t q_lane = static_cast<uint32_t>((dma_head * (wave == 0 ? p.q_grp : p.do_grp) + 8 * dma_piece) * 2);
+    const uint32_t do_lane = q_lane;
     const uint32_t stat_lane = static_cast<uint32_t>((lane & 31) * 4);
     const elem_bits* q_head = p.q + static_cast<int64_t>(h) * p.q_kvh;
     const elem_bits* do_head = p.dout + static_cast<int64_t>(h) * p.do_kvh;
     const float* stat_head = p.rowstat + static_cast<int64_t>(h) * p.total_q * 32;
-    const bool handoff = p.ds_buf != nullptr;                  // uniform over the launch
+    constexpr bool handoff = kHandoff;                         // the launcher picks the variant: p.ds_buf != nullptr
     const uint32_t rank_lane = static_cast<uint32_t>((lane & 3) * 4);
     const uint4* rank_head = handoff ? p.rankinfo + static_cast<int64_t>(h) * p.total_q * p.n64_fwd + (j >> 6) : nullptr;
     const uint64_t below_j = (1ull << (j & 63)) - 1ull;        // the mask bits of the blocks before j in its word
@@ -236,21 +241,23 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
         const unsigned char* qb = q_bytes + ub * q_tok_bytes;
         const unsigned char* da = do_bytes + ua * do_tok_bytes;
         const unsigned char* db = do_bytes + ub * do_tok_bytes;
-        dma16<0, 0>(qa, q_lane, st);        dma16<64, 1024>(qa, q_lane, st);
-        dma16<128, 2048>(qa, q_lane, st);   dma16<192, 3072>(qa, q_lane, st);
-        dma16<0, 4096>(qb, q_lane, st);     dma16<64, 5120>(qb, q_lane, st);
-        dma16<128, 6144>(qb, q_lane, st);   dma16<192, 7168>(qb, q_lane, st);
-        dma16<0, 8192>(da, do_lane, st);    dma16<64, 9216>(da, do_lane, st);
-        dma16<128, 10240>(da, do_lane, st); dma16<192, 11264>(da, do_lane, st);
-        dma16<0, 12288>(db, do_lane, st);   dma16<64, 13312>(db, do_lane, st);
-        dma16<128, 14336>(db, do_lane, st); dma16<192, 15360>(db, do_lane, st);
-        // token a's [lse * log2e (16) | D (16)] (both half-wavefronts fetch the same 128 bytes), then token b's
-        dma4<16384>(stat_bytes + (ua << 7), stat_lane, st);
-        dma4<16384 + 256>(stat_bytes + (ub << 7), stat_lane, st);
-        if (handoff) {
+        // the two wavefronts share the pair's transfers: wavefront 0 fetches q, wavefront 1 dout
+        if (wave == 0) {
+            dma16<0, 0>(qa, q_lane, st);        dma16<64, 1024>(qa, q_lane, st);
+            dma16<128, 2048>(qa, q_lane, st);   dma16<192, 3072>(qa, q_lane, st);
+            dma16<0, 4096>(qb, q_lane, st);     dma16<64, 5120>(qb, q_lane, st);
+            dma16<128, 6144>(qb, q_lane, st);   dma16<192, 7168>(qb, q_lane, st);
+            // token a's [lse * log2e (16) | D (16)] (both half-wavefronts fetch the same 128 bytes)
+            dma4<16384>(stat_bytes + (ua << 7), stat_lane, st);
             // the 16-byte rank record of (token, mask word of block j), replicated over the 256-byte region
-            dma4<16896>(rank_bytes + ua * rank_tok_bytes, rank_lane, st);
-            dma4<16896 + 256>(rank_bytes + ub * rank_tok_bytes, rank_lane, st);
+            if (handoff) dma4<16896>(rank_bytes + ua * rank_tok_bytes, rank_lane, st);
+        } else {
+            dma16<0, 8192>(da, do_lane, st);    dma16<64, 9216>(da, do_lane, st);
+            dma16<128, 10240>(da, do_lane, st); dma16<192, 11264>(da, do_lane, st);
+            dma16<0, 12288>(db, do_lane, st);   dma16<64, 13312>(db, do_lane, st);
+            dma16<128, 14336>(db, do_lane, st); dma16<192, 15360>(db, do_lane, st);
+            dma4<16384 + 256>(stat_bytes + (ub << 7), stat_lane, st);
+            if (handoff) dma4<16896 + 256>(rank_bytes + ub * rank_tok_bytes, rank_lane, st);
         }
     };
 
@@ -259,7 +266,7 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
     // meant to stay in flight.
     __builtin_amdgcn_s_waitcnt(0x0F70);                        // vmcnt(0)
 #pragma unroll
-    for (int kt = 0; kt < 4; ++kt)
+    for (int kt = 0; kt < kWaveTiles; ++kt)
 #pragma unroll
         for (int c = 0; c < 4; ++c) asm volatile("" : "+v"(kreg[kt][c]), "+v"(vreg[kt][c]));
 
@@ -277,22 +284,15 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
     bool more = next_pair(ta, tb, has_b);
     if (more) issue(ta, tb, 0);
     int stage = 0;
-    bool first_turn = true;
     while (more) {
+        // This wavefront's half of the pair's transfers has landed (nothing younger is in flight: the next pair goes out
+        // below); the barrier adds the other wavefront's half and says that both are done with the other stage.
+        __builtin_amdgcn_s_waitcnt(0x0F70);                    // vmcnt(0)
+        __syncthreads();
         int64_t na, nb2;
         bool nhb;
         const bool have_next = next_pair(na, nb2, nhb);
-        if (have_next) {
-            issue(na, nb2, stage ^ 1);                         // the other stage was consumed by the previous turn
-            // this turn's loads have landed when only the younger operations are still in flight: the next pair's 18
-            // loads, or with the hand-off its 20 loads and the previous turn's 8 tile stores
-            if (!handoff) __builtin_amdgcn_s_waitcnt(0x4F72);                  // vmcnt(18)
-            else if (first_turn) __builtin_amdgcn_s_waitcnt(0x4F74);           // vmcnt(20)
-            else __builtin_amdgcn_s_waitcnt(0x4F7C);                           // vmcnt(28)
-        } else {
-            __builtin_amdgcn_s_waitcnt(0x0F70);
-        }
-        first_turn = false;
+        if (have_next) issue(na, nb2, stage ^ 1);
         const unsigned char* st = ring + stage * kStage;
 
         int lim_a, lim_b;                                      // in-block key index limit (inclusive)
@@ -309,12 +309,6 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
         }
 
         const float* scal = reinterpret_cast<const float*>(st + 16384);
-        const float4 la = *reinterpret_cast<const float4*>(scal + 4 * g);
-        const float4 Da = *reinterpret_cast<const float4*>(scal + 16 + 4 * g);
-        const float4 lb = *reinterpret_cast<const float4*>(scal + 64 + 4 * g);
-        const float4 Db = *reinterpret_cast<const float4*>(scal + 80 + 4 * g);
-        const float lse_a[4] = {la.x, la.y, la.z, la.w};
-        const float lse_b[4] = {lb.x, lb.y, lb.z, lb.w};
         const bool edge = (lim_a < kBlockN - 1) || (lim_b < kBlockN - 1);
         // hand-off: where the dS^T tiles of this pair go (rank of block j among the set bits of each token's mask row)
         elem_bits* ds_a = nullptr;
@@ -336,63 +330,71 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
             ds_b = p.ds_buf + ((static_cast<int64_t>(h) * p.total_q + tb) * row_tiles + rank_b) * (kBlockN * 16);
         }
 
-        // Four phases, each 32 MFMAs, with the VALU work of the softmax backward hidden behind the matrix pipeline:
-        //   A  S = Q K^T                       (both tokens, all 64 keys; every fragment read from LDS feeds 4 MFMAs)
-        //   B  dP = dO V^T                     while the VALU turns S into P = exp2(scale S - LSE) (fp32 and bf16)
+        // Per wavefront 64 MFMAs in four GEMM phases with the softmax backward between them; the other wavefront of the
+        // SIMD fills the matrix pipeline while this one does vector work:
+        //   A  S = Q K^T                       (both tokens, this wavefront's 32 keys; a fragment read from LDS feeds 2 MFMAs)
+        //      P = exp2(scale S - LSE)         (fp32 in place of S, and bf16)
+        //   B  dP = dO V^T                     (accumulators start at -D)
         //   C  dV^T += dO^T P                  while the VALU forms dS = P (dP - D) (bf16)
         //   D  dK^T += Q^T dS
         const uint4* frag = reinterpret_cast<const uint4*>(st) + frag_unit;      // tile t, chunk c at frag[t * 256 + c * 64]
-        elem8 pfr[4], dsfr[4];                                // per key tile: [token a heads 4g..4g+3 | token b heads 4g..4g+3]
-        floatx4 sa[4], sb[4], dpa[4], dpb[4];
-        // the dP accumulators start at -D, so that dS = P (dP - D) is one multiplication per element
-        const floatx4 negD_a = {-Da.x, -Da.y, -Da.z, -Da.w}, negD_b = {-Db.x, -Db.y, -Db.z, -Db.w};
+        elem8 pfr[kWaveTiles], dsfr[kWaveTiles];              // per key tile: [token a heads 4g..4g+3 | token b heads 4g..4g+3]
+        floatx4 sa[kWaveTiles], sb[kWaveTiles], dpa[kWaveTiles], dpb[kWaveTiles];
 #pragma unroll
-        for (int kt = 0; kt < 4; ++kt) {
+        for (int kt = 0; kt < kWaveTiles; ++kt) {
             sa[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
-            sb[kt] = sa[kt]; dpa[kt] = negD_a; dpb[kt] = negD_b;
+            sb[kt] = sa[kt];
         }
         {   // A
-            uint4 fr[2][2];
-            fr[0][0] = frag[0]; fr[0][1] = frag[256];
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
-                if (c < 3) { fr[(c + 1) & 1][0] = frag[(c + 1) * 64]; fr[(c + 1) & 1][1] = frag[256 + (c + 1) * 64]; }
+                const uint4 fa = frag[c * 64], fb = frag[256 + c * 64];
                 elem8 qa, qb;
-                __builtin_memcpy(&qa, &fr[c & 1][0], 16);
-                __builtin_memcpy(&qb, &fr[c & 1][1], 16);
+                __builtin_memcpy(&qa, &fa, 16);
+                __builtin_memcpy(&qb, &fb, 16);
 #pragma unroll
-                for (int kt = 0; kt < 4; ++kt) {
+                for (int kt = 0; kt < kWaveTiles; ++kt) {
                     sa[kt] = IV2_MFMA(qa, kreg[kt][c], sa[kt], 0, 0, 0);
                     sb[kt] = IV2_MFMA(qb, kreg[kt][c], sb[kt], 0, 0, 0);
                 }
             }
         }
         __builtin_amdgcn_sched_barrier(0);
+        {   // P, kept in fp32 in place of S
+            const float4 la = *reinterpret_cast<const float4*>(scal + 4 * g);
+            const float4 lb = *reinterpret_cast<const float4*>(scal + 64 + 4 * g);
+            const float lse_a[4] = {la.x, la.y, la.z, la.w};
+            const float lse_b[4] = {lb.x, lb.y, lb.z, lb.w};
+#pragma unroll
+            for (int kt = 0; kt < kWaveTiles; ++kt)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float xa = __builtin_amdgcn_exp2f(sa[kt][e] * p.scale_log2 - lse_a[e]);
+                    float xb = __builtin_amdgcn_exp2f(sb[kt][e] * p.scale_log2 - lse_b[e]);
+                    sa[kt][e] = xa;
+                    sb[kt][e] = xb;
+                    pfr[kt][e] = static_cast<elem_t>(xa);
+                    pfr[kt][4 + e] = static_cast<elem_t>(xb);
+                }
+        }
+        __builtin_amdgcn_sched_barrier(0);
         {   // B
-            uint4 fr[2][2];
-            fr[0][0] = frag[512]; fr[0][1] = frag[768];
+            const float4 Da = *reinterpret_cast<const float4*>(scal + 16 + 4 * g);
+            const float4 Db = *reinterpret_cast<const float4*>(scal + 80 + 4 * g);
+            // the dP accumulators start at -D, so that dS = P (dP - D) is one multiplication per element
+            const floatx4 negD_a = {-Da.x, -Da.y, -Da.z, -Da.w}, negD_b = {-Db.x, -Db.y, -Db.z, -Db.w};
+#pragma unroll
+            for (int kt = 0; kt < kWaveTiles; ++kt) { dpa[kt] = negD_a; dpb[kt] = negD_b; }
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
-                if (c < 3) { fr[(c + 1) & 1][0] = frag[512 + (c + 1) * 64]; fr[(c + 1) & 1][1] = frag[768 + (c + 1) * 64]; }
+                const uint4 fa = frag[512 + c * 64], fb = frag[768 + c * 64];
                 elem8 doa, dob;
-                __builtin_memcpy(&doa, &fr[c & 1][0], 16);
-                __builtin_memcpy(&dob, &fr[c & 1][1], 16);
+                __builtin_memcpy(&doa, &fa, 16);
+                __builtin_memcpy(&dob, &fb, 16);
 #pragma unroll
-                for (int kt = 0; kt < 4; ++kt) {
+                for (int kt = 0; kt < kWaveTiles; ++kt) {
                     dpa[kt] = IV2_MFMA(doa, vreg[kt][c], dpa[kt], 0, 0, 0);
                     dpb[kt] = IV2_MFMA(dob, vreg[kt][c], dpb[kt], 0, 0, 0);
-                }
-                {   // P of key tile c, kept in fp32 in place of S
-                    const int kt = c;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        float xa = __builtin_amdgcn_exp2f(sa[kt][e] * p.scale_log2 - lse_a[e]);
-                        float xb = __builtin_amdgcn_exp2f(sb[kt][e] * p.scale_log2 - lse_b[e]);
-                        sa[kt][e] = xa;
-                        sb[kt][e] = xb;
-                        pfr[kt][e] = static_cast<elem_t>(xa);
-                        pfr[kt][4 + e] = static_cast<elem_t>(xb);
-                    }
                 }
             }
         }
@@ -400,8 +402,9 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
         if (edge) {
             // a block cut by the causal diagonal or by the sequence end (rare): keys beyond the limit get P = 0
 #pragma unroll
-            for (int kt = 0; kt < 4; ++kt) {
-                const bool off_a = n > lim_a - 16 * kt, off_b = n > lim_b - 16 * kt;
+            for (int kt = 0; kt < kWaveTiles; ++kt) {
+                const int key0 = 16 * (kWaveTiles * wave + kt);
+                const bool off_a = n > lim_a - key0, off_b = n > lim_b - key0;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     sa[kt][e] = off_a ? 0.f : sa[kt][e];
@@ -425,24 +428,21 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
                 __builtin_memcpy(&ad, &t_a[dt & 1], 8);
                 __builtin_memcpy(reinterpret_cast<unsigned char*>(&ad) + 8, &t_b[dt & 1], 8);
                 mfma_dtile(dVt[dt], ad, pfr);
-                {   // dS of half a key tile
-                    const int kt = dt >> 1, e0 = (dt & 1) * 2;
-#pragma unroll
-                    for (int e = e0; e < e0 + 2; ++e) {
-                        dsfr[kt][e] = static_cast<elem_t>(sa[kt][e] * dpa[kt][e]);
-                        dsfr[kt][4 + e] = static_cast<elem_t>(sb[kt][e] * dpb[kt][e]);
-                    }
+                {   // dS of a quarter key tile
+                    const int kt = dt >> 2, e = dt & 3;
+                    dsfr[kt][e] = static_cast<elem_t>(sa[kt][e] * dpa[kt][e]);
+                    dsfr[kt][4 + e] = static_cast<elem_t>(sb[kt][e] * dpb[kt][e]);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
         if (handoff) {
-            // dS^T tiles [key][head]: lane (key n of tile kt, heads 4g..4g+3) holds 8 bytes per token; always 8 stores
+            // dS^T tiles [key][head]: lane (key n of tile kt, heads 4g..4g+3) holds 8 bytes per token; always 4 stores
 #pragma unroll
-            for (int kt = 0; kt < 4; ++kt) {
+            for (int kt = 0; kt < kWaveTiles; ++kt) {
                 uint4 raw;
                 __builtin_memcpy(&raw, &dsfr[kt], 16);
-                const int at = kt * 256 + n * 16 + 4 * g;         // the tile bases are wave-uniform: scalar base + lane offset
+                const int at = (kWaveTiles * wave + kt) * 256 + n * 16 + 4 * g;    // the tile bases are wave-uniform: scalar base + lane offset
                 // streaming stores: the tiles are read much later, by another kernel, and should not push q / dout out of L2
                 typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
                 __builtin_nontemporal_store(u32x2{raw.x, raw.y}, reinterpret_cast<u32x2*>(ds_a + at));
@@ -474,15 +474,17 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
     float* tile = reinterpret_cast<float*>(ring);
     const int valid_keys = (Sk - j * kBlockN) < kBlockN ? (Sk - j * kBlockN) : kBlockN;
     const int64_t row0 = static_cast<int64_t>(k0) + static_cast<int64_t>(j) * kBlockN;
+    const int key_lo = 16 * kWaveTiles * wave;                 // this wavefront's rows of the tile
+    const int key_hi = key_lo + 16 * kWaveTiles < valid_keys ? key_lo + 16 * kWaveTiles : valid_keys;
 #pragma unroll
     for (int which = 0; which < 2; ++which) {
         __syncthreads();
 #pragma unroll
         for (int dt = 0; dt < 8; ++dt)
 #pragma unroll
-            for (int kt = 0; kt < 4; ++kt) {
+            for (int kt = 0; kt < kWaveTiles; ++kt) {
                 const floatx4 v = which == 0 ? dKt[dt][kt] : dVt[dt][kt];
-                *reinterpret_cast<float4*>(tile + (16 * kt + n) * kFlushPitch + 16 * dt + 4 * g) = make_float4(v[0], v[1], v[2], v[3]);
+                *reinterpret_cast<float4*>(tile + (key_lo + 16 * kt + n) * kFlushPitch + 16 * dt + 4 * g) = make_float4(v[0], v[1], v[2], v[3]);
             }
         __syncthreads();
         const float mul = which == 0 ? p.scale : 1.f;
@@ -491,15 +493,15 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
             // end hold zeros), to be added in slice order by bwd_dkdv_reduce_kernel
             const int64_t item = (static_cast<int64_t>(h) * p.n_slots + image_slot0(p.cu_seqlens_k, b) + j) * p.det_slices + slice;
             float* dst = p.det_slots + (item * 2 + which) * (kBlockN * kHeadDim) + lane;
-            for (int key = 0; key < kBlockN; ++key) {
+            for (int key = key_lo; key < key_lo + 16 * kWaveTiles; ++key) {
                 dst[key * kHeadDim] = tile[key * kFlushPitch + lane] * mul;
                 dst[key * kHeadDim + 64] = tile[key * kFlushPitch + 64 + lane] * mul;
             }
-            if (which == 1 && lane == 0) p.det_flags[item] = 1u;
+            if (which == 1 && lane == 0 && wave == 0) p.det_flags[item] = 1u;
             continue;
         }
         float* acc = (which == 0 ? p.dk_acc : p.dv_acc) + (row0 * p.num_heads_k + h) * kHeadDim + lane;
-        for (int key = 0; key < valid_keys; ++key) {
+        for (int key = key_lo; key < key_hi; ++key) {
             float* dst = acc + static_cast<int64_t>(key) * p.num_heads_k * kHeadDim;
             unsafeAtomicAdd(dst, tile[key * kFlushPitch + lane] * mul);
             unsafeAtomicAdd(dst + 64, tile[key * kFlushPitch + 64 + lane] * mul);
@@ -560,8 +562,11 @@ int launch_bwd_dkdv_wave(hipStream_t st, const BwdParams& p, int batch, int max_
               "varlen_bwd: token strides of q and dout must lie in [0, 2^31) elements");
     const dim3 grid(static_cast<unsigned>(items), batch, p.num_heads_k);
     const size_t lds = kWaveLds + kGroupWords * 8;
-    if (causal) hipLaunchKernelGGL(bwd_dkdv_wave_kernel<true>, grid, dim3(64), lds, st, p);
-    else hipLaunchKernelGGL(bwd_dkdv_wave_kernel<false>, grid, dim3(64), lds, st, p);
+    const bool handoff = p.ds_buf != nullptr;
+    if (causal && handoff) hipLaunchKernelGGL((bwd_dkdv_wave_kernel<true, true>), grid, dim3(128), lds, st, p);
+    else if (causal) hipLaunchKernelGGL((bwd_dkdv_wave_kernel<true, false>), grid, dim3(128), lds, st, p);
+    else if (handoff) hipLaunchKernelGGL((bwd_dkdv_wave_kernel<false, true>), grid, dim3(128), lds, st, p);
+    else hipLaunchKernelGGL((bwd_dkdv_wave_kernel<false, false>), grid, dim3(128), lds, st, p);
     IV2_LAUNCH_CHECK();
     return 0;
 }
