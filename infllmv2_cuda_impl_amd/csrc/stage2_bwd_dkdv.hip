@@ -32,8 +32,9 @@
 namespace IV2_NS {
 
 constexpr int kColSlice = kDkdvSlice;                          // query tokens per work item
-constexpr int kGroupSlices = 4;                                // slices that pool their light members
-constexpr int kGroupWords = kGroupSlices * kColSlice / 64;     // = 32: one mask word per lane of the lower half
+constexpr int kSliceWords = kColSlice / 64;                    // mask words per slice (a power of two)
+constexpr int kGroupWords = 32;                                // one mask word per lane of the lower half-wavefront: 2048 tokens
+constexpr int kGroupSlices = kGroupWords / kSliceWords;        // slices that pool their light members
 constexpr int kHeavyPairs = 128;                               // a slice with fewer selected tokens is "light"
 constexpr int kStage = 16384 + 512 + 512;                      // q a|b, dout a|b (4 KiB each), the pair's 64 row scalars, its two rank records
 constexpr int kWaveLds = 2 * kStage;                           // = 64 rows x 132 floats: also the flush tile
@@ -96,17 +97,21 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
     const int nb = (Sk + kBlockN - 1) / kBlockN;               // key blocks of this sequence
 
     // ---- which (512-token slice, block) ----
-    // Slices are cut on the packed token axis (so they are whole mask words) and clipped to the sequence.
-    // Workgroup ids go round-robin over the 8 XCDs: each XCD takes one slice at a time (latest first), so the
-    // wavefronts sharing an L2 stream the same tokens of q and dout; within a slice the shared first block
-    // comes first, then the diagonal block and outwards, so the long items are dispatched early.
+    // Slices are cut on the packed token axis (so they are whole mask words) and clipped to the sequence; four
+    // consecutive slices form a group.  Workgroup ids go round-robin over the 8 XCDs, and XCD x takes the groups
+    // whose index on the packed axis is x modulo 8, latest first, one slice at a time: the wavefronts sharing an L2
+    // stream the same tokens of q and dout, and because the assignment follows the packed axis (not each
+    // sequence's own first group) the groups of a batch of sequences spread evenly over the XCDs.  Within a slice
+    // the shared first block comes first, then the diagonal block and outwards, so the long items are dispatched early.
     const int xcd = blockIdx.x & 7, turn = blockIdx.x >> 3;
     const int rel = turn % p.k_blocks;
     if (Sq <= 0 || rel >= nb) return;                          // uniform
     const int last_slice = (q0 + Sq - 1) / kColSlice;
-    const int top_slice = last_slice | (kGroupSlices - 1);     // last slice of the last group
+    const int top_group = last_slice / kGroupSlices;
     const int round = turn / p.k_blocks;                       // an XCD works through one group of slices in consecutive rounds
-    const int slice = top_slice - (((round / kGroupSlices) * 8 + xcd) * kGroupSlices + round % kGroupSlices);
+    const int grp_idx = top_group - ((top_group - xcd) & 7) - 8 * (round / kGroupSlices);
+    if (grp_idx < 0) return;                                   // uniform
+    const int slice = grp_idx * kGroupSlices + (kGroupSlices - 1 - round % kGroupSlices);
     if (slice > last_slice || slice < q0 / kColSlice) return;  // uniform
     int j;
     if (rel == 0) {
@@ -132,7 +137,7 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
     // A flush costs 32768 fp32 atomics whatever the slice held, so a slice works on its own only if at least
     // kHeavyPairs of its tokens selected the block; the other slices of the same group of 4 hand their tokens
     // to the first non-empty one among them.  Every workgroup of the group takes the same decision from the
-    // group's 32 mask words (lane l < 32 holds word l; a slice is 8 words = 8 lanes).
+    // group's 32 mask words (lane l < 32 holds word l; a slice is kSliceWords consecutive lanes).
     unsigned long long* wbuf = reinterpret_cast<unsigned long long*>(ring + kWaveLds);      // [kGroupWords]
     const int group = slice / kGroupSlices, sub = slice % kGroupSlices;
     const int64_t w0 = static_cast<int64_t>(group) * kGroupWords;
@@ -149,17 +154,16 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
             }
         }
         int cnt = __builtin_popcountll(wv);
-        cnt += __shfl_xor(cnt, 1);
-        cnt += __shfl_xor(cnt, 2);
-        cnt += __shfl_xor(cnt, 4);                             // tokens of this lane's slice that selected the block
-        const uint64_t heavy = __ballot(cnt >= kHeavyPairs);   // 8 equal bits per slice
+#pragma unroll
+        for (int off = 1; off < kSliceWords; off <<= 1) cnt += __shfl_xor(cnt, off);   // tokens of this lane's slice that selected the block
+        const uint64_t heavy = __ballot(cnt >= kHeavyPairs);   // kSliceWords equal bits per slice
         const uint64_t filled = __ballot(cnt > 0);
         bool keep;
-        if ((heavy >> (8 * sub)) & 1ull) {
-            keep = (lane >> 3) == sub;
+        if ((heavy >> (kSliceWords * sub)) & 1ull) {
+            keep = (lane / kSliceWords) == sub;
         } else {
             const uint64_t light = filled & ~heavy;
-            if (light == 0ull || (__builtin_ctzll(light) >> 3) != sub) return;   // uniform: empty, or another slice collects
+            if (light == 0ull || (__builtin_ctzll(light) / kSliceWords) != sub) return;   // uniform: empty, or another slice collects
             keep = !((heavy >> lane) & 1ull);
         }
         if (lane < kGroupWords) wbuf[lane] = keep ? wv : 0ull;
@@ -554,8 +558,11 @@ int launch_bwd_dkdv_reduce(hipStream_t st, const BwdParams& p, int batch) {
 }
 
 int launch_bwd_dkdv_wave(hipStream_t st, const BwdParams& p, int batch, int max_seqlen_q, bool causal) {
-    const int n_slices = (max_seqlen_q + kColSlice - 1) / kColSlice + 1 + kGroupSlices;   // sequences need not start or end on group boundaries
-    const int n_slices8 = (n_slices + 8 * kGroupSlices - 1) / (8 * kGroupSlices) * (8 * kGroupSlices);
+    // a sequence of max_seqlen_q tokens touches at most `groups` consecutive slice groups wherever it starts, and an
+    // XCD takes every 8th of them: ceil(groups / 8) rounds of kGroupSlices slices each
+    const int group_tokens = kGroupSlices * kColSlice;
+    const int groups = (max_seqlen_q + group_tokens - 1) / group_tokens + 1;
+    const int n_slices8 = (groups + 7) / 8 * (8 * kGroupSlices);
     const int64_t items = static_cast<int64_t>(n_slices8) * p.k_blocks;
     IV2_CHECK(items <= 0x7fffffffll, "varlen_bwd: too many (slice, block) work items");
     IV2_CHECK(p.q_tok >= 0 && p.q_tok < (1ll << 31) && p.do_tok >= 0 && p.do_tok < (1ll << 31) && p.total_q < (1ll << 31),
