@@ -248,6 +248,23 @@ def decode_bench(torch, ops, dev):
         _, m = ops.topk_blocks(p, topk, return_mask=True, by_index=True)
         return ops.infllmv2_attn_with_kvcache(q, kc, vc, cache_seqlens=L, block_mask=m.unsqueeze(2))
     step_ms = event_ms(torch, step, 20)
+
+    # the same step with the two compressed-key appends in front, once launched call by call and once as one captured
+    # HIP graph (a serving loop replays the graph: the gaps between the step's ten small launches disappear)
+    def full_step():
+        ops.compress_keys_cache(kc, L, 32, 16, out=fine, old_lens=pos, max_new_rows=1)
+        ops.compress_keys_cache(kc, L, 128, 64, out=coarse, old_lens=pos, max_new_rows=1)
+        return step()
+    full_ms = event_ms(torch, full_step, 20)
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream(device=dev)
+    side.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            captured = full_step()
+    torch.cuda.synchronize()
+    graph_ms = event_ms(torch, graph.replay, 20)
+    graph_ok = bool(torch.equal(captured, full_step()))
     s1_bytes = 2 * 128 * 2 * (int(fl.sum()) + int(cl.sum()))           # Hk * (Lk_b + Lc_b) * d * 2 bytes over the batch
     s2_bytes = B * 2 * 64 * 64 * 128 * 2 * 2 + 2 * B * 32 * 128 * 2
     gbs = lambda b, ms: b / ms / 1e6
@@ -260,6 +277,8 @@ def decode_bench(torch, ops, dev):
             "stage1_ms": s1_ms, "stage1_algorithmic_bytes": s1_bytes, "stage1_hbm_gbs": gbs(s1_bytes, s1_ms),
             "stage1_frac_hbm_peak": gbs(s1_bytes, s1_ms) / PEAK_HBM_GBS,
             "topk_ms": topk_ms, "compressed_key_append_ms": append_ms, "step_ms": step_ms,
+            "step_with_append_ms": full_ms, "step_with_append_graph_ms": graph_ms, "graph_equals_eager": graph_ok,
+            "step_graph_frac_hbm_peak": gbs(s1_bytes + s2_bytes, graph_ms) / PEAK_HBM_GBS,
             "step_hbm_gbs": gbs(s1_bytes + s2_bytes, step_ms),
             "step_frac_hbm_peak": gbs(s1_bytes + s2_bytes, step_ms) / PEAK_HBM_GBS}
 

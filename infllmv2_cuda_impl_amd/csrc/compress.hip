@@ -127,6 +127,47 @@ void compress_keys_cache_kernel(const CompressCacheParams p) {
     }
 }
 
+// The append of a decode step: few new rows per sequence, so one workgroup takes ONE output row (32 of its 16-byte
+// units).  Walking the window row by row in one thread, as the kernel above does, is a chain of kernel_size dependent
+// round trips to memory when only a handful of threads are busy; here the whole window goes into LDS with every
+// load in flight at once, and then one thread per output element adds its column in window order (the same fp32
+// additions in the same order as above: the results are the same bits).
+constexpr int kAppendUnits = 32;
+constexpr int kAppendMaxLds = 65536;
+
+__global__ __launch_bounds__(256)
+void compress_keys_cache_append_kernel(const CompressCacheParams p) {
+    extern __shared__ uint4 window[];                          // [kernel_size][kAppendUnits]
+    const int b = blockIdx.y;
+    const int rows = compressed_rows(p.new_lens[b], p.kernel_size, p.stride);
+    const int first = p.old_lens ? compressed_rows(p.old_lens[b], p.kernel_size, p.stride) : 0;
+    if (blockIdx.x == 0 && blockIdx.z == 0 && threadIdx.x == 0 && p.out_lens) p.out_lens[b] = rows;
+    const int j = first + blockIdx.x;
+    if (j >= rows) return;                                     // uniform per workgroup
+    const int u0 = blockIdx.z * kAppendUnits;
+    const int nu = p.units_per_row - u0 < kAppendUnits ? p.units_per_row - u0 : kAppendUnits;
+    const elem_bits* src = p.k + b * p.k_batch + static_cast<int64_t>(j) * p.stride * p.k_row;
+    const int items = p.kernel_size * kAppendUnits;
+#pragma unroll 8
+    for (int it = threadIdx.x; it < items; it += 256) {
+        const int i = it / kAppendUnits, uu = it % kAppendUnits;
+        if (uu < nu) {
+            const int u = u0 + uu;
+            window[it] = *reinterpret_cast<const uint4*>(src + i * p.k_row + (u / p.units_per_head) * p.k_head + (u % p.units_per_head) * 8);
+        }
+    }
+    __syncthreads();
+    const int uu = threadIdx.x >> 3, e = threadIdx.x & 7;      // one thread per (unit, element)
+    if (uu >= nu) return;
+    const elem_bits* col = reinterpret_cast<const elem_bits*>(window) + uu * 8 + e;
+    float acc = 0.f;
+    for (int i = 0; i < p.kernel_size; ++i) acc += elem_to_f32(col[i * kAppendUnits * 8]);
+    const float n = static_cast<float>(p.kernel_size);
+    const int u = u0 + uu;
+    p.out[b * p.o_batch + static_cast<int64_t>(j) * p.o_row + (u / p.units_per_head) * p.o_head + (u % p.units_per_head) * 8 + e] =
+        f32_to_elem(acc / n);
+}
+
 }  // namespace IV2_NS
 
 using namespace IV2_NS;
@@ -181,6 +222,14 @@ extern "C" int IV2_ENTRY(infllmv2_compress_keys_cache)(void* stream, const void*
     p.o_batch = out_strides[0]; p.o_row = out_strides[1]; p.o_head = out_strides[2];
     p.units_per_row = num_heads_k * head_dim / 8; p.units_per_head = head_dim / 8;
     p.kernel_size = kernel_size; p.stride = stride;
+    const size_t window_bytes = static_cast<size_t>(kernel_size) * kAppendUnits * 16;
+    if (max_new_rows >= 1 && max_new_rows <= 8 && window_bytes <= kAppendMaxLds) {
+        // a decode step's append: one workgroup per new row and 32 units
+        const dim3 grid(max_new_rows, batch, (p.units_per_row + kAppendUnits - 1) / kAppendUnits);
+        hipLaunchKernelGGL(compress_keys_cache_append_kernel, grid, dim3(256), window_bytes, static_cast<hipStream_t>(stream), p);
+        IV2_LAUNCH_CHECK();
+        return 0;
+    }
     // at least one workgroup per sequence so that out_lens is always written
     const int groups = max_new_rows > 0 ? (max_new_rows + kCompressRowsPerWg - 1) / kCompressRowsPerWg : 1;
     hipLaunchKernelGGL(compress_keys_cache_kernel, dim3(groups, batch), dim3(256), 0, static_cast<hipStream_t>(stream), p);
