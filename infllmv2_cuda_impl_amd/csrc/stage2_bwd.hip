@@ -11,9 +11,9 @@
 //   * dQ: its own row-parallel kernel with the forward's schedule (stage2_bwd_dq.hip); S and dP
 //     are recomputed, dQ stays in registers and is written once as bf16.  No dq scratch, no zero
 //     fill, no conversion pass, bit-reproducible.
-//   * dK/dV: column-parallel (stage2_bwd_dkdv.hip).  One wavefront owns a 64-key block and a
-//     slice of 512 query tokens, walks the transposed mask, keeps the 64x128 dK^T and dV^T tiles
-//     in accumulation registers and flushes once per slice with fp32 atomics.
+//   * dK/dV: column-parallel (stage2_bwd_dkdv.hip).  Two wavefronts own a 64-key block (32 keys each) and a
+//     slice of 512 query tokens, walk the transposed mask, keep their 32x128 dK^T and dV^T tiles
+//     in accumulation registers and flush once per slice with fp32 atomics.
 // This file holds the preprocessing kernel, the fp32 -> bf16 conversion of dK/dV and the C entry
 // point.
 #include "common.h"
