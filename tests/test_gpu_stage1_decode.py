@@ -147,6 +147,30 @@ def test_compressed_key_caches_follow_the_key_caches(ops):
                 assert bool((out[b, r:] == 7.0).all())
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("Hk,d,ks,st,jump", [(8, 128, 32, 16, 40), (3, 64, 24, 8, 20), (2, 128, 128, 64, 200), (5, 128, 160, 32, 7)])
+def test_append_of_a_few_rows_equals_the_full_build(ops, dtype, Hk, d, ks, st, jump):
+    """The append path (at most 8 new rows per sequence, window staged in LDS; several workgroups per row when a row
+    has more than 32 sixteen-byte units) and the general path (windows too large for it, or many new rows) write the
+    same bits as a build from scratch, and nothing else."""
+    lens = [0, 5, ks - 1, ks, 3 * ks + 1, 500]
+    B, cap = len(lens), 800
+    g = torch.Generator(device="cpu").manual_seed(17)
+    kcache = torch.randn(B, cap, Hk, d, generator=g).to(dtype).to(DEV)
+    old = torch.tensor(lens, dtype=torch.int32, device=DEV)
+    new = old + jump
+    rows_max = (cap - ks) // st + 1
+    full = torch.full((B, rows_max, Hk, d), 7.0, dtype=dtype, device=DEV)
+    rows_full = ops.compress_keys_cache(kcache, new, ks, st, out=full)
+    inc = torch.full((B, rows_max, Hk, d), 7.0, dtype=dtype, device=DEV)
+    ops.compress_keys_cache(kcache, old, ks, st, out=inc)
+    max_new = max(O.compressed_len(n + jump, ks, st) - O.compressed_len(n, ks, st) for n in lens)
+    rows_inc = ops.compress_keys_cache(kcache, new, ks, st, out=inc, old_lens=old, max_new_rows=max_new)
+    assert torch.equal(rows_inc, rows_full)
+    assert [int(r) for r in rows_full] == [O.compressed_len(n + jump, ks, st) for n in lens]
+    assert torch.equal(inc, full)
+
+
 def test_batched_decode_steps_equal_single_sequence_decode(ops):
     """decode_batch on sequences of different lengths == the single-sequence decode loop run on each of them: same
     caches afterwards (bit for bit), outputs to the Stage-2 tolerance (the two paths cut the compressed keys into
