@@ -23,7 +23,7 @@ namespace IV2_NS {
 constexpr int kDqTokens = 8;
 constexpr int kDqChunk = 16;                                   // token groups per XCD chunk
 constexpr int kDqTileBytes = 32768;
-constexpr int kDqMaskWords = 256;                              // LDS copies of the mask rows: up to 16384 key blocks
+constexpr int kDqMaskWords = 256;                              // LDS copies of the mask rows hold at most this many words each: 16384 key blocks
 constexpr int kDqLdsTiles = 2 * kDqTileBytes + 8 * 8192;       // 2-tile ring + 8 private half K tiles
 
 typedef short short4q __attribute__((ext_vector_type(4)));
@@ -32,6 +32,7 @@ struct DqExtra {
     int groups_per_seq;
     int batch;
     int total_groups;
+    int mask_words;                                            // words per LDS mask row: what the longest key sequence needs
 };
 
 __device__ __forceinline__ uint32_t lds_address_dq(const void* ptr) {
@@ -85,8 +86,8 @@ __global__ __launch_bounds__(512)
 void bwd_dq_hybrid_kernel(const BwdParams p, const DqExtra x) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     uint4* ring = reinterpret_cast<uint4*>(smem_raw);                               // [2][2048]: K units 0..1023, V (K-image order) 1024..2047
-    unsigned long long* com = reinterpret_cast<unsigned long long*>(smem_raw + kDqLdsTiles);       // [kDqMaskWords]
-    unsigned long long* rows = com + kDqMaskWords;                                                  // [kDqTokens][kDqMaskWords]
+    unsigned long long* com = reinterpret_cast<unsigned long long*>(smem_raw + kDqLdsTiles);       // [mask_words]
+    unsigned long long* rows = com + x.mask_words;                                                  // [kDqTokens][mask_words]
 
     const int bid = blockIdx.x;
     const int xcd = bid & 7, sidx = bid >> 3;
@@ -123,9 +124,10 @@ void bwd_dq_hybrid_kernel(const BwdParams p, const DqExtra x) {
         int lk = kCausal ? (i_last + Sk - Sq) : (Sk - 1);
         if (lk > Sk - 1) lk = Sk - 1;
         nw = lk < 0 ? 0 : (lk >> 12) + 1;
-        if (mrow && nw > p.n64_fwd) nw = p.n64_fwd;                                  // nw <= kDqMaskWords: checked by the launcher
+        if (mrow && nw > p.n64_fwd) nw = p.n64_fwd;
+        if (nw > x.mask_words) nw = x.mask_words;                                    // a sequence longer than the announced max_seqlen_k
     }
-    unsigned long long* own = rows + wave * kDqMaskWords;
+    unsigned long long* own = rows + wave * x.mask_words;
     for (int w = tid; w < nw; w += 512) com[w] = ~0ull;
     __syncthreads();
     for (int w = lane; w < nw; w += 64) {
@@ -358,9 +360,10 @@ int launch_bwd_dq_hybrid(hipStream_t st, const BwdParams& p, int batch, int max_
     IV2_CHECK(total <= 0x3fffffff, "varlen_bwd: too many token groups");
     IV2_CHECK(p.k_blocks <= kDqMaskWords * 64, "varlen_bwd: more than %d key blocks per sequence", kDqMaskWords * 64);
     x.total_groups = static_cast<int>(total);
+    x.mask_words = (p.k_blocks + 63) / 64 > 0 ? (p.k_blocks + 63) / 64 : 1;
     const int64_t per_round = 8 * kDqChunk;
     const int64_t grid = (total + per_round - 1) / per_round * per_round;
-    const size_t lds = kDqLdsTiles + (1 + kDqTokens) * kDqMaskWords * 8;
+    const size_t lds = kDqLdsTiles + static_cast<size_t>(1 + kDqTokens) * x.mask_words * 8;
     const void* fn = causal ? reinterpret_cast<const void*>(&bwd_dq_hybrid_kernel<true>)
                             : reinterpret_cast<const void*>(&bwd_dq_hybrid_kernel<false>);
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));

@@ -34,12 +34,13 @@ constexpr int kHybTokens = 8;                                  // tokens (= wave
 constexpr int kHybChunk = 16;                                  // token groups per XCD chunk
 constexpr int kRingTiles = 4;
 constexpr int kTileBytes = 32768;                              // K image | V image of one block
-constexpr int kMaxMaskWords = 256;                             // LDS copies of the mask rows: up to 16384 key blocks
+constexpr int kMaxMaskWords = 256;                             // LDS copies of the mask rows hold at most this many words each: 16384 key blocks
 
 struct HybridExtra {
     int groups_per_seq;                                        // ceil(max_seqlen_q / kHybTokens)
     int batch;
     int total_groups;                                          // num_heads_k * batch * groups_per_seq
+    int mask_words;                                            // words per LDS mask row: what max_seqlen_k needs, not the maximum
 };
 
 __device__ __forceinline__ uint32_t lds_address_of(const void* ptr) {
@@ -112,8 +113,8 @@ __global__ __launch_bounds__(512)
 void stage2_fwd_hybrid_kernel(const FwdParams p, const HybridExtra x) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     uint4* ring = reinterpret_cast<uint4*>(smem_raw);                               // [kRingTiles][2048]: K units 0..1023, V units 1024..2047
-    unsigned long long* com = reinterpret_cast<unsigned long long*>(smem_raw + kRingTiles * kTileBytes);   // [kMaxMaskWords]
-    unsigned long long* rows = com + kMaxMaskWords;                                 // [kHybTokens][kMaxMaskWords]
+    unsigned long long* com = reinterpret_cast<unsigned long long*>(smem_raw + kRingTiles * kTileBytes);   // [mask_words]
+    unsigned long long* rows = com + x.mask_words;                                  // [kHybTokens][mask_words]
 
     // ---- which tokens: XCD-chunked, heaviest first ----
     const int bid = blockIdx.x;
@@ -151,9 +152,10 @@ void stage2_fwd_hybrid_kernel(const FwdParams p, const HybridExtra x) {
         int lk = kCausal ? (i_last + Sk - Sq) : (Sk - 1);
         if (lk > Sk - 1) lk = Sk - 1;
         nw = lk < 0 ? 0 : (lk >> 12) + 1;
-        if (mrow && nw > p.n64) nw = p.n64;                                          // nw <= kMaxMaskWords: checked by the launcher
+        if (mrow && nw > p.n64) nw = p.n64;
+        if (nw > x.mask_words) nw = x.mask_words;                                    // a sequence longer than the announced max_seqlen_k
     }
-    unsigned long long* own = rows + wave * kMaxMaskWords;                           // this token's row, later minus the common part
+    unsigned long long* own = rows + wave * x.mask_words;                           // this token's row, later minus the common part
     for (int w = tid; w < nw; w += 512) com[w] = ~0ull;
     __syncthreads();
     for (int w = lane; w < nw; w += 64) {
@@ -352,9 +354,11 @@ int launch_stage2_fwd_hybrid(hipStream_t st, const FwdParams& p, int batch, int 
     IV2_CHECK(total <= 0x3fffffff, "varlen_fwd: too many token groups");
     IV2_CHECK((max_seqlen_k + kBlockN - 1) / kBlockN <= kMaxMaskWords * 64, "varlen_fwd: more than %d key blocks per sequence", kMaxMaskWords * 64);
     x.total_groups = static_cast<int>(total);
+    x.mask_words = ((max_seqlen_k + kBlockN - 1) / kBlockN + 63) / 64;
+    if (x.mask_words < 1) x.mask_words = 1;
     const int64_t per_round = 8 * kHybChunk;
     const int64_t grid = (total + per_round - 1) / per_round * per_round;
-    const size_t lds = kRingTiles * kTileBytes + (1 + kHybTokens) * kMaxMaskWords * 8;
+    const size_t lds = kRingTiles * kTileBytes + static_cast<size_t>(1 + kHybTokens) * x.mask_words * 8;
     const void* fn = causal ? reinterpret_cast<const void*>(&stage2_fwd_hybrid_kernel<true>)
                             : reinterpret_cast<const void*>(&stage2_fwd_hybrid_kernel<false>);
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
