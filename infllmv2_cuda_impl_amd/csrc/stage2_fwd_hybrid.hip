@@ -65,7 +65,17 @@ __device__ __forceinline__ uint64_t uniform_u64(uint64_t v) {
     return (static_cast<uint64_t>(hi) << 32) | lo;
 }
 
-// online-softmax update with one 16 x 64 score tile (s: S^T accumulators); returns P as the B operand of P.V
+// Online-softmax update with one 16 x 64 score tile (s: S^T accumulators); returns P as the B operand of P.V.
+//
+// m is the REFERENCE exponent of the lane's head (log2 units, the same in the four lanes that share a head), not
+// necessarily its running maximum: P = exp2(scale s - m), l and O are all kept relative to m, and out = O / l and
+// LSE = m ln2 + log l hold for any finite m.  So the common path takes m as it is - no row maximum, no cross-lane
+// exchange, no rescale of O - and only checks afterwards that its sixteen P values stayed small (their sum is needed
+// anyway): a lane whose sum exceeds 2^kLazyBits, or whose head has no reference yet, sends the wavefront through the
+// exact path, which moves m to the true running maximum and rescales.  P is rounded to the element type relative to
+// m: its relative rounding error does not depend on the offset, and fp32 l and O have room for 2^kLazyBits many times over.
+constexpr float kLazyLimit = 64.f;                             // 2^6
+
 __device__ __forceinline__ void softmax_step(floatx4 (&s)[4], float& m, float& l, floatx4 (&o)[8], elem8 (&pf)[2],
                                              int lim, int g, float scale_log2) {
     if (lim < kBlockN - 1) {
@@ -75,36 +85,45 @@ __device__ __forceinline__ void softmax_step(floatx4 (&s)[4], float& m, float& l
             for (int e = 0; e < 4; ++e)
                 if (16 * kt + 4 * g + e > lim) s[kt][e] = -INFINITY;
     }
-    float mx = -INFINITY;
-#pragma unroll
-    for (int kt = 0; kt < 4; ++kt)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) mx = fmaxf(mx, s[kt][e]);
-    mx = wave_max_over_g(mx);
-    const float m_new = fmaxf(m, mx * scale_log2);
-    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-    const float alpha = __builtin_amdgcn_exp2f(m - m_use);
+    floatx4 pv[4];
     float rs = 0.f;
 #pragma unroll
     for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            const float pv = __builtin_amdgcn_exp2f(s[kt][e] * scale_log2 - m_use);
-            s[kt][e] = pv;
-            rs += pv;
+            pv[kt][e] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][e], scale_log2, -m));   // m = -inf (no reference yet): +inf or NaN, caught below
+            rs += pv[kt][e];
         }
-    l = l * alpha + rs;
-    m = m_new;
-    if (__ballot(alpha != 1.f) != 0ull) {                      // the running maxima moved (rare after the first blocks)
+    if (__ballot(!(rs <= kLazyLimit)) != 0ull) {               // rare after a row's first blocks; also catches NaN
+        float mx = -INFINITY;
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) mx = fmaxf(mx, s[kt][e]);
+        mx = wave_max_over_g(mx);
+        const float m_new = fmaxf(m, mx * scale_log2);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f(m - m_use);  // 0 when there was no reference
+        rs = 0.f;
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                pv[kt][e] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][e], scale_log2, -m_use));
+                rs += pv[kt][e];
+            }
+        l *= alpha;
+        m = m_new;
 #pragma unroll
         for (int dt = 0; dt < 8; ++dt) o[dt] *= alpha;
     }
+    l += rs;
 #pragma unroll
     for (int cc = 0; cc < 2; ++cc)
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            pf[cc][e] = static_cast<elem_t>(s[2 * cc][e]);
-            pf[cc][4 + e] = static_cast<elem_t>(s[2 * cc + 1][e]);
+            pf[cc][e] = static_cast<elem_t>(pv[2 * cc][e]);
+            pf[cc][4 + e] = static_cast<elem_t>(pv[2 * cc + 1][e]);
         }
 }
 
