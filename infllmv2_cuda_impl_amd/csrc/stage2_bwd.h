@@ -46,6 +46,7 @@ struct BwdParams {
     const elem_bits* ktimg;         // K in V-image order (keys contracted): the A operand of dQ^T = K^T dS^T
     const uint4* rankinfo;          // (Hk, total_q, n64_fwd): {mask word lo, hi, set bits in the row's earlier words, 0}
     int max_sel;                    // upper bound of set bits per mask row
+    int dkdv_spread;                // dK/dV work items: 1 = all XCDs share every slice (few slices), 0 = an XCD owns whole slice groups
 };
 
 // dQ, 8 consecutive tokens per workgroup sharing their common blocks through LDS: stage2_bwd_dq.hip
@@ -57,6 +58,11 @@ int launch_bwd_dkdv_wave(hipStream_t st, const BwdParams& p, int batch, int max_
 int launch_bwd_dq_handoff(hipStream_t st, const BwdParams& p, int batch, int max_seqlen_q, bool causal);
 // deterministic mode only: adds the slots of every key block in slice order into dk_acc / dv_acc
 int launch_bwd_dkdv_reduce(hipStream_t st, const BwdParams& p, int batch);
-constexpr int kDkdvSlice = 512;     // query tokens per dK/dV work item (slices are cut on the packed token axis)
+// Query tokens per dK/dV work item (slices are cut on the packed token axis).  Long inputs use 512-token slices (one
+// flush of the accumulators per 512 tokens); short ones 128, so that a few thousand tokens still make enough work
+// items to fill the device.  The deterministic mode's slot count follows the same rule.
+constexpr int kDkdvSlice = 512;
+constexpr int kDkdvSliceSmall = 128;
+inline int dkdv_slice_tokens(int64_t total_q) { return total_q <= 8192 ? kDkdvSliceSmall : kDkdvSlice; }
 
 }  // namespace IV2_NS

@@ -1,4 +1,5 @@
-// Stage-2 backward, dK / dV (gfx950): two wavefronts per (64-key block, 512-token slice), each owning 32 of the keys.
+// Stage-2 backward, dK / dV (gfx950): two wavefronts per (64-key block, slice of 512 or 128 query tokens), each owning
+// 32 of the keys.
 //
 // Mathematics as in compute_dq_dk_dv_1colblock (csrc/flash_attn/src/flash_bwd_kernel.h:498-794):
 // P = exp(scale S - LSE), dV += P^T dO, dS = P (dP - D), dK += scale dS^T Q, the 16 grouped heads
@@ -31,11 +32,7 @@
 
 namespace IV2_NS {
 
-constexpr int kColSlice = kDkdvSlice;                          // query tokens per work item
-constexpr int kSliceWords = kColSlice / 64;                    // mask words per slice (a power of two)
-constexpr int kGroupWords = 32;                                // one mask word per lane of the lower half-wavefront: 2048 tokens
-constexpr int kGroupSlices = kGroupWords / kSliceWords;        // slices that pool their light members
-constexpr int kHeavyPairs = 128;                               // a slice with fewer selected tokens is "light"
+constexpr int kGroupWords = 32;                                // one mask word per lane of the lower half-wavefront: a group is 2048 tokens
 constexpr int kStage = 16384 + 512 + 512;                      // q a|b, dout a|b (4 KiB each), the pair's 64 row scalars, its two rank records
 constexpr int kWaveLds = 2 * kStage;                           // = 64 rows x 132 floats: also the flush tile
 constexpr int kFlushPitch = 132;                               // floats per key row of the flush tile
@@ -82,9 +79,13 @@ __device__ __forceinline__ short4v lds_read_tr(const unsigned char* ptr) {
     return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v*)(ptr));
 }
 
-template <bool kCausal, bool kHandoff>
+// kColSlice: query tokens per work item (512, or 128 for short inputs)
+template <bool kCausal, bool kHandoff, int kColSlice>
 __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void bwd_dkdv_wave_kernel(const BwdParams p) {
+    constexpr int kSliceWords = kColSlice / 64;                // mask words per slice (a power of two)
+    constexpr int kGroupSlices = kGroupWords / kSliceWords;    // slices that pool their light members
+    constexpr int kHeavyPairs = kColSlice / 4;                 // a slice with fewer selected tokens is "light"
     extern __shared__ __attribute__((aligned(16))) unsigned char ring[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));   // which half of the block's keys
@@ -96,23 +97,31 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
     const int Sk = p.cu_seqlens_k[b + 1] - k0;
     const int nb = (Sk + kBlockN - 1) / kBlockN;               // key blocks of this sequence
 
-    // ---- which (512-token slice, block) ----
-    // Slices are cut on the packed token axis (so they are whole mask words) and clipped to the sequence; four
-    // consecutive slices form a group.  Workgroup ids go round-robin over the 8 XCDs, and XCD x takes the groups
+    // ---- which (slice, block) ----
+    // Slices are cut on the packed token axis (so they are whole mask words) and clipped to the sequence; the slices
+    // of 2048 consecutive tokens form a group.  Workgroup ids go round-robin over the 8 XCDs, and XCD x takes the groups
     // whose index on the packed axis is x modulo 8, latest first, one slice at a time: the wavefronts sharing an L2
     // stream the same tokens of q and dout, and because the assignment follows the packed axis (not each
     // sequence's own first group) the groups of a batch of sequences spread evenly over the XCDs.  Within a slice
     // the shared first block comes first, then the diagonal block and outwards, so the long items are dispatched early.
+    // With fewer groups than XCDs (short inputs) that would leave XCDs idle: then all 8 XCDs share every slice, block
+    // rel going to XCD rel % 8, slices latest first.
     const int xcd = blockIdx.x & 7, turn = blockIdx.x >> 3;
-    const int rel = turn % p.k_blocks;
-    if (Sq <= 0 || rel >= nb) return;                          // uniform
+    if (Sq <= 0) return;                                       // uniform
     const int last_slice = (q0 + Sq - 1) / kColSlice;
-    const int top_group = last_slice / kGroupSlices;
-    const int round = turn / p.k_blocks;                       // an XCD works through one group of slices in consecutive rounds
-    const int grp_idx = top_group - ((top_group - xcd) & 7) - 8 * (round / kGroupSlices);
-    if (grp_idx < 0) return;                                   // uniform
-    const int slice = grp_idx * kGroupSlices + (kGroupSlices - 1 - round % kGroupSlices);
-    if (slice > last_slice || slice < q0 / kColSlice) return;  // uniform
+    int rel, slice;
+    if (p.dkdv_spread) {
+        const int turns_per_slice = (p.k_blocks + 7) >> 3;
+        rel = (turn % turns_per_slice) * 8 + xcd;
+        slice = last_slice - turn / turns_per_slice;
+    } else {
+        rel = turn % p.k_blocks;
+        const int top_group = last_slice / kGroupSlices;
+        const int round = turn / p.k_blocks;                   // an XCD works through one group of slices in consecutive rounds
+        const int grp_idx = top_group - ((top_group - xcd) & 7) - 8 * (round / kGroupSlices);
+        slice = grp_idx < 0 ? -1 : grp_idx * kGroupSlices + (kGroupSlices - 1 - round % kGroupSlices);
+    }
+    if (rel >= nb || slice > last_slice || slice < q0 / kColSlice) return;      // uniform
     int j;
     if (rel == 0) {
         j = 0;
@@ -135,7 +144,7 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
 
     // ---- light slices are merged ----
     // A flush costs 32768 fp32 atomics whatever the slice held, so a slice works on its own only if at least
-    // kHeavyPairs of its tokens selected the block; the other slices of the same group of 4 hand their tokens
+    // kHeavyPairs of its tokens selected the block; the other slices of the same group hand their tokens
     // to the first non-empty one among them.  Every workgroup of the group takes the same decision from the
     // group's 32 mask words (lane l < 32 holds word l; a slice is kSliceWords consecutive lanes).
     unsigned long long* wbuf = reinterpret_cast<unsigned long long*>(ring + kWaveLds);      // [kGroupWords]
@@ -557,25 +566,41 @@ int launch_bwd_dkdv_reduce(hipStream_t st, const BwdParams& p, int batch) {
     return 0;
 }
 
-int launch_bwd_dkdv_wave(hipStream_t st, const BwdParams& p, int batch, int max_seqlen_q, bool causal) {
-    // a sequence of max_seqlen_q tokens touches at most `groups` consecutive slice groups wherever it starts, and an
-    // XCD takes every 8th of them: ceil(groups / 8) rounds of kGroupSlices slices each
-    const int group_tokens = kGroupSlices * kColSlice;
+template <int kColSlice>
+static int launch_bwd_dkdv_sliced(hipStream_t st, const BwdParams& p_in, int batch, int max_seqlen_q, bool causal) {
+    BwdParams p = p_in;
+    constexpr int kGroupSlices = kGroupWords * 64 / kColSlice;
+    // a sequence of max_seqlen_q tokens touches at most `groups` consecutive slice groups wherever it starts
+    const int group_tokens = kGroupWords * 64;
     const int groups = (max_seqlen_q + group_tokens - 1) / group_tokens + 1;
-    const int n_slices8 = (groups + 7) / 8 * (8 * kGroupSlices);
-    const int64_t items = static_cast<int64_t>(n_slices8) * p.k_blocks;
+    int64_t items;
+    // fewer groups than XCDs in the whole batch: every XCD takes a share of every slice
+    p.dkdv_spread = static_cast<int64_t>(batch) * (groups - 1) < 8 ? 1 : 0;
+    if (p.dkdv_spread) {
+        const int n_slices = (max_seqlen_q + kColSlice - 1) / kColSlice + 1;               // a sequence need not start on a slice boundary
+        items = static_cast<int64_t>(n_slices) * ((p.k_blocks + 7) / 8 * 8);
+    } else {
+        // an XCD takes every 8th group: ceil(groups / 8) rounds of kGroupSlices slices each
+        const int n_slices8 = (groups + 7) / 8 * (8 * kGroupSlices);
+        items = static_cast<int64_t>(n_slices8) * p.k_blocks;
+    }
     IV2_CHECK(items <= 0x7fffffffll, "varlen_bwd: too many (slice, block) work items");
     IV2_CHECK(p.q_tok >= 0 && p.q_tok < (1ll << 31) && p.do_tok >= 0 && p.do_tok < (1ll << 31) && p.total_q < (1ll << 31),
               "varlen_bwd: token strides of q and dout must lie in [0, 2^31) elements");
     const dim3 grid(static_cast<unsigned>(items), batch, p.num_heads_k);
     const size_t lds = kWaveLds + kGroupWords * 8;
     const bool handoff = p.ds_buf != nullptr;
-    if (causal && handoff) hipLaunchKernelGGL((bwd_dkdv_wave_kernel<true, true>), grid, dim3(128), lds, st, p);
-    else if (causal) hipLaunchKernelGGL((bwd_dkdv_wave_kernel<true, false>), grid, dim3(128), lds, st, p);
-    else if (handoff) hipLaunchKernelGGL((bwd_dkdv_wave_kernel<false, true>), grid, dim3(128), lds, st, p);
-    else hipLaunchKernelGGL((bwd_dkdv_wave_kernel<false, false>), grid, dim3(128), lds, st, p);
+    if (causal && handoff) hipLaunchKernelGGL((bwd_dkdv_wave_kernel<true, true, kColSlice>), grid, dim3(128), lds, st, p);
+    else if (causal) hipLaunchKernelGGL((bwd_dkdv_wave_kernel<true, false, kColSlice>), grid, dim3(128), lds, st, p);
+    else if (handoff) hipLaunchKernelGGL((bwd_dkdv_wave_kernel<false, true, kColSlice>), grid, dim3(128), lds, st, p);
+    else hipLaunchKernelGGL((bwd_dkdv_wave_kernel<false, false, kColSlice>), grid, dim3(128), lds, st, p);
     IV2_LAUNCH_CHECK();
     return 0;
+}
+
+int launch_bwd_dkdv_wave(hipStream_t st, const BwdParams& p, int batch, int max_seqlen_q, bool causal) {
+    if (dkdv_slice_tokens(p.total_q) == kDkdvSliceSmall) return launch_bwd_dkdv_sliced<kDkdvSliceSmall>(st, p, batch, max_seqlen_q, causal);
+    return launch_bwd_dkdv_sliced<kDkdvSlice>(st, p, batch, max_seqlen_q, causal);
 }
 
 }  // namespace IV2_NS
