@@ -252,7 +252,7 @@ int infllmv2_pack_kv(void* stream, const void* k, const void* v, const int32_t* 
 size_t infllmv2_varlen_bwd_workspace_bytes(int batch, int64_t total_q, int64_t total_k, int num_heads_k,
                                            int max_seqlen_k);
 /* The same plus the slots of the deterministic mode of infllmv2_varlen_bwd (one 64 KiB slot per KV head, key block
- * and 512-token slice of the packed query axis: 4.4 GB at 32768 tokens, growing with the square of the length). */
+ * and slice of the packed query axis (512 tokens; 128 when total_q <= 8192): 4.4 GB at 32768 tokens, growing with the square of the length). */
 size_t infllmv2_varlen_bwd_deterministic_workspace_bytes(int batch, int64_t total_q, int64_t total_k, int num_heads_k,
                                                          int max_seqlen_k);
 /* Workspace of infllmv2_varlen_bwd for any combination of its modes. */
@@ -267,7 +267,7 @@ size_t infllmv2_varlen_bwd_workspace_bytes_ex(int batch, int64_t total_q, int64_
  * dout, q, out, dq: strides {token, head-in-group, kv-head} as in infllmv2_varlen_fwd; k, v, dk, dv:
  * {row, head}; softmax_lse: the forward's output with its strides.  dq, dk, dv are fully written
  * (bf16).  workspace: infllmv2_varlen_bwd_workspace_bytes() bytes, 256-byte aligned.  dQ is always
- * bit-reproducible.  dK/dV are accumulated with fp32 atomics (one flush per 64-key block and 512-token slice),
+ * bit-reproducible.  dK/dV are accumulated with fp32 atomics (one flush per 64-key block and slice of 512 query tokens, 128 when total_q <= 8192),
  * so their last bits can differ between runs, unless `deterministic` is set (the flag of flash_api.cpp:1448-1453,
  * which there concerns dQ): then every work item stores its tiles in a slot of its own and a second kernel adds them
  * in a fixed order; the workspace must then hold infllmv2_varlen_bwd_deterministic_workspace_bytes() bytes.
