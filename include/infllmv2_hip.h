@@ -252,7 +252,7 @@ int infllmv2_pack_kv(void* stream, const void* k, const void* v, const int32_t* 
 size_t infllmv2_varlen_bwd_workspace_bytes(int batch, int64_t total_q, int64_t total_k, int num_heads_k,
                                            int max_seqlen_k);
 /* The same plus the slots of the deterministic mode of infllmv2_varlen_bwd (one 64 KiB slot per KV head, key block
- * and slice of the packed query axis (512 tokens; 128 when total_q <= 8192): 4.4 GB at 32768 tokens, growing with the square of the length). */
+ * and 512-token slice of the packed query axis: 4.4 GB at 32768 tokens, growing with the square of the length). */
 size_t infllmv2_varlen_bwd_deterministic_workspace_bytes(int batch, int64_t total_q, int64_t total_k, int num_heads_k,
                                                          int max_seqlen_k);
 /* Workspace of infllmv2_varlen_bwd for any combination of its modes. */

@@ -60,9 +60,11 @@ int launch_bwd_dq_handoff(hipStream_t st, const BwdParams& p, int batch, int max
 int launch_bwd_dkdv_reduce(hipStream_t st, const BwdParams& p, int batch);
 // Query tokens per dK/dV work item (slices are cut on the packed token axis).  Long inputs use 512-token slices (one
 // flush of the accumulators per 512 tokens); short ones 128, so that a few thousand tokens still make enough work
-// items to fill the device.  The deterministic mode's slot count follows the same rule.
+// items to fill the device; the deterministic mode, whose workspace grows with the slice count, keeps 512.
 constexpr int kDkdvSlice = 512;
 constexpr int kDkdvSliceSmall = 128;
-inline int dkdv_slice_tokens(int64_t total_q) { return total_q <= 8192 ? kDkdvSliceSmall : kDkdvSlice; }
+inline int dkdv_slice_tokens(int64_t total_q, bool deterministic) {
+    return (total_q <= 8192 && !deterministic) ? kDkdvSliceSmall : kDkdvSlice;   // deterministic mode: one slot per slice, so few slices
+}
 
 }  // namespace IV2_NS

@@ -126,7 +126,7 @@ static BwdLayout bwd_layout(int batch, int64_t total_q, int64_t total_k, int num
         L.ds_buf = off; off += align256(static_cast<size_t>(num_heads_k) * total_q * (max_selected + 1) * (kBlockN * 16 * 2));
     }
     L.total = off;
-    L.det_slices = static_cast<int>((total_q + dkdv_slice_tokens(total_q) - 1) / dkdv_slice_tokens(total_q)) + 1;
+    L.det_slices = static_cast<int>((total_q + kDkdvSlice - 1) / kDkdvSlice) + 1;
     const size_t items = static_cast<size_t>(num_heads_k) * image_slots(total_k, batch) * L.det_slices;
     L.det_flags = off; off += align256(items * 4);
     L.det_slots = off; off += align256(items * 2 * kBlockN * kHeadDim * 4);

@@ -599,7 +599,7 @@ static int launch_bwd_dkdv_sliced(hipStream_t st, const BwdParams& p_in, int bat
 }
 
 int launch_bwd_dkdv_wave(hipStream_t st, const BwdParams& p, int batch, int max_seqlen_q, bool causal) {
-    if (dkdv_slice_tokens(p.total_q) == kDkdvSliceSmall) return launch_bwd_dkdv_sliced<kDkdvSliceSmall>(st, p, batch, max_seqlen_q, causal);
+    if (dkdv_slice_tokens(p.total_q, p.det_slots != nullptr) == kDkdvSliceSmall) return launch_bwd_dkdv_sliced<kDkdvSliceSmall>(st, p, batch, max_seqlen_q, causal);
     return launch_bwd_dkdv_sliced<kDkdvSlice>(st, p, batch, max_seqlen_q, causal);
 }
 
