@@ -106,6 +106,14 @@ constexpr elem_bits kElemPosInf = 0x7f80, kElemNegInf = 0xff80;
 __device__ __forceinline__ float elem_to_f32(elem_bits b) { return bf16_to_f32(b); }
 __device__ __forceinline__ elem_bits f32_to_elem(float f) { return f32_to_bf16(f); }
 #endif
+// the same rounding by the conversion instruction (v_cvt_pk_bf16_f32 / v_cvt_f16_f32: round to nearest even): one
+// instruction where f32_to_bf16 spells the rounding out in integer steps; for kernels bound by vector instructions
+__device__ __forceinline__ elem_bits f32_to_elem_hw(float f) {
+    const elem_t x = static_cast<elem_t>(f);
+    elem_bits b;
+    __builtin_memcpy(&b, &x, 2);
+    return b;
+}
 __device__ __forceinline__ uint32_t pack_elem2(float lo, float hi) {
     return static_cast<uint32_t>(f32_to_elem(lo)) | (static_cast<uint32_t>(f32_to_elem(hi)) << 16);
 }

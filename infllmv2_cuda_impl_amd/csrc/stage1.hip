@@ -136,7 +136,8 @@ __global__ __launch_bounds__(64 * kWavesS1) __attribute__((amdgpu_waves_per_eu(k
 void stage1_kernel(const Stage1Params p) {
     __shared__ uint4 tile[2][1024];                            // two 16 KiB operand-ordered key tiles
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);     // wavefront-uniform: what depends on it alone stays in scalar registers
     const int n = lane & 15, g = lane >> 4;
     const int b = blockIdx.y, h = blockIdx.z;
     const int q0 = p.cu_seqlens_q[b];
@@ -189,7 +190,7 @@ void stage1_kernel(const Stage1Params p) {
     const elem_bits* cbase = p.c + static_cast<int64_t>(c0) * p.c_row_stride + h * p.c_head_stride;
     const elem_bits* kbase = p.k + static_cast<int64_t>(k0) * p.k_row_stride + h * p.k_head_stride;
     const uint32_t lds_tiles = __builtin_amdgcn_readfirstlane(s1_lds_addr(tile));
-    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const int wave_u = wave;
     const int c_stride = static_cast<int>(p.c_row_stride), k_stride = static_cast<int>(p.k_row_stride);
     // every ordinary load so far (q) lands before the first LDS-DMA goes out
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -296,7 +297,7 @@ void stage1_kernel(const Stage1Params p) {
         const bool forced = (kb < p.init_blocks) || (bq_t >= kb && bq_t <= kb + p.local_blocks);
         const int first = kb * kKeysPerBlock - 1;              // first key of the window (before clipping at 0)
         const bool empty = (first < 0 ? 0 : first) >= (Lk < p.score_cols ? Lk : p.score_cols);
-        return forced ? kElemPosInf : (empty ? kElemNegInf : f32_to_elem(reached));
+        return forced ? kElemPosInf : (empty ? kElemNegInf : f32_to_elem_hw(reached));
     };
 
     for (int ti = 0; ti < tiles_f; ++ti) {
@@ -331,19 +332,30 @@ void stage1_kernel(const Stage1Params p) {
             // sum over the four 16-lane rows (the head groups) and hand row kt the total of key tile kt, in three
             // exchanges: (row0 + row1 | row2 + row3) of tiles 0/1 and of tiles 2/3, then the two halves
             float mine = fold_rows32(fold_rows16(part[t][0], part[t][1]), fold_rows16(part[t][2], part[t][3]));
-            mine = (col < vis_f[t]) ? mine : 0.f;              // keys the token may not see score 0
+            if ((ti + 1) * 64 > vis_f[t]) mine = (col < vis_f[t]) ? mine : 0.f;   // keys the token may not see score 0 (last tiles only)
             if (!kPool) {
-                if (live[t] && col < p.score_cols) out_rows[t][col] = f32_to_elem(mine);
+                if (live[t] && col < p.score_cols) out_rows[t][col] = f32_to_elem_hw(mine);
             } else {
                 // block kb = col / 4 pools keys 4 kb - 1 .. 4 kb + 3: its quad and the last key of the quad before
-                float left = __shfl_up(mine, 1);
-                if (lane == 0) left = carry[t];
-                carry[t] = __shfl(mine, 63);
+                // the score of the key before: the lane below (one DPP shift over the whole wavefront; lane 0 takes the
+                // last key of the tile before), no trip through the LDS crossbar
+                float left = __uint_as_float(__builtin_amdgcn_update_dpp(__float_as_uint(carry[t]), __float_as_uint(mine),
+                                                                         0x138 /* wave_shr:1 */, 0xF, 0xF, false));
+                carry[t] = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(mine), 63));
                 float best = fmaxf(mine, dpp_quad_xor1(mine));
                 best = fmaxf(best, dpp_quad_xor2(best));
                 best = fmaxf(best, left);
                 const int kb = col >> 2;
-                if (live[t] && (lane & 3) == 0 && kb < p.pool_len) out_rows[t][kb] = pool_rest(kb, bq[t], best);
+                // most tiles lie wholly before the token's local window and after the initial blocks, inside the visible
+                // keys and the pooled row: no block of theirs is forced or empty (wavefront-uniform test)
+                const int kb0 = ti * 16;
+                const bool plain = live[t] && (ti + 1) * 64 <= vis_f[t] && kb0 >= p.init_blocks && kb0 + 15 < bq[t] - p.local_blocks &&
+                                   kb0 + 15 < p.pool_len;
+                if (plain) {
+                    if ((lane & 3) == 0) out_rows[t][kb] = f32_to_elem_hw(best);
+                } else if (live[t] && (lane & 3) == 0 && kb < p.pool_len) {
+                    out_rows[t][kb] = pool_rest(kb, bq[t], best);
+                }
             }
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");

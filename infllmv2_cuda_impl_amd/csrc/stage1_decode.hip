@@ -246,7 +246,7 @@ __device__ __forceinline__ void s1d_score_run(const S1DecodeParams& p, const S1D
         const bool forced = (kb < p.init_blocks) || (bq >= kb && bq <= kb + p.local_blocks);
         const int first = kb * 4 - 1;
         const bool empty = (first < 0 ? 0 : first) >= Lk_cols;
-        return forced ? kElemPosInf : (empty ? kElemNegInf : f32_to_elem(reached));
+        return forced ? kElemPosInf : (empty ? kElemNegInf : f32_to_elem_hw(reached));
     };
     // one 16-key group: this lane's four heads summed for key 16 kt + n of the tile
     auto group_part = [&](const elem8* t4) -> float {
@@ -280,7 +280,7 @@ __device__ __forceinline__ void s1d_score_run(const S1DecodeParams& p, const S1D
         float mine = s1d_fold_rows32(s1d_fold_rows16(part[0], part[1]), s1d_fold_rows16(part[2], part[3]));
         mine = (col < vis_f) ? mine : 0.f;
         if (!kPool) {
-            if (col < p.cols) out[col] = f32_to_elem(mine);
+            if (col < p.cols) out[col] = f32_to_elem_hw(mine);
         } else {
             float left = __shfl_up(mine, 1);
             if (lane == 0) left = carry;
