@@ -301,6 +301,20 @@ def stream_probes(torch, _lib, dev):
         record[name] = {"tbs_all_cus": wgs * iters * 131072 / ms / 1e9,
                         "gbs_per_cu": iters * 131072 / ms / 1e6,
                         "bytes_per_counter_tick_per_cu": float(np.median(o[:, 1] / o[:, 0]))}
+    issue_iters = 20000
+    ticks = torch.zeros(wgs, dtype=torch.int64, device=dev)
+    issue = {}
+    for mode, name in ((0, "8_mfma"), (1, "32_fma"), (2, "8_exp2"), (3, "8x(mfma+2fma)"), (4, "8x(mfma+4fma)"),
+                       (5, "attention_block"), (6, "attention_block_with_branch_on_row_sum")):
+        launch = lambda: _lib.call("infllmv2_probe_issue", stream, ticks.data_ptr(), wgs, issue_iters, mode)
+        ms = min(event_ms(torch, launch, 3) for _ in range(3))
+        issue[name] = {"ns_per_round_two_wavefronts": ms * 1e6 / issue_iters,
+                       "counter_ticks_per_round": float(np.median(ticks.cpu().numpy().astype(np.float64))) / issue_iters}
+    issue["what"] = ("256 workgroups of 8 wavefronts (one per CU, two wavefronts per SIMD), register operands only, "
+                     "20000 rounds; a round is what the name says PER WAVEFRONT (an attention block = 16 S MFMA, "
+                     "16 x (multiply-add, exp2, add), 8 conversions, 16 P.V MFMA); ns per round is the time a SIMD "
+                     "needs for the round of both its wavefronts")
+    record["issue"] = issue
     record["what"] = ("each of 256 workgroups (8 wavefronts, one per CU) re-reads its own 128 KiB 400 times, 16 KiB "
                       "in flight per wavefront; wall time from HIP events (includes the 128 KiB LDS fill and the launch), "
                       "ticks from s_memtime inside the kernel, median over workgroups")

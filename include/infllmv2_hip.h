@@ -44,6 +44,13 @@ int infllmv2_check_device(int device);
 int infllmv2_probe_stream(void* stream, const void* src, size_t src_bytes, unsigned long long* out, int workgroups,
                           int iters, int mode);
 
+/* Measurement aid, no counterpart in the reference and not on the attention path: `workgroups` workgroups of eight
+ * wavefronts (two per SIMD) run `iters` rounds of register-only arithmetic: 8 MFMA (mode 0), 32 fp32 multiply-adds
+ * (1), 8 exp2 (2), 8 x (MFMA + 2 multiply-adds) (3), 8 x (MFMA + 4 multiply-adds) (4), one attention block as the
+ * Stage-2 forward issues it (5), the same with a branch on the row sum (6).  out[w] = cycle-counter ticks of workgroup
+ * w; with one workgroup per CU, time per round is what the SIMD's shared MFMA / VALU issue costs. */
+int infllmv2_probe_issue(void* stream, unsigned long long* out, int workgroups, int iters, int mode);
+
 /* ---- block-mask bit operations -------------------------------------------------------------- */
 
 /* csrc/entry.cu:78-96 `topk_to_uint64` (kernel csrc/topk_to_uint64.cuh:10-76).

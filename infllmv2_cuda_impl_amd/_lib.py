@@ -19,6 +19,7 @@ _p, _i, _i64, _sz, _f = C.c_void_p, C.c_int, C.c_int64, C.c_size_t, C.c_float
 SIGNATURES = {
     "infllmv2_check_device": [_i],
     "infllmv2_probe_stream": [_p, _p, _sz, _p, _i, _i, _i],
+    "infllmv2_probe_issue": [_p, _p, _i, _i, _i],
     "infllmv2_topk_to_uint64": [_p, _p, _p, _i64, _i, _i, _i],
     "infllmv2_uint64_to_bool": [_p, _p, _p, _i64, _i, _i],
     "infllmv2_blockmask_to_uint64": [_p, _p, _p, _i64, _i, _i],
