@@ -148,6 +148,21 @@ def test_config3_varlen_fwd_bwd_64k(ops, monkeypatch):
         dk_scale = float(kg.grad[sl].float().abs().sum(0).max())
         assert float(dk_sum.abs().max()) <= 2e-2 * dk_scale
     assert bool(torch.isfinite(qg.grad.float()).all() and torch.isfinite(kg.grad.float()).all())
+    # whole-tensor inner products: O is linear in V, so <dO, O> = <dV, V>; S is bilinear in (Q, K), so scaling Q up and K
+    # down by the same factor changes nothing and <dQ, Q> = <dK, K>.  Every element of dQ, dK and dV enters; the
+    # tolerance is 3.5 times the largest difference these inputs give (1.7e-3 of the terms' root sum of squares), which rounding
+    # each factor to bf16 explains; the inner products themselves are 0.5 to 3 of that norm.
+    def inner(a, b):
+        prod = a.detach().double() * b.detach().double()
+        return float(prod.sum()), float(prod.pow(2).sum().sqrt())
+    for b in range(4):
+        sl = slice(int(cu_l[b]), int(cu_l[b + 1]))
+        x_o, n_o = inner(dout[sl], out[sl])
+        x_v, n_v = inner(vg.grad[sl], v[sl])
+        assert abs(x_o - x_v) <= 6e-3 * (n_o + n_v), ("<dO,O> vs <dV,V>", b, x_o, x_v, n_o, n_v)
+        x_q, n_q = inner(qg.grad[sl], q[sl])
+        x_k, n_k = inner(kg.grad[sl], k[sl])
+        assert abs(x_q - x_k) <= 6e-3 * (n_q + n_k), ("<dQ,Q> vs <dK,K>", b, x_q, x_k, n_q, n_k)
     # dK / dV element by element on sampled key blocks: per sequence one late block (few tokens, all near its diagonal:
     # a light slice that the column kernel merges with others) and one mid-prefix block that many distant tokens
     # chose by score (many 512-token slices, multi-slice accumulation); never block 0.  The oracle only needs the
