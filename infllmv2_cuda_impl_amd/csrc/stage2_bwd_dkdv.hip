@@ -353,10 +353,23 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
         const uint4* frag = reinterpret_cast<const uint4*>(st) + frag_unit;      // tile t, chunk c at frag[t * 256 + c * 64]
         elem8 pfr[kWaveTiles], dsfr[kWaveTiles];              // per key tile: [token a heads 4g..4g+3 | token b heads 4g..4g+3]
         floatx4 sa[kWaveTiles], sb[kWaveTiles], dpa[kWaveTiles], dpb[kWaveTiles];
+        // Without the hand-off the S accumulators start at -LSE / scale, so that P = exp2(scale S') needs no subtraction
+        // (and the LSE no registers) after the MFMAs; a row without visible keys has LSE = +inf: S' = -inf, P = 0.  With
+        // the hand-off's extra addresses live that form spills a register, so there the LSE is subtracted after the MFMAs.
+        constexpr bool kFoldLse = !kHandoff;
+        if (kFoldLse) {
+            const float4 la = *reinterpret_cast<const float4*>(scal + 4 * g);
+            const float4 lb = *reinterpret_cast<const float4*>(scal + 64 + 4 * g);
+            const float inv = -1.f / p.scale_log2;
+            const floatx4 ia = {la.x * inv, la.y * inv, la.z * inv, la.w * inv}, ib = {lb.x * inv, lb.y * inv, lb.z * inv, lb.w * inv};
 #pragma unroll
-        for (int kt = 0; kt < kWaveTiles; ++kt) {
-            sa[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
-            sb[kt] = sa[kt];
+            for (int kt = 0; kt < kWaveTiles; ++kt) { sa[kt] = ia; sb[kt] = ib; }
+        } else {
+#pragma unroll
+            for (int kt = 0; kt < kWaveTiles; ++kt) {
+                sa[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
+                sb[kt] = sa[kt];
+            }
         }
         {   // A
 #pragma unroll
@@ -374,16 +387,19 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
         }
         __builtin_amdgcn_sched_barrier(0);
         {   // P, kept in fp32 in place of S
-            const float4 la = *reinterpret_cast<const float4*>(scal + 4 * g);
-            const float4 lb = *reinterpret_cast<const float4*>(scal + 64 + 4 * g);
-            const float lse_a[4] = {la.x, la.y, la.z, la.w};
-            const float lse_b[4] = {lb.x, lb.y, lb.z, lb.w};
+            float lse_a[4] = {0.f, 0.f, 0.f, 0.f}, lse_b[4] = {0.f, 0.f, 0.f, 0.f};
+            if (!kFoldLse) {
+                const float4 la = *reinterpret_cast<const float4*>(scal + 4 * g);
+                const float4 lb = *reinterpret_cast<const float4*>(scal + 64 + 4 * g);
+                lse_a[0] = la.x; lse_a[1] = la.y; lse_a[2] = la.z; lse_a[3] = la.w;
+                lse_b[0] = lb.x; lse_b[1] = lb.y; lse_b[2] = lb.z; lse_b[3] = lb.w;
+            }
 #pragma unroll
             for (int kt = 0; kt < kWaveTiles; ++kt)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    float xa = __builtin_amdgcn_exp2f(sa[kt][e] * p.scale_log2 - lse_a[e]);
-                    float xb = __builtin_amdgcn_exp2f(sb[kt][e] * p.scale_log2 - lse_b[e]);
+                    float xa = __builtin_amdgcn_exp2f(kFoldLse ? sa[kt][e] * p.scale_log2 : sa[kt][e] * p.scale_log2 - lse_a[e]);
+                    float xb = __builtin_amdgcn_exp2f(kFoldLse ? sb[kt][e] * p.scale_log2 : sb[kt][e] * p.scale_log2 - lse_b[e]);
                     sa[kt][e] = xa;
                     sb[kt][e] = xb;
                     pfr[kt][e] = static_cast<elem_t>(xa);
