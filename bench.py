@@ -83,9 +83,6 @@ def parse_args():
                     help="skip BASELINE configs 3, 4 and 5 (keeps a profile to the default workload)")
     ap.add_argument("--only-config", type=int, default=0, choices=[0, 3, 4, 5],
                     help="run one of the extra configurations alone (for profiling it) and print its record")
-    ap.add_argument("--probe", action="store_true",
-                    help="run the streaming probes (bytes per clock a CU gets through its L1 return path and from LDS) "
-                         "and print their record instead of the benchmark")
     ap.add_argument("--print-source-hash", action="store_true",
                     help="print the hash of the Stage-2 forward kernel sources (what a traffic summary must name) and exit")
     return ap.parse_args()
@@ -283,44 +280,6 @@ def decode_bench(torch, ops, dev):
             "step_frac_hbm_peak": gbs(s1_bytes + s2_bytes, step_ms) / PEAK_HBM_GBS}
 
 
-def stream_probes(torch, _lib, dev):
-    """What one CU receives per unit time from L2-resident data through global_load_dwordx4 and through LDS-DMA (the
-    L1 return path that bounds the Stage-2 gather) and from LDS through ds_read_b128.  One workgroup of eight
-    wavefronts per CU, 256 CUs; wall time from HIP events, ticks from the kernel's own cycle counter."""
-    import numpy as np
-    wgs, iters = 256, 400
-    src = torch.arange(wgs * 131072 // 4, dtype=torch.int32, device=dev)
-    out = torch.zeros(2 * wgs, dtype=torch.int64, device=dev)
-    stream = torch.cuda.current_stream(dev).cuda_stream
-    record = {}
-    for mode, name in ((0, "global_load_dwordx4"), (1, "lds_dma_dwordx4"), (2, "ds_read_b128"), (3, "ds_read_b64_tr_b16")):
-        launch = lambda: _lib.call("infllmv2_probe_stream", stream, src.data_ptr(), src.numel() * 4, out.data_ptr(),
-                                   wgs, iters, mode)
-        ms = min(event_ms(torch, launch, 3) for _ in range(3))
-        o = out.cpu().numpy().reshape(wgs, 2).astype(np.float64)
-        record[name] = {"tbs_all_cus": wgs * iters * 131072 / ms / 1e9,
-                        "gbs_per_cu": iters * 131072 / ms / 1e6,
-                        "bytes_per_counter_tick_per_cu": float(np.median(o[:, 1] / o[:, 0]))}
-    issue_iters = 20000
-    ticks = torch.zeros(wgs, dtype=torch.int64, device=dev)
-    issue = {}
-    for mode, name in ((0, "8_mfma"), (1, "32_fma"), (2, "8_exp2"), (3, "8x(mfma+2fma)"), (4, "8x(mfma+4fma)"),
-                       (5, "attention_block"), (6, "attention_block_with_branch_on_row_sum")):
-        launch = lambda: _lib.call("infllmv2_probe_issue", stream, ticks.data_ptr(), wgs, issue_iters, mode)
-        ms = min(event_ms(torch, launch, 3) for _ in range(3))
-        issue[name] = {"ns_per_round_two_wavefronts": ms * 1e6 / issue_iters,
-                       "counter_ticks_per_round": float(np.median(ticks.cpu().numpy().astype(np.float64))) / issue_iters}
-    issue["what"] = ("256 workgroups of 8 wavefronts (one per CU, two wavefronts per SIMD), register operands only, "
-                     "20000 rounds; a round is what the name says PER WAVEFRONT (an attention block = 16 S MFMA, "
-                     "16 x (multiply-add, exp2, add), 8 conversions, 16 P.V MFMA); ns per round is the time a SIMD "
-                     "needs for the round of both its wavefronts")
-    record["issue"] = issue
-    record["what"] = ("each of 256 workgroups (8 wavefronts, one per CU) re-reads its own 128 KiB 400 times, 16 KiB "
-                      "in flight per wavefront; wall time from HIP events (includes the 128 KiB LDS fill and the launch), "
-                      "ticks from s_memtime inside the kernel, median over workgroups")
-    return record
-
-
 def cpu_model():
     try:
         with open("/proc/cpuinfo") as f:
@@ -396,9 +355,6 @@ def main():
     from infllmv2_cuda_impl_amd import _lib
 
     dev = torch.device("cuda:0")
-    if args.probe:
-        print(json.dumps(stream_probes(torch, _lib, dev)))
-        return
     if args.only_config:
         fn = {3: config3_bench, 4: config4_bench, 5: decode_bench}[args.only_config]
         print(json.dumps(fn(torch, ops, dev)))

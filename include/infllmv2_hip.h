@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define INFLLMV2_ABI_VERSION 8
+#define INFLLMV2_ABI_VERSION 9
 
 /* ---- library ------------------------------------------------------------------------------ */
 
@@ -35,21 +35,6 @@ int infllmv2_abi_version(void);
 /* 0 iff `device` is a gfx950 GPU.  Replaces the sm80/sm90 gate of
  * csrc/flash_attn/flash_api.cpp:546-550. */
 int infllmv2_check_device(int device);
-
-/* Measurement aid, no counterpart in the reference and not on the attention path: `workgroups` workgroups of eight
- * wavefronts each re-read their own 128 KiB of `src` `iters` times with global_load_dwordx4 (mode 0), LDS-DMA
- * (mode 1), ds_read_b128 from an LDS copy (mode 2) or ds_read_b64_tr_b16 from it (mode 3).  out[2 w] = cycle-counter ticks workgroup w took, out[2 w + 1] =
- * bytes it moved: with one workgroup per CU, bytes over time is what a CU's L1 return path (modes 0, 1) or its LDS
- * (mode 2) delivers, the rates the Stage-2 gather is held against. */
-int infllmv2_probe_stream(void* stream, const void* src, size_t src_bytes, unsigned long long* out, int workgroups,
-                          int iters, int mode);
-
-/* Measurement aid, no counterpart in the reference and not on the attention path: `workgroups` workgroups of eight
- * wavefronts (two per SIMD) run `iters` rounds of register-only arithmetic: 8 MFMA (mode 0), 32 fp32 multiply-adds
- * (1), 8 exp2 (2), 8 x (MFMA + 2 multiply-adds) (3), 8 x (MFMA + 4 multiply-adds) (4), one attention block as the
- * Stage-2 forward issues it (5), the same with a branch on the row sum (6).  out[w] = cycle-counter ticks of workgroup
- * w; with one workgroup per CU, time per round is what the SIMD's shared MFMA / VALU issue costs. */
-int infllmv2_probe_issue(void* stream, unsigned long long* out, int workgroups, int iters, int mode);
 
 /* ---- block-mask bit operations -------------------------------------------------------------- */
 
@@ -153,12 +138,15 @@ int infllmv2_compress_keys(void* stream, const void* k, void* out, const int32_t
  * holds new_lens[b] keys of sequence b, out_cache (batch, rows capacity, Hk, d) its compressed keys; strides
  * {batch, row, head}.  Rows whose windows were completed between old_lens[b] (null: 0) and new_lens[b] tokens are
  * written, at most max_new_rows per sequence (the caller's bound: 1 for a one-token step with kernel_size a multiple
- * of stride); out_lens (batch, or null) receives the number of rows the compressed cache then holds.  The caller
+ * of stride); out_lens (batch, or null) receives the number of rows the compressed cache then holds.  kcache_rows and
+ * out_rows are the row capacities of one sequence's key cache and compressed cache: a length beyond the key cache is
+ * read as its capacity, no row >= out_rows is written, and out_lens never counts a row this call did not cover.  The caller
  * side of the reference does this in Python for one sequence at a time (tests/test_stage1_compressed_lse.py:56-99). */
 int infllmv2_compress_keys_cache(void* stream, const void* kcache, void* out_cache, const int32_t* old_lens,
                                  const int32_t* new_lens, int32_t* out_lens, int batch, int max_new_rows,
                                  int num_heads_k, int head_dim, const int64_t* kcache_strides,
-                                 const int64_t* out_strides, int kernel_size, int stride);
+                                 const int64_t* out_strides, int kernel_size, int stride, int kcache_rows,
+                                 int out_rows);
 
 /* ---- Stage 1: scoring over compressed keys --------------------------------------------------- */
 
@@ -370,7 +358,8 @@ int infllmv2_compress_keys_f16(void* stream, const void* k, void* out, const int
 int infllmv2_compress_keys_cache_f16(void* stream, const void* kcache, void* out_cache, const int32_t* old_lens,
                                      const int32_t* new_lens, int32_t* out_lens, int batch, int max_new_rows,
                                      int num_heads_k, int head_dim, const int64_t* kcache_strides,
-                                     const int64_t* out_strides, int kernel_size, int stride);
+                                     const int64_t* out_strides, int kernel_size, int stride, int kcache_rows,
+                                     int out_rows);
 int infllmv2_varlen_fwd_stage1_f16(void* stream, const void* q, const void* k, const void* v, void* score,
                                    const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
                                    const int32_t* cu_seqlens_v, int batch, int64_t total_q, int num_heads,

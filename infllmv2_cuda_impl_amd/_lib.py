@@ -11,15 +11,13 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libinfllmv2_hip.so")
 
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 _p, _i, _i64, _sz, _f = C.c_void_p, C.c_int, C.c_int64, C.c_size_t, C.c_float
 
 # name -> argtypes; every function returns int except the three noted below
 SIGNATURES = {
     "infllmv2_check_device": [_i],
-    "infllmv2_probe_stream": [_p, _p, _sz, _p, _i, _i, _i],
-    "infllmv2_probe_issue": [_p, _p, _i, _i, _i],
     "infllmv2_topk_to_uint64": [_p, _p, _p, _i64, _i, _i, _i],
     "infllmv2_uint64_to_bool": [_p, _p, _p, _i64, _i, _i],
     "infllmv2_blockmask_to_uint64": [_p, _p, _p, _i64, _i, _i],
@@ -32,7 +30,7 @@ SIGNATURES = {
     "infllmv2_topk_blocks": [_p, _p, _i64, _p, _i64, _i, _i],
     "infllmv2_topk_select": [_p, _p, _i64, _i, _p, _p, _i64, _i, _i, _i, _i, _i],
     "infllmv2_compress_keys": [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i64, _i64, _i, _i, _i],
-    "infllmv2_compress_keys_cache": [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _p, _p, _i, _i],
+    "infllmv2_compress_keys_cache": [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _p, _p, _i, _i, _i, _i],
     "infllmv2_varlen_fwd_stage1": [_p, _p, _p, _p, _p, _p, _p, _p, _i, _i64, _i, _i, _i, _i, _i, _p, _p, _p, _i64, _i64, _f, _i],
     "infllmv2_varlen_fwd_stage1_pooled": [_p] * 9 + [_i, _i, _i64, _i, _i, _i, _i, _i, _p, _p, _p, _i, _f] + [_i] * 7,
     "infllmv2_stage1_decode": [_p] * 11 + [_sz] + [_i] * 6 + [_p] * 3 + [_i64, _i64, _f, _i, _i, _p] + [_i] * 8,

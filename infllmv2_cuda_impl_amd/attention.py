@@ -181,9 +181,13 @@ class Infllmv2AttnVarlenFunc(torch.autograd.Function):
         sparse = topk_idx is not None or block_mask is not None
         if block_mask is not None:
             # the packed selection itself (topk_blocks(return_mask=True)): nothing to pack
+            # rows may be wider than max_seqlen_k needs (select_blocks widens them for cached tokens): the kernels take
+            # the width as a row stride and never look at a block beyond the sequence
             n64 = ((max_seqlen_k + BLOCK_N - 1) // BLOCK_N + 63) // 64
-            if block_mask.dtype != torch.int64 or tuple(block_mask.shape) != (k.shape[1], q.shape[0], n64):
-                raise RuntimeError("block_mask must be int64 of shape (num_heads_k, total_q, ceil(ceil(max_seqlen_k / 64) / 64))")
+            if block_mask.dtype != torch.int64 or block_mask.dim() != 3 or \
+                    tuple(block_mask.shape[:2]) != (k.shape[1], q.shape[0]) or block_mask.shape[2] < n64:
+                raise RuntimeError("block_mask must be int64 of shape (num_heads_k, total_q, words) with "
+                                   "words >= ceil(ceil(max_seqlen_k / 64) / 64)")
             require_gpu(block_mask, "block_mask")
             fwd_mask = block_mask.contiguous()
         elif topk_idx is not None:
@@ -200,7 +204,9 @@ class Infllmv2AttnVarlenFunc(torch.autograd.Function):
         ctx.causal = causal
         ctx.deterministic = deterministic
         ctx.sparse = sparse
-        ctx.max_selected = topk_idx.shape[-1] if topk_idx is not None else 0     # a mask row has at most k set bits
+        # the bound on set bits per mask row that the dS hand-off of the backward sizes its tiles by: known only when
+        # the mask was packed here from topk_idx (a caller's own mask may hold more blocks per row than k)
+        ctx.max_selected = topk_idx.shape[-1] if (topk_idx is not None and block_mask is None) else 0
         if not return_softmax:
             return out
         # S_dmask is only materialised with dropout, which this build rejects
@@ -408,8 +414,10 @@ def infllmv2_attn_with_kvcache(q, k_cache, v_cache, k=None, v=None, rotary_cos=N
     mask = None
     if block_mask is not None:
         # the packed selection (batch, nheads_k, 1, words) as topk_blocks(return_mask=True) writes it
-        if block_mask.dtype != torch.int64 or block_mask.dim() != 4:
-            raise RuntimeError("block_mask must be int64 of shape (batch_size, num_heads_k, 1, words)")
+        require_gpu(block_mask, "block_mask")
+        if block_mask.dtype != torch.int64 or block_mask.dim() != 4 or block_mask.shape[0] != q.shape[0] or \
+                block_mask.shape[2] != 1 or block_mask.shape[1] != k_cache.shape[-2] or block_mask.device != q.device:
+            raise RuntimeError("block_mask must be an int64 tensor of shape (batch_size, num_heads_k, 1, words) on q's device")
         mask = block_mask.contiguous()
     elif topk_idx is not None:
         assert topk_idx.dtype == torch.int32

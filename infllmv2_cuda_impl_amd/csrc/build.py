@@ -15,6 +15,17 @@ PKG = os.path.dirname(CSRC)
 LIB_PATH = os.path.join(PKG, "libinfllmv2_hip.so")
 OBJ_DIR = os.path.join(PKG, "build")
 
+
+def include_dir() -> str:
+    """Directory that holds infllmv2_hip.h, the C-ABI header the sources include by name: `include/` beside the
+    package in a source checkout, `include/` inside the package where it was installed from a built distribution
+    (setup.py copies the header there)."""
+    for cand in (os.path.join(PKG, "include"), os.path.join(os.path.dirname(PKG), "include")):
+        if os.path.exists(os.path.join(cand, "infllmv2_hip.h")):
+            return cand
+    raise RuntimeError("infllmv2_hip.h not found: expected in " + os.path.join(PKG, "include") + " or "
+                       + os.path.join(os.path.dirname(PKG), "include"))
+
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffast-math", "-fno-finite-math-only", *os.environ.get("IV2_EXTRA_FLAGS", "").split(),
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
@@ -46,7 +57,7 @@ def sources():
 def _compile(unit, verbose: bool) -> str:
     src, extra, obj_name = unit
     obj = os.path.join(OBJ_DIR, obj_name)
-    cmd = ["hipcc", *HIPCC_FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = ["hipcc", *HIPCC_FLAGS, "-I", include_dir(), *extra, "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
     if r.returncode != 0:

@@ -1,6 +1,6 @@
 // Library-level C entry points: error text, version, device check.
 #include "common.h"
-#include "../../include/infllmv2_hip.h"
+#include "infllmv2_hip.h"
 #include <string.h>
 
 namespace infllmv2 {

@@ -9,7 +9,7 @@
 // HBM-bound and small: K is read once from memory (the overlapping windows hit in cache) and
 // the output is 1/stride of its size.  A thread owns 8 contiguous d values (16 bytes) of one output row.
 #include "common.h"
-#include "../../include/infllmv2_hip.h"
+#include "infllmv2_hip.h"
 
 namespace IV2_NS {
 
@@ -90,13 +90,29 @@ struct CompressCacheParams {
     int64_t k_batch, k_row, k_head, o_batch, o_row, o_head;
     int units_per_row, units_per_head;
     int kernel_size, stride;
+    int k_capacity;                  // rows of one sequence's key cache: a length beyond it is read as the capacity
+    int out_capacity;                // rows of one sequence's compressed cache: nothing is written beyond it
+    int max_new_rows;                // rows this call may add per sequence (what the launch covers)
 };
+
+// Rows sequence b's compressed cache holds after the call, and the first of them this call writes: the windows
+// completed by new_lens[b] tokens, never more than the output has rows, the key cache has windows, or the launch
+// covers (so that the reported length never includes a row that was not written).
+__device__ __forceinline__ void cache_row_range(const CompressCacheParams& p, int b, int& first, int& rows) {
+    int new_len = p.new_lens[b];
+    if (new_len > p.k_capacity) new_len = p.k_capacity;
+    rows = compressed_rows(new_len, p.kernel_size, p.stride);
+    first = p.old_lens ? compressed_rows(p.old_lens[b], p.kernel_size, p.stride) : 0;
+    if (first < 0) first = 0;
+    if (rows > p.out_capacity) rows = p.out_capacity;
+    if (rows > first + p.max_new_rows) rows = first + p.max_new_rows;
+}
 
 __global__ __launch_bounds__(256)
 void compress_keys_cache_kernel(const CompressCacheParams p) {
     const int b = blockIdx.y;
-    const int rows = compressed_rows(p.new_lens[b], p.kernel_size, p.stride);
-    const int first = p.old_lens ? compressed_rows(p.old_lens[b], p.kernel_size, p.stride) : 0;
+    int first, rows;
+    cache_row_range(p, b, first, rows);
     if (blockIdx.x == 0 && threadIdx.x == 0 && p.out_lens) p.out_lens[b] = rows;
     const int j0 = first + blockIdx.x * kCompressRowsPerWg;
     for (int item = threadIdx.x; item < kCompressRowsPerWg * p.units_per_row; item += 256) {
@@ -139,8 +155,8 @@ __global__ __launch_bounds__(256)
 void compress_keys_cache_append_kernel(const CompressCacheParams p) {
     extern __shared__ uint4 window[];                          // [kernel_size][kAppendUnits]
     const int b = blockIdx.y;
-    const int rows = compressed_rows(p.new_lens[b], p.kernel_size, p.stride);
-    const int first = p.old_lens ? compressed_rows(p.old_lens[b], p.kernel_size, p.stride) : 0;
+    int first, rows;
+    cache_row_range(p, b, first, rows);
     if (blockIdx.x == 0 && blockIdx.z == 0 && threadIdx.x == 0 && p.out_lens) p.out_lens[b] = rows;
     const int j = first + blockIdx.x;
     if (j >= rows) return;                                     // uniform per workgroup
@@ -205,8 +221,10 @@ extern "C" int IV2_ENTRY(infllmv2_compress_keys)(void* stream, const void* k, vo
 extern "C" int IV2_ENTRY(infllmv2_compress_keys_cache)(void* stream, const void* kcache, void* out_cache, const int32_t* old_lens,
                                             const int32_t* new_lens, int32_t* out_lens, int batch, int max_new_rows,
                                             int num_heads_k, int head_dim, const int64_t* kcache_strides,
-                                            const int64_t* out_strides, int kernel_size, int stride) {
+                                            const int64_t* out_strides, int kernel_size, int stride,
+                                            int kcache_rows, int out_rows) {
     IV2_CHECK(batch > 0 && batch <= 65535 && max_new_rows >= 0, "compress_keys_cache: bad batch or max_new_rows");
+    IV2_CHECK(kcache_rows >= 0 && out_rows >= 0, "compress_keys_cache: negative cache capacity");
     IV2_CHECK(kernel_size > 0 && stride > 0, "compress_keys_cache: kernel_size and stride must be positive");
     IV2_CHECK(kcache && out_cache && new_lens, "compress_keys_cache: null pointer");
     IV2_CHECK(head_dim > 0 && head_dim % 8 == 0 && num_heads_k > 0, "compress_keys_cache: head_dim must be a multiple of 8");
@@ -222,6 +240,7 @@ extern "C" int IV2_ENTRY(infllmv2_compress_keys_cache)(void* stream, const void*
     p.o_batch = out_strides[0]; p.o_row = out_strides[1]; p.o_head = out_strides[2];
     p.units_per_row = num_heads_k * head_dim / 8; p.units_per_head = head_dim / 8;
     p.kernel_size = kernel_size; p.stride = stride;
+    p.k_capacity = kcache_rows; p.out_capacity = out_rows; p.max_new_rows = max_new_rows;
     const size_t window_bytes = static_cast<size_t>(kernel_size) * kAppendUnits * 16;
     if (max_new_rows >= 1 && max_new_rows <= 8 && window_bytes <= kAppendMaxLds) {
         // a decode step's append: one workgroup per new row and 32 units

@@ -17,7 +17,7 @@
 // is read back transposed.  Partial results are merged by a small combine kernel.
 #include "common.h"
 #include "block_walker.h"
-#include "../../include/infllmv2_hip.h"
+#include "infllmv2_hip.h"
 #include <math.h>
 #include <mutex>
 
@@ -538,9 +538,17 @@ extern "C" int infllmv2_fwd_kvcache_static(void* stream, const void* q, void* kc
               "fwd_kvcache_static: batch %d x %d KV heads x %d splits needs %zu bytes of scratch, the built-in buffer holds %zu; "
               "use fewer splits or infllmv2_fwd_kvcache with a workspace", batch, num_heads_k, num_splits, need,
               static_cast<size_t>(INFLLMV2_STATIC_SCRATCH_BYTES));
-    int dev = -1;
+    // the copy of the array that belongs to the GPU the stream runs on (the null stream: the current device); the
+    // symbol lookup below answers for the current device, so the two must be the same
+    int dev = -1, stream_dev = -1;
     hipError_t e = hipGetDevice(&dev);
     IV2_CHECK(e == hipSuccess && dev >= 0 && dev < kMaxDevices, "fwd_kvcache_static: hipGetDevice failed or device index %d out of range", dev);
+    if (stream != nullptr) {
+        e = hipStreamGetDevice(static_cast<hipStream_t>(stream), &stream_dev);
+        IV2_CHECK(e == hipSuccess, "fwd_kvcache_static: hipStreamGetDevice failed: %s", hipGetErrorString(e));
+        IV2_CHECK(stream_dev == dev, "fwd_kvcache_static: the stream belongs to device %d but the current device is %d; "
+                  "make the stream's device current before the call", stream_dev, dev);
+    }
     void* ws = nullptr;
     {
         std::lock_guard<std::mutex> lock(g_scratch_mutex);

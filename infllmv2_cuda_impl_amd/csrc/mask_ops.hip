@@ -6,7 +6,7 @@
 // csrc/blockmask_to_uint64.cuh:10-51 and infllm_v2/infllmv2_sparse_attention.py:344-350 of the
 // reference; the kernels themselves are new.
 #include "common.h"
-#include "../../include/infllmv2_hip.h"
+#include "infllmv2_hip.h"
 
 namespace infllmv2 {
 

@@ -14,7 +14,7 @@
 // read before and after the row cannot fault), and every window is then read from LDS.  Rows too
 // long for LDS take the direct kernel, one workgroup per (query row, head).
 #include "common.h"
-#include "../../include/infllmv2_hip.h"
+#include "infllmv2_hip.h"
 
 namespace infllmv2 {
 

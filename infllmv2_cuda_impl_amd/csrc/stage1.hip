@@ -20,7 +20,7 @@
 // by all 16 tokens, and inside a wavefront one operand read feeds two MFMAs.
 #include "common.h"
 #include "block_walker.h"
-#include "../../include/infllmv2_hip.h"
+#include "infllmv2_hip.h"
 #include <math.h>
 
 namespace IV2_NS {

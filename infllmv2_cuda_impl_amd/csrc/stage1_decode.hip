@@ -22,7 +22,7 @@
 //      same operands, same bits).
 // Keys can be packed (cu_seqlens) or lie in per-sequence caches (batch stride + lengths).
 #include "common.h"
-#include "../../include/infllmv2_hip.h"
+#include "infllmv2_hip.h"
 #include <math.h>
 
 namespace IV2_NS {

@@ -20,7 +20,7 @@
 #include "kv_image.h"
 #include "block_walker.h"
 #include "stage2_bwd.h"
-#include "../../include/infllmv2_hip.h"
+#include "infllmv2_hip.h"
 #include <math.h>
 #include <stdlib.h>
 

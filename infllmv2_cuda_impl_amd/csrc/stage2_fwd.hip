@@ -1,5 +1,5 @@
-// Stage-2 block-sparse flash-attention forward for gfx950 (bf16, head_dim 128, 16 query heads
-// per KV head).
+// Stage-2 block-sparse flash-attention forward for gfx950 (head_dim 128, up to 16 query heads per KV head): the
+// K/V image pre-pass and the C entry point; the attention kernel itself is in stage2_fwd_hybrid.hip.
 //
 // Semantics follow compute_attn_1rowblock (csrc/flash_attn/src/flash_fwd_kernel.h:137-602) with
 // the bitmask walk of flash_blockmask.h:5-100: token i of a sequence attends key t iff
@@ -17,9 +17,8 @@
 #include "kv_image.h"
 #include "block_walker.h"
 #include "stage2_fwd.h"
-#include "../../include/infllmv2_hip.h"
+#include "infllmv2_hip.h"
 #include <math.h>
-#include <stdlib.h>
 
 namespace IV2_NS {
 
@@ -96,136 +95,6 @@ void pack_kv_kernel(const PackParams p) {
             }
             *reinterpret_cast<uint4*>(dst + img_off + u * 8) = make_uint4(w[0], w[1], w[2], w[3]);
         }
-    }
-}
-
-// ---------------------------------------------------------------------------------------------
-// forward
-// ---------------------------------------------------------------------------------------------
-template <bool kCausal>
-__global__ __launch_bounds__(256)
-void stage2_fwd_kernel(const FwdParams p) {
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const int b = blockIdx.y, h = blockIdx.z;
-    const int i = blockIdx.x * 4 + wave;                        // token inside the sequence
-    const int q0 = p.cu_seqlens_q[b];
-    const int Sq = p.cu_seqlens_q[b + 1] - q0;
-    if (i >= Sq) return;                                        // uniform per wavefront; no barriers in this kernel
-    const int k0 = p.cu_seqlens_k[b];
-    const int Sk = p.cu_seqlens_k[b + 1] - k0;
-    const int64_t tok = static_cast<int64_t>(q0) + i;
-    const int n = lane & 15, g = lane >> 4;
-
-    const int nq = n < p.group ? n : p.group - 1;               // rows beyond the group repeat its last head and are never stored
-    const elem_bits* qp = p.q + tok * p.q_tok_stride + h * p.q_kvh_stride + nq * p.q_grp_stride + 8 * g;
-    elem8 qf[4];
-#pragma unroll
-    for (int c = 0; c < 4; ++c) qf[c] = *reinterpret_cast<const elem8*>(qp + 32 * c);
-
-    int last_key = kCausal ? (i + Sk - Sq) : (Sk - 1);          // largest allowed key index
-    if (last_key > Sk - 1) last_key = Sk - 1;
-    const int last_blk = last_key < 0 ? -1 : (last_key >> 6);
-
-    BlockWalker walk;
-    walk.init(p.mask ? p.mask + (static_cast<int64_t>(h) * p.total_q + tok) * p.n64 : nullptr, p.n64, last_blk);
-
-    const int64_t img0 = (static_cast<int64_t>(h) * p.n_slots + image_slot0(p.cu_seqlens_k, b)) * kImageElems;
-    const elem_bits* kimg = p.kimg + img0 + lane * 8;
-    const elem_bits* vimg = p.vimg + img0 + lane * 8;
-
-    float m = -INFINITY, l = 0.f;
-    floatx4 o[8];
-#pragma unroll
-    for (int dt = 0; dt < 8; ++dt) o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
-
-    elem8 kreg[16], vreg[16];
-    int j = walk.next();
-    if (j >= 0) {
-        const elem_bits* src = kimg + static_cast<int64_t>(j) * kImageElems;
-#pragma unroll
-        for (int f = 0; f < 16; ++f) kreg[f] = *reinterpret_cast<const elem8*>(src + f * 512);
-    }
-    while (j >= 0) {
-        {
-            const elem_bits* src = vimg + static_cast<int64_t>(j) * kImageElems;
-#pragma unroll
-            for (int f = 0; f < 16; ++f) vreg[f] = *reinterpret_cast<const elem8*>(src + f * 512);
-        }
-        floatx4 s[4];
-#pragma unroll
-        for (int kt = 0; kt < 4; ++kt) {
-            s[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int c = 0; c < 4; ++c)
-                s[kt] = IV2_MFMA(kreg[kt * 4 + c], qf[c], s[kt], 0, 0, 0);
-        }
-        const int jn = walk.next();
-        if (jn >= 0) {
-            const elem_bits* src = kimg + static_cast<int64_t>(jn) * kImageElems;
-#pragma unroll
-            for (int f = 0; f < 16; ++f) kreg[f] = *reinterpret_cast<const elem8*>(src + f * 512);
-        }
-        if (j == last_blk) {                                    // only the last allowed block needs element masking
-            const int lim = last_key - j * kBlockN;              // keys with in-block index > lim are masked
-#pragma unroll
-            for (int kt = 0; kt < 4; ++kt)
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    if (16 * kt + 4 * g + e > lim) s[kt][e] = -INFINITY;
-        }
-        float mx = -INFINITY;
-#pragma unroll
-        for (int kt = 0; kt < 4; ++kt)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) mx = fmaxf(mx, s[kt][e]);
-        mx = wave_max_over_g(mx);
-        const float m_new = fmaxf(m, mx * p.scale_log2);
-        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = __builtin_amdgcn_exp2f(m - m_use);
-        float rs = 0.f;
-#pragma unroll
-        for (int kt = 0; kt < 4; ++kt)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const float pv = __builtin_amdgcn_exp2f(s[kt][e] * p.scale_log2 - m_use);
-                s[kt][e] = pv;
-                rs += pv;
-            }
-        l = l * alpha + rs;
-        m = m_new;
-#pragma unroll
-        for (int dt = 0; dt < 8; ++dt) o[dt] *= alpha;
-        elem8 pf[2];
-#pragma unroll
-        for (int cc = 0; cc < 2; ++cc)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                pf[cc][e] = static_cast<elem_t>(s[2 * cc][e]);
-                pf[cc][4 + e] = static_cast<elem_t>(s[2 * cc + 1][e]);
-            }
-#pragma unroll
-        for (int dt = 0; dt < 8; ++dt)
-#pragma unroll
-            for (int cc = 0; cc < 2; ++cc)
-                o[dt] = IV2_MFMA(vreg[dt * 2 + cc], pf[cc], o[dt], 0, 0, 0);
-        j = jn;
-    }
-
-    const float l_tot = wave_sum_over_g(l);
-    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-    if (n >= p.group) return;
-    elem_bits* op = p.out + tok * p.o_tok_stride + h * p.o_kvh_stride + n * p.o_grp_stride + 4 * g;
-#pragma unroll
-    for (int dt = 0; dt < 8; ++dt) {
-        uint2 w;
-        w.x = pack_elem2(o[dt][0] * inv, o[dt][1] * inv);
-        w.y = pack_elem2(o[dt][2] * inv, o[dt][3] * inv);
-        *reinterpret_cast<uint2*>(op + 16 * dt) = w;
-    }
-    if (g == 0) {
-        const float lse = l_tot > 0.f ? m * 0.69314718055994530942f + logf(l_tot) : INFINITY;
-        p.lse[h * p.lse_kvh_stride + tok * p.lse_tok_stride + n * p.lse_grp_stride] = lse;
     }
 }
 
@@ -328,14 +197,5 @@ extern "C" int IV2_ENTRY(infllmv2_varlen_fwd)(void* stream, const void* q, const
     fp.group = num_heads / num_heads_k;
     fp.n64 = n_uint64_per_row;
     fp.scale_log2 = softmax_scale * 1.44269504088896340736f;
-    static const bool per_token = [] {                         // diagnostic switch: the one-wavefront-per-token kernel
-        const char* e = getenv("INFLLMV2_FWD_PER_TOKEN");
-        return e != nullptr && e[0] == '1';
-    }();
-    if (!per_token) return launch_stage2_fwd_hybrid(st, fp, batch, num_heads_k, max_seqlen_q, max_seqlen_k, is_causal != 0);
-    const dim3 grid((max_seqlen_q + 3) / 4, batch, num_heads_k);
-    if (is_causal) hipLaunchKernelGGL(stage2_fwd_kernel<true>, grid, dim3(256), 0, st, fp);
-    else hipLaunchKernelGGL(stage2_fwd_kernel<false>, grid, dim3(256), 0, st, fp);
-    IV2_LAUNCH_CHECK();
-    return 0;
+    return launch_stage2_fwd_hybrid(st, fp, batch, num_heads_k, max_seqlen_q, max_seqlen_k, is_causal != 0);
 }

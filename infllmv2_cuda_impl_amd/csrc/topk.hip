@@ -25,7 +25,7 @@
 //    counting in LDS.  Index order (ascending column) needs no ordering step at all;
 //  * the next row's scores are requested before the current row's search starts.
 #include "common.h"
-#include "../../include/infllmv2_hip.h"
+#include "infllmv2_hip.h"
 
 namespace infllmv2 {
 

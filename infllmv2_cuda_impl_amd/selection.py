@@ -88,7 +88,8 @@ def compress_keys_cache(k_cache: torch.Tensor, new_lens: torch.Tensor, kernel_si
     ``(batch, capacity, nheads_k, d)`` holds ``new_lens[b]`` keys of sequence b; rows of ``out``
     ``(batch, rows, nheads_k, d)`` whose windows were completed since ``old_lens[b]`` tokens (``None``: all of them)
     are written in place.  ``max_new_rows`` bounds the new rows per sequence (default: every row of ``out``; 1 suffices
-    for a one-token step).  Returns ``out_lens`` int32 ``(batch,)``: the rows each compressed cache now holds."""
+    for a one-token step).  Returns ``out_lens`` int32 ``(batch,)``: the rows each compressed cache now holds - never
+    more than ``out`` has rows or than this call covered (the kernels get both capacities and write nothing beyond)."""
     require_gpu(k_cache, "k_cache")
     if k_cache.dtype not in (torch.float16, torch.bfloat16) or out.dtype != k_cache.dtype:
         raise RuntimeError("FlashAttention only support fp16 and bf16 data type")
@@ -100,17 +101,19 @@ def compress_keys_cache(k_cache: torch.Tensor, new_lens: torch.Tensor, kernel_si
     for name, t in (("new_lens", new_lens), ("old_lens", old_lens)):
         if t is not None and (t.dtype != torch.int32 or tuple(t.shape) != (batch,) or not t.is_contiguous()):
             raise RuntimeError(f"{name} must be a contiguous int32 tensor of shape (batch_size)")
-    if (cap - kernel_size) // stride + 1 > out.shape[1] and max_new_rows is None:
-        raise RuntimeError("out has fewer rows than the key cache has windows")
     if max_new_rows is None:
+        if (cap - kernel_size) // stride + 1 > out.shape[1]:
+            raise RuntimeError("out has fewer rows than the key cache has windows")
         max_new_rows = out.shape[1]
+    elif max_new_rows < 0:
+        raise RuntimeError("max_new_rows must not be negative")
     if out_lens is None:
         out_lens = torch.empty(batch, dtype=torch.int32, device=k_cache.device)
     s3 = lambda t: _lib.i64_array([t.stride(0), t.stride(1), t.stride(2)])
     with torch.cuda.device(k_cache.device):
         _lib.call_for(k_cache.dtype, "infllmv2_compress_keys_cache", stream_ptr(k_cache.device), k_cache.data_ptr(), out.data_ptr(),
                   None if old_lens is None else old_lens.data_ptr(), new_lens.data_ptr(), out_lens.data_ptr(), batch,
-                  int(max_new_rows), Hk, d, s3(k_cache), s3(out), kernel_size, stride)
+                  int(max_new_rows), Hk, d, s3(k_cache), s3(out), kernel_size, stride, cap, out.shape[1])
     return out_lens
 
 

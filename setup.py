@@ -21,6 +21,12 @@ class BuildWithHip(build_py):
         mod = importlib.util.module_from_spec(spec)
         spec.loader.exec_module(mod)
         mod.build(verbose=True)
+        # the sources include the C-ABI header by name: ship a copy inside the package so that an installed copy
+        # can be rebuilt without the repository root
+        import shutil
+        dst = os.path.join(ROOT, "infllmv2_cuda_impl_amd", "include")
+        os.makedirs(dst, exist_ok=True)
+        shutil.copy2(os.path.join(ROOT, "include", "infllmv2_hip.h"), os.path.join(dst, "infllmv2_hip.h"))
         super().run()
 
 
@@ -29,7 +35,7 @@ setup(
     version="0.1.0",
     description="InfLLM-V2 two-stage sparse attention for AMD MI355X (gfx950): hand-written HIP kernels behind a C ABI",
     packages=["infllmv2_cuda_impl_amd", "infllm_v2"],
-    package_data={"infllmv2_cuda_impl_amd": ["libinfllmv2_hip.so", "csrc/*.hip", "csrc/*.h", "csrc/build.py"]},
+    package_data={"infllmv2_cuda_impl_amd": ["libinfllmv2_hip.so", "csrc/*.hip", "csrc/*.h", "csrc/build.py", "include/*.h"]},
     include_package_data=True,
     python_requires=">=3.9",
     cmdclass={"build_py": BuildWithHip},

@@ -67,6 +67,10 @@ def test_new_entry_points_validate_before_launch():
     assert rc != 0 and "must be positive" in _err(lib)
     rc = lib.infllmv2_compress_keys(None, None, fake, fake, fake, 1, 128, 2, 128, 256, 128, 32, 16, 0)
     assert rc != 0 and "null pointer" in _err(lib)
+    # compressed-key caches: the row capacities are arguments of the entry point and are checked before any launch
+    rc = lib.infllmv2_compress_keys_cache(None, fake, fake, None, fake, None, 2, 1, 2, 128, i64([262144, 256, 128]),
+                                          i64([16384, 256, 128]), 32, 16, 1024, -1)
+    assert rc != 0 and "negative cache capacity" in _err(lib)
     # decode: option conflicts carry the reference's messages (flash_api.cpp:1596, 1763, 1774)
     def kv(**o):
         a = dict(knew=None, cbi=None, lp=None, bt=None, page=0, cos=None, sin=None, rd=0)

@@ -171,6 +171,36 @@ def test_append_of_a_few_rows_equals_the_full_build(ops, dtype, Hk, d, ks, st, j
     assert torch.equal(inc, full)
 
 
+def test_compressed_cache_capacity_bounds_what_is_written(ops):
+    """An undersized compressed cache, or a step that completes more windows than max_new_rows covers: nothing is
+    written beyond the cache's rows, and out_lens counts only rows the call did write (the kernels get both
+    capacities; the guard rows behind the view stay untouched)."""
+    B, cap, ks, st = 3, 512, 32, 16
+    g = torch.Generator(device="cpu").manual_seed(23)
+    kcache = torch.randn(B, cap, 2, 128, generator=g).to(torch.bfloat16).to(DEV)
+    backing = torch.full((B, 12, 2, 128), 7.0, dtype=torch.bfloat16, device=DEV)
+    out = backing[:, :8]                                       # 8 rows of capacity, 4 guard rows behind each sequence
+    new = torch.tensor([200, 400, 40], dtype=torch.int32, device=DEV)       # 11, 24 and 1 complete windows
+    old = torch.tensor([128, 399, 0], dtype=torch.int32, device=DEV)        # 7, 23 and 0 rows held before
+    rows = ops.compress_keys_cache(kcache, new, ks, st, out=out, old_lens=old, max_new_rows=1)
+    assert [int(r) for r in rows] == [8, 8, 1]                 # 7 + 1; nothing fits (23 >= 8 rows): the capacity; 0 + 1
+    assert bool((backing[:, 8:] == 7.0).all())
+    ref0, _ = ops.compress_keys(kcache[0, :200], torch.tensor([0, 200], dtype=torch.int32, device=DEV), 200, ks, st)
+    assert torch.equal(out[0, 7], ref0[7]) and bool((out[0, :7] == 7.0).all())
+    assert bool((out[1] == 7.0).all())
+    # a jump of several windows with max_new_rows = 2: two rows written, two reported
+    rows = ops.compress_keys_cache(kcache, torch.tensor([200, 0, 0], dtype=torch.int32, device=DEV), ks, st, out=out,
+                                   old_lens=torch.tensor([32, 0, 0], dtype=torch.int32, device=DEV), max_new_rows=2)
+    assert [int(r) for r in rows] == [3, 0, 0]
+    assert torch.equal(out[0, 1:3], ref0[1:3]) and bool((out[0, 3:7] == 7.0).all())
+    # a length beyond the key cache is read as the capacity
+    big = torch.full((B, 40, 2, 128), 7.0, dtype=torch.bfloat16, device=DEV)
+    rows = ops.compress_keys_cache(kcache, torch.tensor([9999, 0, 0], dtype=torch.int32, device=DEV), ks, st, out=big)
+    assert int(rows[0]) == (cap - ks) // st + 1
+    with pytest.raises(RuntimeError, match="fewer rows"):
+        ops.compress_keys_cache(kcache, new, ks, st, out=out)
+
+
 def test_batched_decode_steps_equal_single_sequence_decode(ops):
     """decode_batch on sequences of different lengths == the single-sequence decode loop run on each of them: same
     caches afterwards (bit for bit), outputs to the Stage-2 tolerance (the two paths cut the compressed keys into
