@@ -97,6 +97,78 @@ def test_config2_prefill_32k(ops):
         assert err.max() <= 2e-2 and err.mean() <= 1e-3, (r, err.max(), err.mean())
 
 
+def test_config3_selection_64k(ops):
+    """The selection leg at BASELINE config 3: four packed sequences (the lengths of the test below), compressed keys,
+    packed Stage 1, varlen pooling, top-k and mask words.  Stage-1 rows of sampled tokens of every sequence (first,
+    last, the pair across each sequence boundary, mid-sequence) against the oracle of the token's own sequence; pooled
+    scores, indices and mask words of those rows bit-exact functions of the GPU's score rows; invariants over all
+    rows; the fused front end bit-identical to the chain of separate calls."""
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(1)
+    lens = [int(64 * x) for x in rng.integers(64, 385, size=4)]
+    T, topk = sum(lens), 64
+    cu_l = np.cumsum([0] + lens).astype(np.int32)
+    cu = torch.from_numpy(cu_l).to(dev)
+    g = torch.Generator(device="cpu").manual_seed(0)
+    q = torch.randn(T, 32, 128, generator=g).to(torch.bfloat16).to(dev)
+    k = torch.randn(T, 2, 128, generator=g).to(torch.bfloat16).to(dev)
+    kf, cu_f = ops.compress_keys(k, cu, max(lens), 32, 16)
+    kc, cu_c = ops.compress_keys(k, cu, max(lens), 128, 64)
+    cf, cc = cu_f.cpu().numpy(), cu_c.cpu().numpy()
+    for b in range(4):                                         # compressed keys of every sequence == its own unfold/mean
+        seg = k[cu_l[b]:cu_l[b + 1]]
+        assert torch.equal(kf[cf[b]:cf[b + 1]], compress(seg, 32, 16)) and torch.equal(kc[cc[b]:cc[b + 1]], compress(seg, 128, 64))
+    max_lk = int(np.diff(cf).max())
+    score = ops.infllmv2_attn_stage1(q, kf, kc, cu, cu_f, cu_c, max(lens), max_lk, causal=True)
+    zeros = torch.zeros(4, dtype=torch.int32, device=dev)
+    pooled = ops.max_pooling_1d_varlen(score, cu, cu_f, zeros, max(lens), max_lk, 31, 1)
+    idx = ops.topk_blocks(pooled, topk)
+    words, kb = ops.topk_to_uint64(idx, max(lens), 64)
+    samples = []                                               # (sequence, local token)
+    for b in range(4):
+        samples += [(b, 0), (b, 1), (b, lens[b] - 1), (b, lens[b] // 2 + 7), (b, 4095), (b, min(4096, lens[b] - 2))]
+    rows = [int(cu_l[b]) + t for b, t in samples]
+    loc = np.array([t for _, t in samples])
+    lk_row = np.array([cf[b + 1] - cf[b] for b, _ in samples])
+    sc = bf16_np(score[:, rows])
+    nblk = (max(lens) + 63) // 64
+    ref_pool = O.max_pooling_1d_fast(sc, nblk, 31, 1, row_cache_lens=np.zeros(len(rows), dtype=np.int64), row_qidx=loc,
+                                     row_klen=lk_row)
+    assert np.array_equal(bf16_np(pooled[:, rows]), ref_pool)
+    ref_idx = O.topk_blocks(ref_pool, topk)
+    assert np.array_equal(idx[:, rows].cpu().numpy(), ref_idx)
+    assert np.array_equal(words_np(words[:, rows]), O.topk_to_uint64(ref_idx, max(lens), 64)[0])
+    # Stage 1 of the sampled rows against the oracle restricted to the token's own sequence
+    kf_np, kc_np = bf16_np(kf), bf16_np(kc)
+    for (b, t), r in zip(samples, rows):
+        Lk, Lc = int(cf[b + 1] - cf[b]), int(cc[b + 1] - cc[b])
+        vf = O.stage1_visible(t, 16, Lk, lens[b], True)
+        vc = O.stage1_visible(t, 64, Lc, lens[b], True)
+        got = bf16_np(score[:, r])
+        if vc == 0:
+            assert np.all(got == 0), (b, t)
+            continue
+        qq = bf16_np(q[r]).reshape(2, 16, 128).astype(np.float64)
+        for h in range(2):
+            sc_c = qq[h] @ kc_np[cc[b]:cc[b] + vc, h].astype(np.float64).T * 128 ** -0.5
+            lse = np.log(np.exp(sc_c - sc_c.max(-1, keepdims=True)).sum(-1, keepdims=True)) + sc_c.max(-1, keepdims=True)
+            ref = np.exp(qq[h] @ kf_np[cf[b]:cf[b] + vf, h].astype(np.float64).T * 128 ** -0.5 - lse).sum(0)
+            assert (np.abs(got[h, :vf] - ref) <= 2.0 ** -7 * np.abs(ref) + 2e-3).all(), (b, t, h)
+            assert np.all(got[h, vf:] == 0), (b, t, h)
+    # invariants over all rows: block 0 and the local window always selected, nothing from the token's future
+    bits = ops.uint64_to_bool(words, kb)
+    local_tok = torch.cat([torch.arange(n, device=dev) for n in lens])
+    bq = local_tok // 64
+    rows_all = torch.arange(T, device=dev)
+    assert bool(bits[:, :, 0].all())
+    assert bool((bits.sum(-1) == topk).all())
+    for d in (0, 1, 15, 31):
+        assert bool(bits[:, rows_all, torch.clamp(bq - d, min=0)].all())
+    # the one-call front end selects the same blocks, bit for bit, without writing the score tensor
+    fused = ops.select_blocks(q, k, cu, cu, max(lens), max(lens), topk, 31, 1, cache_lens=zeros, max_cache_len=0)
+    assert torch.equal(fused, idx)
+
+
 def test_config3_varlen_fwd_bwd_64k(ops, monkeypatch):
     dev = torch.device("cuda:0")
     rng = np.random.default_rng(1)
