@@ -12,11 +12,13 @@
 // Shape of the work: per sequence and KV head the whole compressed-key set is read once (256 bytes per key) for 16
 // query rows, so the launch is bound by memory bandwidth and the stage1.hip kernel (one workgroup per 16 tokens,
 // keys staged for reuse by 16 tokens) is the wrong shape: it would stream every sequence through one workgroup.
-// Here the keys of one (sequence, KV head) are cut into runs of 64-key tiles and every run goes to a
-// single-wavefront workgroup that loads its tiles straight into MFMA operand registers (two tiles in flight).
+// Here the keys of one (sequence, KV head) are cut into runs of 64-key tiles, the same run length (two tiles unless
+// the longest sequence would then need more than 64 runs) for every sequence of the batch, and every run goes to a
+// single-wavefront workgroup that loads its tiles straight into MFMA operand registers: long sequences get many
+// workgroups, short ones few, and every workgroup carries the same load.
 // The log-sum-exp needs all coarse keys before any score can be normalised, so there are two launches:
 //   1. stage1_decode_lse_kernel: per run of coarse tiles the running (max, sum) of the 16 heads -> workspace;
-//   2. stage1_decode_score_kernel: merges the partials of its (sequence, head) in run order, then scores its run of
+//   2. stage1_decode_score_kernel: merges the partials of its (sequence, head) (16 lanes in parallel), then scores its run of
 //      fine tiles and writes either the score row or its pooling onto key blocks.  A pooled block needs the last
 //      key of the tile before the run: that one 16-key group is scored again by the run that needs it (same MFMA,
 //      same operands, same bits).
@@ -46,7 +48,8 @@ struct S1DecodeParams {
     float scale_log2;
     int causal;
     int group;                       // query heads per KV head, 1..16: MFMA rows >= group repeat head group - 1 and add nothing
-    int splits_c, splits_f;
+    int splits_c, splits_f;          // runs the longest sequence is cut into (grid size; record slots per pair)
+    int run_c, run_f;                // tiles per run
     // pooled output
     const int* cache_lens;           // per sequence, or null: cache_len for all
     int cache_len;
@@ -101,15 +104,14 @@ __device__ __forceinline__ void s1d_load_q(elem8 (&qf)[4], const S1DecodeParams&
     for (int c = 0; c < 4; ++c) qf[c] = *reinterpret_cast<const elem8*>(qp + 32 * c);
 }
 
-// run [t0, t1) of `tiles` tiles that split `split` of `splits` works on
-__device__ __forceinline__ void s1d_run(int tiles, int splits, int split, int& t0, int& t1) {
-    const int per = (tiles + splits - 1) / splits;
+// run [t0, t1) of `tiles` tiles that split `split` works on: runs of `per` tiles, the same length for every sequence
+// of the batch (a long sequence has many runs, a short one few: every wavefront gets the same amount of work)
+__device__ __forceinline__ void s1d_run_fixed(int tiles, int per, int split, int& t0, int& t1) {
     t0 = split * per;
     t0 = t0 < tiles ? t0 : tiles;
     t1 = t0 + per;
     t1 = t1 < tiles ? t1 : tiles;
 }
-
 // (max, sum) in log2 units of head 4g + e over the coarse tiles [t0, t1) of one sequence and KV head, merged over the
 // 16 key-column lanes: every lane of row g returns the values of its four heads.
 __device__ __forceinline__ void s1d_lse_run(const S1DecodeParams& p, const S1DecodeSeq& sq, const elem8 (&qf)[4], int vis_c,
@@ -176,16 +178,30 @@ __device__ __forceinline__ void s1d_lse_run(const S1DecodeParams& p, const S1Dec
     }
 }
 
-// log-sum-exp (log2 units) of head 4g + e from `count` partial records {max x 16, sum x 16} merged in order
-__device__ __forceinline__ void s1d_merge_partials(const float* part, int count, int g, int group, float (&lse2)[4]) {
+// log-sum-exp (log2 units) of head 4g + e from `count` partial records {max x 16, sum x 16}: lane (n, g) merges the
+// records n, n + 16, ... for its four heads, then the 16 lanes of a row merge among themselves (the merge of (max,
+// sum) pairs is associative and commutative up to rounding, and every lane of a row ends with the same bits because
+// the butterfly combines the same pairs in the same order on both sides).
+__device__ __forceinline__ void s1d_merge_partials(const float* part, int count, int n, int g, int group, float (&lse2)[4]) {
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         float mm = -INFINITY, ll = 0.f;
-        for (int s = 0; s < count; ++s) {
+        for (int s = n; s < count; s += 16) {
             const float mo = part[s * 32 + 4 * g + e], lo = part[s * 32 + 16 + 4 * g + e];
             const float mn = fmaxf(mm, mo);
             const float mu = (mn == -INFINITY) ? 0.f : mn;
             ll = ll * __builtin_amdgcn_exp2f(mm - mu) + lo * __builtin_amdgcn_exp2f(mo - mu);
+            mm = mn;
+        }
+#pragma unroll
+        for (int off = 1; off < 16; off <<= 1) {
+            const float mo = __shfl_xor(mm, off);
+            const float lo = __shfl_xor(ll, off);
+            const float mn = fmaxf(mm, mo);
+            const float mu = (mn == -INFINITY) ? 0.f : mn;
+            // the same sum on both partners: add the term of the lane with the lower number first
+            const float mine = ll * __builtin_amdgcn_exp2f(mm - mu), theirs = lo * __builtin_amdgcn_exp2f(mo - mu);
+            ll = (n & off) ? theirs + mine : mine + theirs;
             mm = mn;
         }
         lse2[e] = mm + __builtin_amdgcn_logf(ll);                // v_log_f32 is log2
@@ -202,7 +218,8 @@ void stage1_decode_lse_kernel(const S1DecodeParams p) {
     const int s1 = (sq.Lk == sq.Lc) ? 16 : 64;                 // flash_fwd_kernel.h:1236-1240
     const int vis_c = s1d_visible(s1, sq.Lc, p.causal != 0);
     int t0, t1;
-    s1d_run((vis_c + 63) >> 6, p.splits_c, split, t0, t1);
+    s1d_run_fixed((vis_c + 63) >> 6, p.run_c, split, t0, t1);
+    if (t0 >= t1 && split > 0) return;                         // beyond this sequence's runs; run 0 always leaves a record
     elem8 qf[4];
     s1d_load_q(qf, p, sq, h, n, g);
     float mm[4], ll[4];
@@ -331,7 +348,7 @@ void stage1_decode_score_kernel(const S1DecodeParams p) {
     int vis_c, vis_f, tiles;
     s1d_fine_extent<kPool>(p, sq, vis_c, vis_f, tiles);
     int t0, t1;
-    s1d_run(tiles, p.splits_f, split, t0, t1);
+    s1d_run_fixed(tiles, p.run_f, split, t0, t1);
     const bool owns_tail = tiles == 0 ? split == 0 : (t0 < t1 && t1 == tiles);
     if (t0 >= t1 && !owns_tail) return;
 
@@ -343,52 +360,9 @@ void stage1_decode_score_kernel(const S1DecodeParams p) {
     if (t0 + 1 < t1) s1d_load_tile(tb, sq.kbase, p.k_row_stride, (t0 + 1) * 64, sq.Lk, n, g);
     // log-sum-exp of head 4g + e: the partials of the coarse runs merged in run order
     float lse2[4];
-    s1d_merge_partials(p.partial + (static_cast<int64_t>(b) * gridDim.y + h) * p.splits_c * 32, p.splits_c, g, p.group, lse2);
-    s1d_score_run<kPool>(p, sq, qf, lse2, ta, tb, vis_f, tiles, t0, t1, owns_tail, b, h, lane);
-}
-
-// Both passes in one launch, for batches with enough (sequence, KV head) pairs to fill the device without splitting a
-// pair over more than a few workgroups: a workgroup of 8 wavefronts splits ALL coarse tiles of its pair among its
-// wavefronts, merges their (max, sum) records through LDS, and then scores its part of the fine tiles, one run per
-// wavefront.  With `parts` workgroups per pair the coarse keys are read `parts` times (the repeats come from L2), which
-// is why this form is only used for parts <= 4; it saves the second launch and the trip of the records through memory.
-constexpr int kS1dFusedWaves = 8;
-template <bool kPool>
-__global__ __launch_bounds__(64 * kS1dFusedWaves)
-void stage1_decode_fused_kernel(const S1DecodeParams p) {
-    __shared__ float records[kS1dFusedWaves * 32];
-    const int lane = threadIdx.x & 63, n = lane & 15, g = lane >> 4;
-    const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
-    const int part = blockIdx.x, parts = gridDim.x, h = blockIdx.y, b = blockIdx.z;
-    const S1DecodeSeq sq = s1d_sequence(p, b, h);
-    if (sq.Sq <= 0) return;                                    // uniform per workgroup
-    int vis_c, vis_f, tiles;
-    s1d_fine_extent<kPool>(p, sq, vis_c, vis_f, tiles);
-    const int split = part * kS1dFusedWaves + wave, splits = parts * kS1dFusedWaves;
-    int t0, t1;
-    s1d_run(tiles, splits, split, t0, t1);
-    const bool owns_tail = tiles == 0 ? split == 0 : (t0 < t1 && t1 == tiles);
-
-    elem8 qf[4];
-    s1d_load_q(qf, p, sq, h, n, g);
-    {
-        int c0, c1;
-        s1d_run((vis_c + 63) >> 6, kS1dFusedWaves, wave, c0, c1);
-        float mm[4], ll[4];
-        s1d_lse_run(p, sq, qf, vis_c, c0, c1, n, g, mm, ll);
-        if (n == 0) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) { records[wave * 32 + 4 * g + e] = mm[e]; records[wave * 32 + 16 + 4 * g + e] = ll[e]; }
-        }
-    }
-    // the first two fine tiles are on their way while the records are exchanged
-    elem8 ta[16], tb[16];
-    if (t0 < t1) s1d_load_tile(ta, sq.kbase, p.k_row_stride, t0 * 64, sq.Lk, n, g);
-    if (t0 + 1 < t1) s1d_load_tile(tb, sq.kbase, p.k_row_stride, (t0 + 1) * 64, sq.Lk, n, g);
-    __syncthreads();
-    if (t0 >= t1 && !owns_tail) return;                        // per wavefront, after the only barrier
-    float lse2[4];
-    s1d_merge_partials(records, kS1dFusedWaves, g, p.group, lse2);
+    int records = (((vis_c + 63) >> 6) + p.run_c - 1) / p.run_c;                    // the coarse runs of this sequence
+    records = records < 1 ? 1 : records;
+    s1d_merge_partials(p.partial + (static_cast<int64_t>(b) * gridDim.y + h) * p.splits_c * 32, records, n, g, p.group, lse2);
     s1d_score_run<kPool>(p, sq, qf, lse2, ta, tb, vis_f, tiles, t0, t1, owns_tail, b, h, lane);
 }
 
@@ -398,28 +372,26 @@ using namespace IV2_NS;
 
 namespace {
 
-// runs per (sequence, KV head): enough single-wavefront workgroups to keep ~8 per CU of a 256-CU device in flight,
-// but no run shorter than two tiles of the longest sequence
-void s1d_splits(int batch, int num_heads_k, int max_keys, int max_coarse, int& splits_f, int& splits_c) {
-    const int pairs = batch * num_heads_k > 0 ? batch * num_heads_k : 1;
-    int want = (2048 + pairs - 1) / pairs;
-    auto clamp_to = [&](int tiles) {
-        int s = want;
-        const int cap = (tiles + 1) / 2;
-        if (s > cap) s = cap;
-        if (s > 64) s = 64;
-        return s < 1 ? 1 : s;
+// Runs of the two-launch form: every run is `run` tiles long whatever its sequence's length, so the single-wavefront
+// workgroups all carry the same load; the longest sequence is cut into at most 64 runs.
+void s1d_splits(int batch, int num_heads_k, int max_keys, int max_coarse, int& splits_f, int& splits_c, int& run_f, int& run_c) {
+    (void)batch; (void)num_heads_k;
+    auto plan = [&](int tiles, int want_run, int& splits, int& run) {
+        run = want_run;
+        if ((tiles + run - 1) / run > 64) run = (tiles + 63) / 64;
+        splits = (tiles + run - 1) / run;
+        if (splits < 1) splits = 1;
     };
-    splits_f = clamp_to((max_keys + 63) / 64);
-    splits_c = clamp_to((max_coarse + 63) / 64);
+    plan((max_keys + 63) / 64, 2, splits_f, run_f);
+    plan((max_coarse + 63) / 64, 2, splits_c, run_c);
 }
 
 }  // namespace
 
 #ifndef IV2_F16        // element-type independent: defined once
 extern "C" size_t infllmv2_stage1_decode_workspace_bytes(int batch, int num_heads_k, int max_seqlen_k, int max_seqlen_v) {
-    int sf, sc;
-    s1d_splits(batch, num_heads_k, max_seqlen_k, max_seqlen_v, sf, sc);
+    int sf, sc, rf, rc;
+    s1d_splits(batch, num_heads_k, max_seqlen_k, max_seqlen_v, sf, sc, rf, rc);
     return static_cast<size_t>(batch > 0 ? batch : 0) * (num_heads_k > 0 ? num_heads_k : 0) * sc * 32 * sizeof(float);
 }
 #endif
@@ -457,7 +429,7 @@ extern "C" int IV2_ENTRY(infllmv2_stage1_decode)(void* stream, const void* q, co
         IV2_CHECK(out_row_stride >= max_seqlen_k, "%s: score row stride shorter than max_seqlen_k", who);
     }
     S1DecodeParams p{};
-    s1d_splits(batch, num_heads_k, max_seqlen_k, max_seqlen_v, p.splits_f, p.splits_c);
+    s1d_splits(batch, num_heads_k, max_seqlen_k, max_seqlen_v, p.splits_f, p.splits_c, p.run_f, p.run_c);
     IV2_CHECK(workspace != nullptr && reinterpret_cast<uintptr_t>(workspace) % 16 == 0 &&
               workspace_bytes >= infllmv2_stage1_decode_workspace_bytes(batch, num_heads_k, max_seqlen_k, max_seqlen_v),
               "%s: workspace missing, misaligned or too small", who);
@@ -480,21 +452,6 @@ extern "C" int IV2_ENTRY(infllmv2_stage1_decode)(void* stream, const void* q, co
     p.cache_lens = cache_lens; p.cache_len = cache_len; p.pool_len = out_len;
     p.local_blocks = local_blocks; p.init_blocks = init_blocks;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    // enough pairs to fill the device with at most 4 workgroups of 8 wavefronts per pair: both passes in one launch
-    const int pairs = batch * num_heads_k;
-    if (pairs >= 64) {
-        int parts = (256 + pairs - 1) / pairs;
-        const int tiles_max = (max_seqlen_k + 63) / 64;
-        const int cap = (tiles_max + 2 * kS1dFusedWaves - 1) / (2 * kS1dFusedWaves);    // no run shorter than two tiles of the longest sequence
-        if (parts > cap) parts = cap;
-        if (parts > 4) parts = 4;
-        if (parts < 1) parts = 1;
-        const dim3 fgrid(parts, num_heads_k, batch);
-        if (pooled) hipLaunchKernelGGL(stage1_decode_fused_kernel<true>, fgrid, dim3(64 * kS1dFusedWaves), 0, st, p);
-        else hipLaunchKernelGGL(stage1_decode_fused_kernel<false>, fgrid, dim3(64 * kS1dFusedWaves), 0, st, p);
-        IV2_LAUNCH_CHECK();
-        return 0;
-    }
     hipLaunchKernelGGL(stage1_decode_lse_kernel, dim3(p.splits_c, num_heads_k, batch), dim3(64), 0, st, p);
     IV2_LAUNCH_CHECK();
     const dim3 grid(p.splits_f, num_heads_k, batch);
