@@ -81,5 +81,36 @@ def build(verbose: bool = True, jobs: int | None = None) -> str:
     return LIB_PATH
 
 
+TORCH_MODULE = "_C"
+
+
+def torch_module_path() -> str:
+    import sysconfig
+    return os.path.join(PKG, TORCH_MODULE + (sysconfig.get_config_var("EXT_SUFFIX") or ".so"))
+
+
+def build_torch_module(verbose: bool = True) -> str:
+    """Compiles csrc/torch_module.cpp, the native module `infllmv2_cuda_impl_amd._C` (`infllm_v2.C`): host code only
+    (pybind11 + ATen for tensors and the current stream) that links against libinfllmv2_hip.so beside it."""
+    import sysconfig
+    import torch
+    from torch.utils import cpp_extension as ce
+    out = torch_module_path()
+    torch_lib = ce.library_paths()[0]
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           f"-DTORCH_EXTENSION_NAME={TORCH_MODULE}", f"-D_GLIBCXX_USE_CXX11_ABI={int(torch.compiled_with_cxx11_abi())}",
+           *[f"-I{d}" for d in ce.include_paths()], "-I", sysconfig.get_paths()["include"], "-I", "/opt/rocm/include",
+           "-I", include_dir(), os.path.join(CSRC, "torch_module.cpp"), "-o", out,
+           f"-L{torch_lib}", "-ltorch", "-ltorch_cpu", "-ltorch_python", "-lc10", "-lc10_hip", f"-L{PKG}", "-linfllmv2_hip",
+           "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{torch_lib}"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("building the torch module failed:\n" + r.stderr)
+    if verbose:
+        print(f"built {out}")
+    return out
+
+
 if __name__ == "__main__":
     build()
+    build_torch_module()

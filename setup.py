@@ -21,6 +21,7 @@ class BuildWithHip(build_py):
         mod = importlib.util.module_from_spec(spec)
         spec.loader.exec_module(mod)
         mod.build(verbose=True)
+        mod.build_torch_module(verbose=True)
         # the sources include the C-ABI header by name: ship a copy inside the package so that an installed copy
         # can be rebuilt without the repository root
         import shutil
@@ -35,7 +36,7 @@ setup(
     version="0.1.0",
     description="InfLLM-V2 two-stage sparse attention for AMD MI355X (gfx950): hand-written HIP kernels behind a C ABI",
     packages=["infllmv2_cuda_impl_amd", "infllm_v2"],
-    package_data={"infllmv2_cuda_impl_amd": ["libinfllmv2_hip.so", "csrc/*.hip", "csrc/*.h", "csrc/build.py", "include/*.h"]},
+    package_data={"infllmv2_cuda_impl_amd": ["libinfllmv2_hip.so", "_C*.so", "csrc/*.cpp", "csrc/*.hip", "csrc/*.h", "csrc/build.py", "include/*.h"]},
     include_package_data=True,
     python_requires=">=3.9",
     cmdclass={"build_py": BuildWithHip},

@@ -1,4 +1,5 @@
-"""The mirror of the reference's native module (`infllm_v2.C`) called the way the reference's own Python
+"""The reference's native module (`infllm_v2.C`: the compiled extension `infllmv2_cuda_impl_amd._C`, and its
+pure-Python twin `infllmv2_cuda_impl_amd.C`) called the way the reference's own Python
 wrappers call it (infllm_v2/infllmv2_sparse_attention.py:71-130, 174-263, 551-589, max_pooling_1d.py:25-41,
 topk_to_uint64.py:60-68): re-laid-out (T*16, Hk, d) queries, cu_seqlens * 16, transposed column mask for
 the backward.  Results must equal those of the package operators, which run the same kernels in place."""
@@ -11,6 +12,18 @@ from test_gpu_stage2_fwd import make_case
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(params=["compiled", "python"])
+def C(request):
+    """Both implementations of the native-module interface: the compiled extension is what `infllm_v2.C` resolves to."""
+    if request.param == "compiled":
+        from infllm_v2 import C as mod
+        import infllmv2_cuda_impl_amd._C as ext
+        assert mod.varlen_fwd is ext.varlen_fwd
+        return mod
+    import infllmv2_cuda_impl_amd.C as mod
+    return mod
+
+
 def expand(x, Hk):           # (T, Hq, d) -> (T*16, Hk, d), as infllmv2_sparse_attention.py:88
     T, Hq, d = x.shape
     return x.reshape(T, Hk, 16, d).transpose(1, 2).reshape(T * 16, Hk, d).contiguous()
@@ -21,9 +34,8 @@ def collapse(x, Hk):         # inverse, as infllmv2_sparse_attention.py:130
     return x.reshape(T16 // 16, 16, Hk, d).transpose(1, 2).reshape(T16 // 16, Hk * 16, d).contiguous()
 
 
-def test_reference_style_forward_backward_through_C():
+def test_reference_style_forward_backward_through_C(C):
     import infllm_v2
-    from infllm_v2 import C
     dev = torch.device("cuda:0")
     sq = [300, 200]
     q, k, v, cu_q, cu_k, idx = make_case(21, sq, sq, 2, 3, dev)
@@ -54,9 +66,8 @@ def test_reference_style_forward_backward_through_C():
     assert (dk.float() - kg.grad.float()).abs().max() <= 0.07 and (dv.float() - vg.grad.float()).abs().max() <= 0.13  # fp32 atomics order
 
 
-def test_reference_style_stage1_and_pooling_through_C():
+def test_reference_style_stage1_and_pooling_through_C(C):
     import infllm_v2
-    from infllm_v2 import C
     dev = torch.device("cuda:0")
     S = 640
     g = torch.Generator(device="cpu").manual_seed(5)
@@ -97,11 +108,10 @@ def test_reference_style_stage1_and_pooling_through_C():
 
 
 @pytest.mark.parametrize("causal", [True, False])
-def test_fixed_length_fwd_bwd_through_C(causal):
+def test_fixed_length_fwd_bwd_through_C(C, causal):
     """`C.fwd` / `C.bwd` (mha_fwd / mha_bwd, flash_api.cpp:349-517, 1062-1276): dense attention over a
     (batch, seqlen, heads, d) batch.  Checked against the fp64 oracle per sequence; gradients land in the
     caller's tensors, also when those are not viewable as packed rows."""
-    from infllm_v2 import C
     from oracle import infllmv2_oracle as O
     from conftest import bf16_np
     dev = torch.device("cuda:0")
@@ -131,3 +141,27 @@ def test_fixed_length_fwd_bwd_through_C(causal):
         s = max(1.0, float(np.abs(ref).max()))
         err = np.abs(gnp - ref)
         assert err.max() <= 2e-2 * s and err.mean() <= 1e-3 * s, (name, err.max(), err.mean())
+
+
+def test_decode_through_C(C):
+    """`C.fwd_kvcache` (mha_fwd_kvcache, flash_api.cpp:1549-1843) as infllmv2_sparse_attention.py:730-760 calls it: packed
+    mask words, new keys appended in place, rotary tables.  Equal to the package operator bit for bit (same kernels)."""
+    import infllm_v2
+    import test_gpu_decode as D
+    dev = torch.device("cuda:0")
+    lens = [700, 64, 1000, 333]
+    q, kc, vc, kn, vn, L, idx = D.make(8, 4, 1024, lens, 5, new=2)
+    cos, sin = D.rotary_tables(9, 1024, 32)
+    d = lambda t: t.to(dev)
+    words, _ = infllm_v2.topk_to_uint64(d(idx), 1024, 64)
+    k1, v1, k2, v2 = d(kc).clone(), d(vc).clone(), d(kc).clone(), d(vc).clone()
+    out, lse = C.fwd_kvcache(d(q), k1, v1, d(kn), d(vn), d(L), d(cos), d(sin), None, None, None, None, None, 128 ** -0.5,
+                             False, -1, -1, 0.0, True, 3, words)
+    ref_out, ref_lse = infllm_v2.infllmv2_attn_with_kvcache(d(q), k2, v2, k=d(kn), v=d(vn), rotary_cos=d(cos),
+                                                            rotary_sin=d(sin), cache_seqlens=d(L), topk_idx=d(idx),
+                                                            num_splits=3, return_softmax_lse=True, rotary_interleaved=True)
+    assert torch.equal(out, ref_out) and torch.equal(lse, ref_lse)
+    assert torch.equal(k1, k2) and torch.equal(v1, v2) and not torch.equal(k1, d(kc))
+    with pytest.raises(RuntimeError, match="does not support alibi"):
+        C.fwd_kvcache(d(q), k1, v1, None, None, d(L), None, None, None, None, None, d(L).float(), None, 128 ** -0.5,
+                      False, -1, -1, 0.0, True, 0, words)

@@ -31,3 +31,29 @@ def test_reject_unsupported_returns_the_launch_flag_and_keeps_the_reference_mess
         r(0.5, (-1, -1), 0.0, None, True, 64)
     with pytest.raises(RuntimeError, match="does not support alibi"):
         r(0.0, (-1, -1), 0.0, object(), True, 64)
+
+
+def test_native_module_binds_the_reference_names():
+    """`infllm_v2.C` is the compiled extension and exports what csrc/entry.cu:197-215 binds; argument errors that need
+    no GPU are reported on the host."""
+    import pytest
+    import torch
+    from infllm_v2 import C
+    import infllmv2_cuda_impl_amd._C as ext
+    names = ["topk", "get_probs", "blockmask_to_uint64", "topk_to_uint64", "uint64_to_bool", "max_pooling_1d",
+             "max_pooling_1d_varlen", "fwd", "varlen_fwd", "varlen_fwd_stage1", "bwd", "varlen_bwd", "fwd_kvcache"]
+    for n in names:
+        assert getattr(C, n) is getattr(ext, n), n
+    with pytest.raises(NotImplementedError):
+        C.get_probs()
+    z = lambda *s: torch.zeros(*s, dtype=torch.bfloat16)
+    cu = torch.tensor([0, 4], dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        C.varlen_fwd(z(4, 32, 128), z(4, 2, 128), z(4, 2, 128), None, cu, cu, None, None, None, None, 4, 4, 0.0, 0.088,
+                     False, True, -1, -1, 0.0, False, None, None)
+    with pytest.raises(RuntimeError, match="same dtype"):
+        C.varlen_fwd(z(4, 32, 128), z(4, 2, 128).float(), z(4, 2, 128), None, cu, cu, None, None, None, None, 4, 4, 0.0,
+                     0.088, False, True, -1, -1, 0.0, False, None, None)
+    with pytest.raises(RuntimeError, match="does not support softcap"):
+        C.fwd_kvcache(z(1, 1, 32, 128), z(1, 64, 2, 128), z(1, 64, 2, 128), None, None, None, None, None, None, None, None,
+                      None, None, 0.088, False, -1, -1, 1.0, True, 0, None)
