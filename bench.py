@@ -83,6 +83,9 @@ def parse_args():
                     help="skip BASELINE configs 3, 4 and 5 (keeps a profile to the default workload)")
     ap.add_argument("--only-config", type=int, default=0, choices=[0, 3, 4, 5],
                     help="run one of the extra configurations alone (for profiling it) and print its record")
+    ap.add_argument("--sharing-stats", action="store_true",
+                    help="print how many fetches a tile of 8 / 16 / 32 / 64 consecutive tokens could share on the selections "
+                         "of BASELINE configs 2, 3 and 4, and exit")
     ap.add_argument("--print-source-hash", action="store_true",
                     help="print the hash of the Stage-2 forward kernel sources (what a traffic summary must name) and exit")
     return ap.parse_args()
@@ -135,6 +138,60 @@ def copy_bandwidth(torch, dev):
     dst = torch.empty_like(src)
     ms = event_ms(torch, lambda: dst.copy_(src), 10)
     return {"gbs": 2 * src.numel() / ms / 1e6, "ms": ms, "what": "torch copy_ of 1 GiB, read + write bytes"}
+
+
+def sharing_stats(torch, ops, dev):
+    """How many fetches of a selected key block a tile of consecutive tokens could share, on the selections the
+    benchmark's own inputs produce (BASELINE configs 2, 3 and 4, real Stage-1 scores): per tile size, selected causal
+    (token, block) pairs divided by the distinct blocks the tiles touch - over all pairs, and over the pairs that are
+    NOT selected by every token of their tile (what the kernels walk per token)."""
+    import numpy as np
+    out = {}
+
+    def stats(idx, lens, mx):
+        words, _ = ops.topk_to_uint64(idx, mx, 64)
+        nblk = (mx + 63) // 64
+        bits = ops.uint64_to_bool(words, nblk).bool()
+        rec = {}
+        for tile in (8, 16, 32, 64):
+            picks = distinct = own_picks = own_distinct = 0
+            start = 0
+            for n in lens:
+                full = n // tile * tile
+                tok = torch.arange(full, device=dev)
+                causal_blk = torch.arange(nblk, device=dev)[None, :] <= (tok // 64)[:, None]
+                b = (bits[:, start:start + full] & causal_blk[None]).view(bits.shape[0], full // tile, tile, nblk)
+                anyb, allb = b.any(2), b.all(2)
+                picks += int(b.sum()); distinct += int(anyb.sum())
+                own = b & ~allb[:, :, None, :]
+                own_picks += int(own.sum()); own_distinct += int(own.any(2).sum())
+                start += n
+            rec[str(tile)] = {"pairs_per_distinct_block": picks / max(distinct, 1),
+                              "own_pairs_per_distinct_own_block": own_picks / max(own_distinct, 1),
+                              "own_share_of_pairs": own_picks / max(picks, 1)}
+        return rec
+
+    for S, name in ((32768, "config2_32k"), (131072, "config4_128k")):
+        g = torch.Generator(device="cuda").manual_seed(0 if S == 32768 else 4)
+        q = torch.randn(S, 32, 128, generator=g, device=dev).to(torch.bfloat16)
+        k = torch.randn(S, 2, 128, generator=g, device=dev).to(torch.bfloat16)
+        cu = torch.tensor([0, S], dtype=torch.int32, device=dev)
+        idx = ops.select_blocks(q, k, cu, cu, S, S, 64, 31, 1)
+        out[name] = stats(idx, [S], S)
+        del q, k, idx
+    rng = np.random.default_rng(1)
+    lens = [int(64 * x) for x in rng.integers(64, 385, size=4)]
+    T, mx = sum(lens), max(lens)
+    cu = torch.tensor(np.cumsum([0] + lens), dtype=torch.int32, device=dev)
+    g = torch.Generator(device="cuda").manual_seed(3)
+    q = torch.randn(T, 32, 128, generator=g, device=dev).to(torch.bfloat16)
+    k = torch.randn(T, 2, 128, generator=g, device=dev).to(torch.bfloat16)
+    zeros = torch.zeros(4, dtype=torch.int32, device=dev)
+    idx = ops.select_blocks(q, k, cu, cu, mx, mx, 64, 31, 1, cache_lens=zeros, max_cache_len=0)
+    out["config3_varlen"] = stats(idx, lens, mx)
+    out["what"] = ("selected causal (token, KV head, block) pairs per distinct block of a tile of consecutive tokens; "
+                   "'own' = pairs whose block is not selected by every token of the tile")
+    return out
 
 
 def config3_bench(torch, ops, dev):
@@ -355,6 +412,9 @@ def main():
     from infllmv2_cuda_impl_amd import _lib
 
     dev = torch.device("cuda:0")
+    if args.sharing_stats:
+        print(json.dumps(sharing_stats(torch, ops, dev)))
+        return
     if args.only_config:
         fn = {3: config3_bench, 4: config4_bench, 5: decode_bench}[args.only_config]
         print(json.dumps(fn(torch, ops, dev)))
