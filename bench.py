@@ -556,20 +556,6 @@ def main():
         result["stage2_bwd_ms"] = fb_ms - stages["stage2_fwd_op"]          # the backward alone (incl. its packing and mask transpose)
         result["stage2_fwd_bwd_tflops"] = 3.5 * fwd_flops / fb_ms / 1e9
         result["stage2_fwd_bwd_frac_peak"] = 3.5 * fwd_flops / fb_ms / 1e9 / PEAK_BF16_TFLOPS
-        # the opt-in backward mode that hands dS from the dK/dV kernel to the dQ kernel instead of recomputing S and dP
-        # there (INFLLMV2_BWD_HANDOFF=1): faster, for (topk + 1) * 2 KiB of transient workspace per token and KV head
-        prev = os.environ.get("INFLLMV2_BWD_HANDOFF")
-        os.environ["INFLLMV2_BWD_HANDOFF"] = "1"
-        try:
-            ho_ms = event_ms(torch, fwd_bwd, 5)
-        finally:
-            if prev is None:
-                del os.environ["INFLLMV2_BWD_HANDOFF"]
-            else:
-                os.environ["INFLLMV2_BWD_HANDOFF"] = prev
-        result["stage2_fwd_bwd_ds_handoff"] = {"ms": ho_ms, "frac_peak": 3.5 * fwd_flops / ho_ms / 1e9 / PEAK_BF16_TFLOPS,
-                                               "workspace_gb": 2 * S * (topk + 1) * 2048 / 1e9,
-                                               "what": "opt-in: dS tiles written by the dK/dV kernel and read by the dQ kernel"}
         del qg, kg, vg, dout, out_k, lse, ws
 
     if not args.no_stages and not args.no_other_configs:

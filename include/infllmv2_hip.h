@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define INFLLMV2_ABI_VERSION 9
+#define INFLLMV2_ABI_VERSION 10
 
 /* ---- library ------------------------------------------------------------------------------ */
 
@@ -242,7 +242,7 @@ int infllmv2_pack_kv(void* stream, const void* k, const void* v, const int32_t* 
                      int num_heads_k, int head_dim, int max_seqlen_k, const int64_t* k_strides,
                      const int64_t* v_strides);
 
-/* Scratch for infllmv2_varlen_bwd: four K/V block images, the transposed mask, D = rowsum(dO*O),
+/* Scratch for infllmv2_varlen_bwd: the K/V block images, the transposed mask, D = rowsum(dO*O),
  * transposed per-token images of q and dout, fp32 dK/dV accumulators. */
 size_t infllmv2_varlen_bwd_workspace_bytes(int batch, int64_t total_q, int64_t total_k, int num_heads_k,
                                            int max_seqlen_k);
@@ -250,11 +250,6 @@ size_t infllmv2_varlen_bwd_workspace_bytes(int batch, int64_t total_q, int64_t t
  * and 512-token slice of the packed query axis: 4.4 GB at 32768 tokens, growing with the square of the length). */
 size_t infllmv2_varlen_bwd_deterministic_workspace_bytes(int batch, int64_t total_q, int64_t total_k, int num_heads_k,
                                                          int max_seqlen_k);
-/* Workspace of infllmv2_varlen_bwd for any combination of its modes. */
-size_t infllmv2_varlen_bwd_workspace_bytes_ex(int batch, int64_t total_q, int64_t total_k, int num_heads_k,
-                                              int max_seqlen_k, int deterministic, int max_selected_blocks,
-                                              int n_uint64_per_row);
-
 /* csrc/entry.cu:17,213 `varlen_bwd` = mha_varlen_bwd (csrc/flash_attn/flash_api.cpp:1278-1547; kernels
  * flash_bwd_kernel.h:80-856, flash_bwd_preprocess_kernel.h:56-137,181-263) together with the mask
  * transposition the reference does in Python (infllmv2_sparse_attention.py:344-350): it takes the
@@ -265,12 +260,7 @@ size_t infllmv2_varlen_bwd_workspace_bytes_ex(int batch, int64_t total_q, int64_
  * bit-reproducible.  dK/dV are accumulated with fp32 atomics (one flush per 64-key block and slice of 512 query tokens, 128 when total_q <= 8192),
  * so their last bits can differ between runs, unless `deterministic` is set (the flag of flash_api.cpp:1448-1453,
  * which there concerns dQ): then every work item stores its tiles in a slot of its own and a second kernel adds them
- * in a fixed order; the workspace must then hold infllmv2_varlen_bwd_deterministic_workspace_bytes() bytes.
- * max_selected_blocks > 0 (an upper bound of the set bits of any mask row, e.g. the k of the top-k that built the
- * mask; rows with more bits would get a wrong dQ) switches on the dS hand-off: the dK/dV kernel stores the dS tile of
- * every (token, block) pair (2 KiB each, (max_selected_blocks + 1) tiles per token and KV head of workspace) and dQ
- * is computed from those tiles and K alone instead of recomputing S and dP; 0 recomputes.  Size the workspace with
- * infllmv2_varlen_bwd_workspace_bytes_ex then. */
+ * in a fixed order; the workspace must then hold infllmv2_varlen_bwd_deterministic_workspace_bytes() bytes. */
 int infllmv2_varlen_bwd(void* stream, const void* dout, const void* q, const void* k, const void* v,
                         const void* out, const float* softmax_lse, void* dq, void* dk, void* dv,
                         const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
@@ -280,8 +270,7 @@ int infllmv2_varlen_bwd(void* stream, const void* dout, const void* q, const voi
                         const int64_t* k_strides, const int64_t* v_strides, const int64_t* o_strides,
                         const int64_t* do_strides, const int64_t* dq_strides, const int64_t* dk_strides,
                         const int64_t* dv_strides, const int64_t* lse_strides, int n_uint64_per_row,
-                        float softmax_scale, int is_causal, int deterministic,
-                        int max_selected_blocks);
+                        float softmax_scale, int is_causal, int deterministic);
 
 /* ---- Stage 2: decode against a KV cache -------------------------------------------------------- */
 
@@ -401,8 +390,7 @@ int infllmv2_varlen_bwd_f16(void* stream, const void* dout, const void* q, const
                             const int64_t* k_strides, const int64_t* v_strides, const int64_t* o_strides,
                             const int64_t* do_strides, const int64_t* dq_strides, const int64_t* dk_strides,
                             const int64_t* dv_strides, const int64_t* lse_strides, int n_uint64_per_row,
-                            float softmax_scale, int is_causal, int deterministic,
-                            int max_selected_blocks);
+                            float softmax_scale, int is_causal, int deterministic);
 int infllmv2_fwd_kvcache_f16(void* stream, const void* q, void* kcache, void* vcache, const void* k_new,
                              const void* v_new, const int32_t* cache_seqlens, void* out, float* softmax_lse,
                              const uint64_t* blockmask, void* workspace, size_t workspace_bytes, int batch,

@@ -206,7 +206,7 @@ def varlen_bwd(dout, q, k, v, out, softmax_lse, dq_, dk_, dv_, cu_seqlens_q, cu_
                   cu_seqlens_k.data_ptr(), ptr(fwd_mask), ws.data_ptr(), ws.numel(), batch, total_q, total_k, Hq, Hk,
                   q.shape[-1], max_q, max_seqlen_k, _layout(q, expanded), _kv(k), _kv(v), _layout(out, expanded),
                   _layout(dout, expanded), _layout(dq, expanded), _kv(dk), _kv(dv), lse_strides, n64,
-                  float(softmax_scale), int(bool(is_causal)), int(bool(deterministic)), 0)
+                  float(softmax_scale), int(bool(is_causal)), int(bool(deterministic)))
     return [dq, dk, dv, torch.empty((0,), dtype=torch.float32, device=q.device)]
 
 

@@ -11,7 +11,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libinfllmv2_hip.so")
 
-ABI_VERSION = 9
+ABI_VERSION = 10
 
 _p, _i, _i64, _sz, _f = C.c_void_p, C.c_int, C.c_int64, C.c_size_t, C.c_float
 
@@ -36,7 +36,7 @@ SIGNATURES = {
     "infllmv2_stage1_decode": [_p] * 11 + [_sz] + [_i] * 6 + [_p] * 3 + [_i64, _i64, _f, _i, _i, _p] + [_i] * 8,
     "infllmv2_varlen_fwd": [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _sz, _i, _i, _i64, _i64, _i, _i, _i, _i, _i,
                             _p, _p, _p, _p, _p, _i, _f, _i],
-    "infllmv2_varlen_bwd": [_p] * 14 + [_sz, _i, _i64, _i64, _i, _i, _i, _i, _i] + [_p] * 9 + [_i, _f, _i, _i, _i],
+    "infllmv2_varlen_bwd": [_p] * 14 + [_sz, _i, _i64, _i64, _i, _i, _i, _i, _i] + [_p] * 9 + [_i, _f, _i, _i],
     "infllmv2_fwd_kvcache": [_p] * 11 + [_sz] + [_i] * 7 + [_p] * 6 + [_i, _i, _f, _p, _p, _p, _i64, _i, _p, _p, _i, _i],
     "infllmv2_fwd_kvcache_static": [_p] * 10 + [_i] * 7 + [_p] * 6 + [_i, _i, _f, _p, _p, _p, _i64, _i, _p, _p, _i, _i],
     "infllmv2_pack_kv": [_p, _p, _p, _p, _p, _sz, _i, _i64, _i, _i, _i, _p, _p],
@@ -56,7 +56,6 @@ OTHER = {
     "infllmv2_fwd_kvcache_num_splits": (_i, [_i, _i, _i]),
     "infllmv2_varlen_bwd_workspace_bytes": (_sz, [_i, _i64, _i64, _i, _i]),
     "infllmv2_varlen_bwd_deterministic_workspace_bytes": (_sz, [_i, _i64, _i64, _i, _i]),
-    "infllmv2_varlen_bwd_workspace_bytes_ex": (_sz, [_i, _i64, _i64, _i, _i, _i, _i, _i]),
 }
 
 

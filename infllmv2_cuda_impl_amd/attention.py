@@ -204,9 +204,6 @@ class Infllmv2AttnVarlenFunc(torch.autograd.Function):
         ctx.causal = causal
         ctx.deterministic = deterministic
         ctx.sparse = sparse
-        # the bound on set bits per mask row that the dS hand-off of the backward sizes its tiles by: known only when
-        # the mask was packed here from topk_idx (a caller's own mask may hold more blocks per row than k)
-        ctx.max_selected = topk_idx.shape[-1] if (topk_idx is not None and block_mask is None) else 0
         if not return_softmax:
             return out
         # S_dmask is only materialised with dropout, which this build rejects
@@ -221,7 +218,7 @@ class Infllmv2AttnVarlenFunc(torch.autograd.Function):
         q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, fwd_mask = ctx.saved_tensors
         dq, dk, dv = sparse_backward(dout, q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, ctx.max_seqlen_q,
                                      ctx.max_seqlen_k, ctx.softmax_scale, ctx.causal, fwd_mask, ctx.sparse,
-                                     ctx.deterministic, ctx.max_selected)
+                                     ctx.deterministic)
         return (dq, dk, dv) + (None,) * 15
 
 

@@ -8,8 +8,6 @@ transposed by a single kernel inside it.
 """
 from __future__ import annotations
 
-import os
-
 import torch
 
 from . import _lib
@@ -17,31 +15,15 @@ from ._util import ptr, stream_ptr
 
 GROUP = 16
 HAVE_BACKWARD = True
-# The dS hand-off (the dK/dV kernel stores its dS tiles, the dQ kernel reads them instead of recomputing S and dP) is
-# opt-in: it buys a few per cent of backward time for (k + 1) * 2 KiB of transient workspace per token and KV head
-# (8.7 GB at 32768 tokens with k = 64).  INFLLMV2_BWD_HANDOFF=1 switches it on for workspaces up to
-# INFLLMV2_BWD_HANDOFF_MAX_BYTES (default 16 GiB); anything larger, or an allocation failure, recomputes.
-HANDOFF_MAX_BYTES = 16 << 30
-
-
-def _handoff_limit() -> int:
-    """Bytes of dS scratch the caller allows; 0 = recompute (the default)."""
-    if os.environ.get("INFLLMV2_BWD_HANDOFF", "0") != "1":
-        return 0
-    return int(os.environ.get("INFLLMV2_BWD_HANDOFF_MAX_BYTES", HANDOFF_MAX_BYTES))
-
 
 def _nat(t, group=GROUP):
     return _lib.i64_array([t.stride(0), t.stride(1), group * t.stride(1)])
 
 
 def sparse_backward(dout, q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, softmax_scale,
-                    causal, fwd_mask, lse_expanded: bool, deterministic: bool = False, max_selected: int = 0):
+                    causal, fwd_mask, lse_expanded: bool, deterministic: bool = False):
     """Returns (dq, dk, dv) with the shapes and dtype of (q, k, v).  dq is always bit-reproducible; with
-    ``deterministic`` dk and dv are too (slots + ordered sum instead of fp32 atomics, at the price of a large workspace).
-    ``max_selected`` > 0 (an upper bound of the set bits per mask row) lets the dK/dV kernel hand its dS tiles to the dQ
-    kernel (2 KiB of workspace per token, KV head and selectable block) when INFLLMV2_BWD_HANDOFF=1 is set; the default
-    recomputes S and dP in the dQ kernel and needs no such workspace."""
+    ``deterministic`` dk and dv are too (slots + ordered sum instead of fp32 atomics, at the price of a large workspace)."""
     if dout.stride(-1) != 1:
         dout = dout.contiguous()
     if dout.dtype != q.dtype or tuple(dout.shape) != tuple(q.shape):
@@ -56,19 +38,9 @@ def sparse_backward(dout, q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, max_seq
     else:
         lse_strides = _lib.i64_array([1, total_q, grp * total_q])
     n64 = 0 if fwd_mask is None else fwd_mask.shape[-1]
-    if fwd_mask is None or Hk * total_q * (max_selected + 1) * 2048 > _handoff_limit():
-        max_selected = 0
-    def allocate(selected):
-        ws_bytes = _lib.lib.infllmv2_varlen_bwd_workspace_bytes_ex(batch, total_q, total_k, Hk, max_seqlen_k,
-                                                                  int(bool(deterministic)), int(selected), n64)
-        return torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=q.device)
-    try:
-        workspace = allocate(max_selected)
-    except torch.cuda.OutOfMemoryError:
-        if max_selected == 0:
-            raise
-        max_selected = 0                                      # no room for the dS tiles: recompute S and dP in the dQ kernel
-        workspace = allocate(0)
+    size_query = (_lib.lib.infllmv2_varlen_bwd_deterministic_workspace_bytes if deterministic
+                  else _lib.lib.infllmv2_varlen_bwd_workspace_bytes)
+    workspace = torch.empty(max(size_query(batch, total_q, total_k, Hk, max_seqlen_k), 256), dtype=torch.uint8, device=q.device)
     kv = lambda t: _lib.i64_array([t.stride(0), t.stride(1)])
     with torch.cuda.device(q.device):
         _lib.call_for(q.dtype, "infllmv2_varlen_bwd", stream_ptr(q.device), dout.data_ptr(), q.data_ptr(), k.data_ptr(),
@@ -76,5 +48,5 @@ def sparse_backward(dout, q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, max_seq
                   cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), ptr(fwd_mask), workspace.data_ptr(),
                   workspace.numel(), batch, total_q, total_k, Hq, Hk, d, max_seqlen_q, max_seqlen_k,
                   _nat(q, grp), kv(k), kv(v), _nat(out, grp), _nat(dout, grp), _nat(dq, grp), kv(dk), kv(dv), lse_strides, n64,
-                  float(softmax_scale), int(bool(causal)), int(bool(deterministic)), int(max_selected))
+                  float(softmax_scale), int(bool(causal)), int(bool(deterministic)))
     return dq, dk, dv

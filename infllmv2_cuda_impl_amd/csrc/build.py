@@ -40,7 +40,7 @@ HIPCC_FLAGS = [
 # -DIV2_F16, for IEEE half (entry points with the suffix _f16); the other files are element-type independent or take
 # the type at run time
 PER_ELEMENT_TYPE = {"compress.hip", "decode.hip", "stage1.hip", "stage1_decode.hip", "stage2_bwd.hip",
-                    "stage2_bwd_dkdv.hip", "stage2_bwd_dq.hip", "stage2_bwd_dq_handoff.hip", "stage2_fwd.hip",
+                    "stage2_bwd_dkdv.hip", "stage2_bwd_dq.hip", "stage2_fwd.hip",
                     "stage2_fwd_hybrid.hip"}
 
 

@@ -33,10 +33,9 @@ __device__ __forceinline__ int64_t image_slot0(const int* cu_seqlens_k, int b) {
 
 // Launches the packing pre-pass.  workspace receives [K image | V image] for the forward or, with
 // backward_images, [K image | V in K-image order] (the backward contracts V over d, and reads K^T out of the
-// K image by transposed LDS loads).  kt_image, if given, receives K in V-image order (one more image per block):
-// the A operand of dQ^T = K^T dS^T for the dQ kernel that works from handed-over dS tiles.
+// K image by transposed LDS loads).
 int launch_pack(hipStream_t st, const void* k, const void* v, const int32_t* cu_seqlens_k, void* workspace,
                 size_t workspace_bytes, int batch, int64_t total_k, int num_heads_k, int max_seqlen_k,
-                const int64_t* k_strides, const int64_t* v_strides, bool backward_images, void* kt_image = nullptr);
+                const int64_t* k_strides, const int64_t* v_strides, bool backward_images);
 
 }  // namespace IV2_NS

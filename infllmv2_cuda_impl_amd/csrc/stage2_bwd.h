@@ -39,13 +39,6 @@ struct BwdParams {
     float* det_slots;               // (Hk, n_slots, det_slices, 2, 64, 128) fp32
     uint32_t* det_flags;            // (Hk, n_slots, det_slices): 1 where a slot was written
     int det_slices;
-    // dS hand-off: the column kernel stores the dS^T tile (64 keys x 16 heads, bf16, 2 KiB) of every (token, block)
-    // pair it forms, and dQ is computed from those tiles and K alone instead of recomputing S and dP from K and V.
-    // The tile of the r-th selected block of a token's mask row is slot (kv head, token, r); null: no hand-off.
-    elem_bits* ds_buf;              // (Hk, total_q, max_sel + 1, 64, 16); slot max_sel of a row takes misdirected stores
-    const elem_bits* ktimg;         // K in V-image order (keys contracted): the A operand of dQ^T = K^T dS^T
-    const uint4* rankinfo;          // (Hk, total_q, n64_fwd): {mask word lo, hi, set bits in the row's earlier words, 0}
-    int max_sel;                    // upper bound of set bits per mask row
     int dkdv_spread;                // dK/dV work items: 1 = all XCDs share every slice (few slices), 0 = an XCD owns whole slice groups
 };
 
@@ -54,8 +47,6 @@ int launch_bwd_dq_hybrid(hipStream_t st, const BwdParams& p, int batch, int max_
 // dK/dV, two wavefronts (32 keys each) per (64-key block, 512-token slice): stage2_bwd_dkdv.hip
 int launch_bwd_dkdv_wave(hipStream_t st, const BwdParams& p, int batch, int max_seqlen_q, bool causal);
 
-// dQ from the dS tiles handed over by the column kernel: stage2_bwd_dq_handoff.hip
-int launch_bwd_dq_handoff(hipStream_t st, const BwdParams& p, int batch, int max_seqlen_q, bool causal);
 // deterministic mode only: adds the slots of every key block in slice order into dk_acc / dv_acc
 int launch_bwd_dkdv_reduce(hipStream_t st, const BwdParams& p, int batch);
 // Query tokens per dK/dV work item (slices are cut on the packed token axis).  Long inputs use 512-token slices (one

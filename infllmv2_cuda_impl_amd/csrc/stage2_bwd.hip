@@ -86,30 +86,15 @@ void bwd_convert_dkdv_kernel(const BwdParams p) {
     *reinterpret_cast<uint2*>(p.dv + row * p.dv_row + h * p.dv_head + d4 * 4) = va;
 }
 
-// rank records for the dS hand-off: for every mask row, per word {the word, set bits in the row's earlier words}
-__global__ __launch_bounds__(256)
-void bwd_rankinfo_kernel(const uint64_t* __restrict__ fwd_mask, uint4* __restrict__ rankinfo, int64_t rows, int n64) {
-    const int64_t r = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-    if (r >= rows) return;
-    unsigned before = 0;
-    for (int w = 0; w < n64; ++w) {
-        const uint64_t v = fwd_mask[r * n64 + w];
-        rankinfo[r * n64 + w] = make_uint4(static_cast<uint32_t>(v), static_cast<uint32_t>(v >> 32), before, 0u);
-        before += __builtin_popcountll(v);
-    }
-}
-
 static size_t align256(size_t x) { return (x + 255) & ~static_cast<size_t>(255); }
 
 struct BwdLayout {
     size_t images, mask, dsum, rowstat, dk_acc, dv_acc, total;
     size_t det_flags, det_slots, det_total;                    // deterministic mode only, after everything else
     int det_slices;
-    size_t rankinfo, ds_buf, ktimg;                            // dS hand-off only
 };
 
-static BwdLayout bwd_layout(int batch, int64_t total_q, int64_t total_k, int num_heads_k, int max_seqlen_k,
-                            int max_selected = 0, int n64_fwd = 0) {
+static BwdLayout bwd_layout(int batch, int64_t total_q, int64_t total_k, int num_heads_k, int max_seqlen_k) {
     BwdLayout L;
     size_t off = 0;
     L.images = off; off += align256(infllmv2_kv_image_bytes(total_k, batch, num_heads_k));   // K image | V in K-image order
@@ -119,12 +104,6 @@ static BwdLayout bwd_layout(int batch, int64_t total_q, int64_t total_k, int num
     L.rowstat = off; off += align256(static_cast<size_t>(num_heads_k) * total_q * 32 * 4);
     L.dk_acc = off; off += align256(static_cast<size_t>(total_k) * num_heads_k * kHeadDim * 4);
     L.dv_acc = off; off += align256(static_cast<size_t>(total_k) * num_heads_k * kHeadDim * 4);
-    L.rankinfo = L.ds_buf = L.ktimg = off;
-    if (max_selected > 0) {
-        L.ktimg = off; off += align256(infllmv2_kv_image_bytes(total_k, batch, num_heads_k) / 2);   // K in V-image order
-        L.rankinfo = off; off += align256(static_cast<size_t>(num_heads_k) * total_q * n64_fwd * 16);
-        L.ds_buf = off; off += align256(static_cast<size_t>(num_heads_k) * total_q * (max_selected + 1) * (kBlockN * 16 * 2));
-    }
     L.total = off;
     L.det_slices = static_cast<int>((total_q + kDkdvSlice - 1) / kDkdvSlice) + 1;
     const size_t items = static_cast<size_t>(num_heads_k) * image_slots(total_k, batch) * L.det_slices;
@@ -149,13 +128,6 @@ extern "C" size_t infllmv2_varlen_bwd_deterministic_workspace_bytes(int batch, i
     return bwd_layout(batch, total_q, total_k, num_heads_k, max_seqlen_k).det_total;
 }
 
-extern "C" size_t infllmv2_varlen_bwd_workspace_bytes_ex(int batch, int64_t total_q, int64_t total_k, int num_heads_k,
-                                                         int max_seqlen_k, int deterministic, int max_selected_blocks,
-                                                         int n_uint64_per_row) {
-    const BwdLayout L = bwd_layout(batch, total_q, total_k, num_heads_k, max_seqlen_k,
-                                   n_uint64_per_row > 0 ? max_selected_blocks : 0, n_uint64_per_row);
-    return deterministic ? L.det_total : L.total;
-}
 #endif
 
 extern "C" int IV2_ENTRY(infllmv2_varlen_bwd)(void* stream, const void* dout, const void* q, const void* k, const void* v,
@@ -167,7 +139,7 @@ extern "C" int IV2_ENTRY(infllmv2_varlen_bwd)(void* stream, const void* dout, co
                                    const int64_t* k_strides, const int64_t* v_strides, const int64_t* o_strides,
                                    const int64_t* do_strides, const int64_t* dq_strides, const int64_t* dk_strides,
                                    const int64_t* dv_strides, const int64_t* lse_strides, int n_uint64_per_row,
-                                   float softmax_scale, int is_causal, int deterministic, int max_selected_blocks) {
+                                   float softmax_scale, int is_causal, int deterministic) {
     IV2_CHECK(head_dim == kHeadDim, "varlen_bwd: this build only supports head_dim 128 (got %d)", head_dim);
     IV2_CHECK(valid_group(num_heads, num_heads_k),
               "varlen_bwd: requires num_heads == g * num_heads_k with g in {1, 2, 4, 8, 16} (got %d and %d)", num_heads, num_heads_k);
@@ -175,10 +147,7 @@ extern "C" int IV2_ENTRY(infllmv2_varlen_bwd)(void* stream, const void* dout, co
     IV2_CHECK(dout && q && k && v && out && softmax_lse && dq && dk && dv && cu_seqlens_q && cu_seqlens_k && workspace,
               "varlen_bwd: null pointer");
     IV2_CHECK(num_heads_k <= 65535 && batch <= 65535, "varlen_bwd: batch and num_heads_k must not exceed 65535");
-    IV2_CHECK(max_selected_blocks >= 0 && max_selected_blocks <= 65535, "varlen_bwd: max_selected_blocks out of range");
-    const bool handoff = max_selected_blocks > 0 && fwd_blockmask != nullptr && n_uint64_per_row > 0;
-    const BwdLayout L = bwd_layout(batch, total_q, total_k, num_heads_k, max_seqlen_k, handoff ? max_selected_blocks : 0,
-                                   n_uint64_per_row);
+    const BwdLayout L = bwd_layout(batch, total_q, total_k, num_heads_k, max_seqlen_k);
     const size_t ws_needed = deterministic ? L.det_total : L.total;
     IV2_CHECK(workspace_bytes >= ws_needed, "varlen_bwd: workspace too small (%zu < %zu)", workspace_bytes, ws_needed);
     IV2_CHECK(reinterpret_cast<uintptr_t>(workspace) % 256 == 0, "varlen_bwd: workspace must be 256-byte aligned");
@@ -246,8 +215,7 @@ extern "C" int IV2_ENTRY(infllmv2_varlen_bwd)(void* stream, const void* dout, co
     }
     if (total_q > 0 && max_seqlen_q > 0 && total_k > 0 && max_seqlen_k > 0) {
         int rc = launch_pack(st, k, v, cu_seqlens_k, ws + L.images, L.mask - L.images, batch, total_k, num_heads_k,
-                             max_seqlen_k, k_strides, v_strides, true,    // K image | V in K-image order
-                             handoff ? ws + L.ktimg : nullptr);
+                             max_seqlen_k, k_strides, v_strides, true);   // K image | V in K-image order
         if (rc != 0) return rc;
         if (fwd_blockmask != nullptr) {
             uint64_t* bwd_mask = reinterpret_cast<uint64_t*>(ws + L.mask);
@@ -259,26 +227,10 @@ extern "C" int IV2_ENTRY(infllmv2_varlen_bwd)(void* stream, const void* dout, co
         IV2_CHECK(total_q <= 0x7fffffffll, "varlen_bwd: too many query tokens");
         hipLaunchKernelGGL(bwd_prep_kernel, dim3(static_cast<unsigned>(total_q), num_heads_k), dim3(256), 0, st, p);
         IV2_LAUNCH_CHECK();
-        if (handoff) {
-            // the column kernel runs first and leaves the dS^T tile of every pair for the dQ kernel
-            p.rankinfo = reinterpret_cast<const uint4*>(ws + L.rankinfo);
-            p.ds_buf = reinterpret_cast<elem_bits*>(ws + L.ds_buf);
-            p.ktimg = reinterpret_cast<const elem_bits*>(ws + L.ktimg);
-            p.max_sel = max_selected_blocks;
-            const int64_t rows = static_cast<int64_t>(num_heads_k) * total_q;
-            hipLaunchKernelGGL(bwd_rankinfo_kernel, dim3(static_cast<unsigned>((rows + 255) / 256)), dim3(256), 0, st,
-                               fwd_blockmask, reinterpret_cast<uint4*>(ws + L.rankinfo), rows, n_uint64_per_row);
-            IV2_LAUNCH_CHECK();
-            rc = launch_bwd_dkdv_wave(st, p, batch, max_seqlen_q, is_causal != 0);
-            if (rc != 0) return rc;
-            rc = launch_bwd_dq_handoff(st, p, batch, max_seqlen_q, is_causal != 0);
-            if (rc != 0) return rc;
-        } else {
-            rc = launch_bwd_dq_hybrid(st, p, batch, max_seqlen_q, is_causal != 0);
-            if (rc != 0) return rc;
-            rc = launch_bwd_dkdv_wave(st, p, batch, max_seqlen_q, is_causal != 0);
-            if (rc != 0) return rc;
-        }
+        rc = launch_bwd_dq_hybrid(st, p, batch, max_seqlen_q, is_causal != 0);
+        if (rc != 0) return rc;
+        rc = launch_bwd_dkdv_wave(st, p, batch, max_seqlen_q, is_causal != 0);
+        if (rc != 0) return rc;
         if (deterministic) {
             rc = launch_bwd_dkdv_reduce(st, p, batch);
             if (rc != 0) return rc;

@@ -33,7 +33,7 @@
 namespace IV2_NS {
 
 constexpr int kGroupWords = 32;                                // one mask word per lane of the lower half-wavefront: a group is 2048 tokens
-constexpr int kStage = 16384 + 512 + 512;                      // q a|b, dout a|b (4 KiB each), the pair's 64 row scalars, its two rank records
+constexpr int kStage = 16384 + 512 + 512;                      // q a|b, dout a|b (4 KiB each), the pair's 64 row scalars; padded so that two stages are the flush tile
 constexpr int kWaveLds = 2 * kStage;                           // = 64 rows x 132 floats: also the flush tile
 constexpr int kFlushPitch = 132;                               // floats per key row of the flush tile
 constexpr int kWaveTiles = 2;                                  // 16-key tiles per wavefront: a wavefront owns 32 of the block's 64 keys
@@ -80,7 +80,7 @@ __device__ __forceinline__ short4v lds_read_tr(const unsigned char* ptr) {
 }
 
 // kColSlice: query tokens per work item (512, or 128 for short inputs)
-template <bool kCausal, bool kHandoff, int kColSlice>
+template <bool kCausal, int kColSlice>
 __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void bwd_dkdv_wave_kernel(const BwdParams p) {
     constexpr int kSliceWords = kColSlice / 64;                // mask words per slice (a power of two)
@@ -235,18 +235,12 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
     const elem_bits* q_head = p.q + static_cast<int64_t>(h) * p.q_kvh;
     const elem_bits* do_head = p.dout + static_cast<int64_t>(h) * p.do_kvh;
     const float* stat_head = p.rowstat + static_cast<int64_t>(h) * p.total_q * 32;
-    constexpr bool handoff = kHandoff;                         // the launcher picks the variant: p.ds_buf != nullptr
-    const uint32_t rank_lane = static_cast<uint32_t>((lane & 3) * 4);
-    const uint4* rank_head = handoff ? p.rankinfo + static_cast<int64_t>(h) * p.total_q * p.n64_fwd + (j >> 6) : nullptr;
-    const uint64_t below_j = (1ull << (j & 63)) - 1ull;        // the mask bits of the blocks before j in its word
     // byte strides per token as 32-bit scalars (checked by the launcher): a token's address is one 32 x 32 -> 64 bit
     // multiplication away
     const uint32_t q_tok_bytes = static_cast<uint32_t>(p.q_tok * 2), do_tok_bytes = static_cast<uint32_t>(p.do_tok * 2);
-    const uint32_t rank_tok_bytes = static_cast<uint32_t>(p.n64_fwd) * 16u;
     const unsigned char* q_bytes = reinterpret_cast<const unsigned char*>(q_head);
     const unsigned char* do_bytes = reinterpret_cast<const unsigned char*>(do_head);
     const unsigned char* stat_bytes = reinterpret_cast<const unsigned char*>(stat_head);
-    const unsigned char* rank_bytes = reinterpret_cast<const unsigned char*>(rank_head);
     auto issue = [&](int64_t ta, int64_t tb, int stage) {
         const uint32_t st = ring_lds + stage * kStage;
         const uint64_t ua = static_cast<uint32_t>(ta), ub = static_cast<uint32_t>(tb);     // packed token indices fit 31 bits
@@ -262,15 +256,12 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
             dma16<128, 6144>(qb, q_lane, st);   dma16<192, 7168>(qb, q_lane, st);
             // token a's [lse * log2e (16) | D (16)] (both half-wavefronts fetch the same 128 bytes)
             dma4<16384>(stat_bytes + (ua << 7), stat_lane, st);
-            // the 16-byte rank record of (token, mask word of block j), replicated over the 256-byte region
-            if (handoff) dma4<16896>(rank_bytes + ua * rank_tok_bytes, rank_lane, st);
         } else {
             dma16<0, 8192>(da, do_lane, st);    dma16<64, 9216>(da, do_lane, st);
             dma16<128, 10240>(da, do_lane, st); dma16<192, 11264>(da, do_lane, st);
             dma16<0, 12288>(db, do_lane, st);   dma16<64, 13312>(db, do_lane, st);
             dma16<128, 14336>(db, do_lane, st); dma16<192, 15360>(db, do_lane, st);
             dma4<16384 + 256>(stat_bytes + (ub << 7), stat_lane, st);
-            if (handoff) dma4<16896 + 256>(rank_bytes + ub * rank_tok_bytes, rank_lane, st);
         }
     };
 
@@ -323,26 +314,6 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
 
         const float* scal = reinterpret_cast<const float*>(st + 16384);
         const bool edge = (lim_a < kBlockN - 1) || (lim_b < kBlockN - 1);
-        // hand-off: where the dS^T tiles of this pair go (rank of block j among the set bits of each token's mask row)
-        elem_bits* ds_a = nullptr;
-        elem_bits* ds_b = nullptr;
-        if (handoff) {
-            const uint4 ra = *reinterpret_cast<const uint4*>(st + 16896);
-            const uint4 rb = *reinterpret_cast<const uint4*>(st + 16896 + 256);
-            const uint32_t alo = __builtin_amdgcn_readfirstlane(ra.x), ahi = __builtin_amdgcn_readfirstlane(ra.y);
-            const uint32_t blo = __builtin_amdgcn_readfirstlane(rb.x), bhi = __builtin_amdgcn_readfirstlane(rb.y);
-            int rank_a = static_cast<int>(__builtin_amdgcn_readfirstlane(ra.z)) +
-                         __builtin_popcountll(((static_cast<uint64_t>(ahi) << 32) | alo) & below_j);
-            int rank_b = static_cast<int>(__builtin_amdgcn_readfirstlane(rb.z)) +
-                         __builtin_popcountll(((static_cast<uint64_t>(bhi) << 32) | blo) & below_j);
-            // a row with more set bits than announced, or the absent second token, writes to the row's spare slot
-            if (rank_a > p.max_sel) rank_a = p.max_sel;
-            if (rank_b > p.max_sel || !has_b) rank_b = p.max_sel;
-            const int64_t row_tiles = p.max_sel + 1;
-            ds_a = p.ds_buf + ((static_cast<int64_t>(h) * p.total_q + ta) * row_tiles + rank_a) * (kBlockN * 16);
-            ds_b = p.ds_buf + ((static_cast<int64_t>(h) * p.total_q + tb) * row_tiles + rank_b) * (kBlockN * 16);
-        }
-
         // Per wavefront 64 MFMAs in four GEMM phases with the softmax backward between them; the other wavefront of the
         // SIMD fills the matrix pipeline while this one does vector work:
         //   A  S = Q K^T                       (both tokens, this wavefront's 32 keys; a fragment read from LDS feeds 2 MFMAs)
@@ -353,23 +324,15 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
         const uint4* frag = reinterpret_cast<const uint4*>(st) + frag_unit;      // tile t, chunk c at frag[t * 256 + c * 64]
         elem8 pfr[kWaveTiles], dsfr[kWaveTiles];              // per key tile: [token a heads 4g..4g+3 | token b heads 4g..4g+3]
         floatx4 sa[kWaveTiles], sb[kWaveTiles], dpa[kWaveTiles], dpb[kWaveTiles];
-        // Without the hand-off the S accumulators start at -LSE / scale, so that P = exp2(scale S') needs no subtraction
-        // (and the LSE no registers) after the MFMAs; a row without visible keys has LSE = +inf: S' = -inf, P = 0.  With
-        // the hand-off's extra addresses live that form spills a register, so there the LSE is subtracted after the MFMAs.
-        constexpr bool kFoldLse = !kHandoff;
-        if (kFoldLse) {
+        // The S accumulators start at -LSE / scale, so that P = exp2(scale S') needs no subtraction (and the LSE no
+        // registers) after the MFMAs; a row without visible keys has LSE = +inf: S' = -inf, P = 0.
+        {
             const float4 la = *reinterpret_cast<const float4*>(scal + 4 * g);
             const float4 lb = *reinterpret_cast<const float4*>(scal + 64 + 4 * g);
             const float inv = -1.f / p.scale_log2;
             const floatx4 ia = {la.x * inv, la.y * inv, la.z * inv, la.w * inv}, ib = {lb.x * inv, lb.y * inv, lb.z * inv, lb.w * inv};
 #pragma unroll
             for (int kt = 0; kt < kWaveTiles; ++kt) { sa[kt] = ia; sb[kt] = ib; }
-        } else {
-#pragma unroll
-            for (int kt = 0; kt < kWaveTiles; ++kt) {
-                sa[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
-                sb[kt] = sa[kt];
-            }
         }
         {   // A
 #pragma unroll
@@ -387,19 +350,12 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
         }
         __builtin_amdgcn_sched_barrier(0);
         {   // P, kept in fp32 in place of S
-            float lse_a[4] = {0.f, 0.f, 0.f, 0.f}, lse_b[4] = {0.f, 0.f, 0.f, 0.f};
-            if (!kFoldLse) {
-                const float4 la = *reinterpret_cast<const float4*>(scal + 4 * g);
-                const float4 lb = *reinterpret_cast<const float4*>(scal + 64 + 4 * g);
-                lse_a[0] = la.x; lse_a[1] = la.y; lse_a[2] = la.z; lse_a[3] = la.w;
-                lse_b[0] = lb.x; lse_b[1] = lb.y; lse_b[2] = lb.z; lse_b[3] = lb.w;
-            }
 #pragma unroll
             for (int kt = 0; kt < kWaveTiles; ++kt)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    float xa = __builtin_amdgcn_exp2f(kFoldLse ? sa[kt][e] * p.scale_log2 : sa[kt][e] * p.scale_log2 - lse_a[e]);
-                    float xb = __builtin_amdgcn_exp2f(kFoldLse ? sb[kt][e] * p.scale_log2 : sb[kt][e] * p.scale_log2 - lse_b[e]);
+                    float xa = __builtin_amdgcn_exp2f(sa[kt][e] * p.scale_log2);
+                    float xb = __builtin_amdgcn_exp2f(sb[kt][e] * p.scale_log2);
                     sa[kt][e] = xa;
                     sb[kt][e] = xb;
                     pfr[kt][e] = static_cast<elem_t>(xa);
@@ -463,19 +419,6 @@ void bwd_dkdv_wave_kernel(const BwdParams p) {
                     dsfr[kt][4 + e] = static_cast<elem_t>(sb[kt][e] * dpb[kt][e]);
                 }
                 __builtin_amdgcn_sched_barrier(0);
-            }
-        }
-        if (handoff) {
-            // dS^T tiles [key][head]: lane (key n of tile kt, heads 4g..4g+3) holds 8 bytes per token; always 4 stores
-#pragma unroll
-            for (int kt = 0; kt < kWaveTiles; ++kt) {
-                uint4 raw;
-                __builtin_memcpy(&raw, &dsfr[kt], 16);
-                const int at = (kWaveTiles * wave + kt) * 256 + n * 16 + 4 * g;    // the tile bases are wave-uniform: scalar base + lane offset
-                // streaming stores: the tiles are read much later, by another kernel, and should not push q / dout out of L2
-                typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
-                __builtin_nontemporal_store(u32x2{raw.x, raw.y}, reinterpret_cast<u32x2*>(ds_a + at));
-                __builtin_nontemporal_store(u32x2{raw.z, raw.w}, reinterpret_cast<u32x2*>(ds_b + at));
             }
         }
         {   // D: transposed reads of the q tiles
@@ -605,11 +548,8 @@ static int launch_bwd_dkdv_sliced(hipStream_t st, const BwdParams& p_in, int bat
               "varlen_bwd: token strides of q and dout must lie in [0, 2^31) elements");
     const dim3 grid(static_cast<unsigned>(items), batch, p.num_heads_k);
     const size_t lds = kWaveLds + kGroupWords * 8;
-    const bool handoff = p.ds_buf != nullptr;
-    if (causal && handoff) hipLaunchKernelGGL((bwd_dkdv_wave_kernel<true, true, kColSlice>), grid, dim3(128), lds, st, p);
-    else if (causal) hipLaunchKernelGGL((bwd_dkdv_wave_kernel<true, false, kColSlice>), grid, dim3(128), lds, st, p);
-    else if (handoff) hipLaunchKernelGGL((bwd_dkdv_wave_kernel<false, true, kColSlice>), grid, dim3(128), lds, st, p);
-    else hipLaunchKernelGGL((bwd_dkdv_wave_kernel<false, false, kColSlice>), grid, dim3(128), lds, st, p);
+    if (causal) hipLaunchKernelGGL((bwd_dkdv_wave_kernel<true, kColSlice>), grid, dim3(128), lds, st, p);
+    else hipLaunchKernelGGL((bwd_dkdv_wave_kernel<false, kColSlice>), grid, dim3(128), lds, st, p);
     IV2_LAUNCH_CHECK();
     return 0;
 }

@@ -31,7 +31,6 @@ struct PackParams {
     elem_bits* kimg;                // K in K-image order (operand of a GEMM contracting over d)
     elem_bits* vimg;                // forward: V in V-image order (A operand of a GEMM contracting over keys), else null
     elem_bits* vimg_r;              // backward: V in K-image order (dP = dO V^T contracts over d), else null
-    elem_bits* ktimg;               // backward with dS hand-off: K in V-image order (A operand of dQ^T = K^T dS^T), else null
     const int* cu_seqlens_k;
     int64_t k_row_stride, k_head_stride;
     int64_t v_row_stride, v_head_stride;
@@ -68,33 +67,27 @@ void pack_kv_kernel(const PackParams p) {
             *reinterpret_cast<uint4*>(p.vimg_r + img_off + u * 8) = vv;
         }
     }
-    // images that contract over the keys: V for the forward, K for the dQ kernel of the dS hand-off
-#pragma unroll 1
-    for (int which = 0; which < 2; ++which) {
-        elem_bits* dst = which == 0 ? p.vimg : p.ktimg;
-        if (dst == nullptr) continue;                         // uniform per workgroup
-        const elem_bits* src = which == 0 ? vb : kb;
-        const int64_t src_row = which == 0 ? p.v_row_stride : p.k_row_stride;
-        __syncthreads();
-        for (int u = tid; u < 1024; u += 256) {
-            const int key = u >> 4, d0 = (u & 15) * 8;
-            uint4 val = zero;
-            if (key < valid) val = *reinterpret_cast<const uint4*>(src + key * src_row + d0);
-            *reinterpret_cast<uint4*>(&vt[key][d0]) = val;
-        }
-        __syncthreads();
-        for (int u = tid; u < 1024; u += 256) {
-            const int dt = u >> 7, cc = (u >> 6) & 1, lane = u & 63;
-            const int r = lane & 15, g = lane >> 4;
-            const int d = 16 * dt + r;
-            uint32_t w[4];
+    // the image that contracts over the keys: V for the forward
+    if (p.vimg == nullptr) return;                            // uniform per workgroup
+    __syncthreads();
+    for (int u = tid; u < 1024; u += 256) {
+        const int key = u >> 4, d0 = (u & 15) * 8;
+        uint4 val = zero;
+        if (key < valid) val = *reinterpret_cast<const uint4*>(vb + key * p.v_row_stride + d0);
+        *reinterpret_cast<uint4*>(&vt[key][d0]) = val;
+    }
+    __syncthreads();
+    for (int u = tid; u < 1024; u += 256) {
+        const int dt = u >> 7, cc = (u >> 6) & 1, lane = u & 63;
+        const int r = lane & 15, g = lane >> 4;
+        const int d = 16 * dt + r;
+        uint32_t w[4];
 #pragma unroll
-            for (int jj = 0; jj < 8; jj += 2) {
-                const int key_a = 32 * cc + (jj < 4 ? 4 * g + jj : 16 + 4 * g + jj - 4);
-                w[jj >> 1] = static_cast<uint32_t>(vt[key_a][d]) | (static_cast<uint32_t>(vt[key_a + 1][d]) << 16);
-            }
-            *reinterpret_cast<uint4*>(dst + img_off + u * 8) = make_uint4(w[0], w[1], w[2], w[3]);
+        for (int jj = 0; jj < 8; jj += 2) {
+            const int key_a = 32 * cc + (jj < 4 ? 4 * g + jj : 16 + 4 * g + jj - 4);
+            w[jj >> 1] = static_cast<uint32_t>(vt[key_a][d]) | (static_cast<uint32_t>(vt[key_a + 1][d]) << 16);
         }
+        *reinterpret_cast<uint4*>(p.vimg + img_off + u * 8) = make_uint4(w[0], w[1], w[2], w[3]);
     }
 }
 
@@ -111,7 +104,7 @@ extern "C" size_t infllmv2_kv_image_bytes(int64_t total_k, int batch, int num_he
 namespace IV2_NS {
 int launch_pack(hipStream_t st, const void* k, const void* v, const int32_t* cu_seqlens_k, void* workspace,
                 size_t workspace_bytes, int batch, int64_t total_k, int num_heads_k, int max_seqlen_k,
-                const int64_t* k_strides, const int64_t* v_strides, bool backward_images, void* kt_image) {
+                const int64_t* k_strides, const int64_t* v_strides, bool backward_images) {
     IV2_CHECK(k && v && cu_seqlens_k && workspace, "pack_kv: null pointer");
     IV2_CHECK(batch > 0 && num_heads_k > 0 && total_k >= 0 && max_seqlen_k >= 0, "pack_kv: bad sizes");
     IV2_CHECK(num_heads_k <= 65535 && batch <= 65535, "pack_kv: batch and num_heads_k must not exceed 65535");
@@ -129,7 +122,6 @@ int launch_pack(hipStream_t st, const void* k, const void* v, const int32_t* cu_
     pp.kimg = static_cast<elem_bits*>(workspace);
     elem_bits* second = pp.kimg + n_slots * num_heads_k * kImageElems;
     if (backward_images) pp.vimg_r = second; else pp.vimg = second;
-    pp.ktimg = static_cast<elem_bits*>(kt_image);
     pp.cu_seqlens_k = cu_seqlens_k;
     pp.k_row_stride = k_strides[0]; pp.k_head_stride = k_strides[1];
     pp.v_row_stride = v_strides[0]; pp.v_head_stride = v_strides[1];

@@ -289,7 +289,7 @@ std::vector<Tensor> varlen_bwd(const Tensor& dout, const Tensor& q, const Tensor
                 ws.data_ptr(), static_cast<size_t>(ws.numel()), batch, total_q, total_k, static_cast<int>(Hq), static_cast<int>(Hk),
                 static_cast<int>(q.size(-1)), static_cast<int>(max_q), static_cast<int>(max_seqlen_k), qs.v, ks.v, vs.v, os.v,
                 dos.v, dqs.v, dks.v, dvs.v, lse_strides, n64, static_cast<float>(softmax_scale), is_causal ? 1 : 0,
-                deterministic ? 1 : 0, 0), "varlen_bwd");
+                deterministic ? 1 : 0), "varlen_bwd");
     return {dq, dk, dv, at::empty({0}, q.options().dtype(at::kFloat))};
 }
 

@@ -99,8 +99,8 @@ def test_stage2_forward_backward_fp16(ops, seqs, Hk, k_sel, causal):
     assert err.mean() < 4e-4
 
 
-def test_backward_modes_fp16(ops, monkeypatch):
-    """dS hand-off and deterministic dK/dV in fp16 agree with the default mode to rounding."""
+def test_backward_modes_fp16(ops):
+    """Deterministic dK/dV in fp16 agrees with the default mode to rounding and is bit-reproducible."""
     seqs = [900]
     T = 900
     q, k, v, dout = rand((T, 32, 128), 7), rand((T, 2, 128), 8), rand((T, 2, 128), 9), rand((T, 32, 128), 10)
@@ -114,13 +114,10 @@ def test_backward_modes_fp16(ops, monkeypatch):
         return [t.grad.float() for t in (qg, kg, vg)]
 
     base = grads()
-    monkeypatch.setenv("INFLLMV2_BWD_HANDOFF", "1")
-    hand = grads()
-    monkeypatch.delenv("INFLLMV2_BWD_HANDOFF")
     det1, det2 = grads(True), grads(True)
-    for a, b, c, d in zip(base, hand, det1, det2):
+    for a, c, d in zip(base, det1, det2):
         s = max(1.0, float(a.abs().max()))
-        assert float((a - b).abs().max()) <= 2e-2 * s and float((a - c).abs().max()) <= 2e-2 * s
+        assert float((a - c).abs().max()) <= 2e-2 * s
         assert torch.equal(c, d)
 
 

@@ -130,19 +130,14 @@ def test_deterministic_mode(ops, sq, sk, k_sel, causal, sparse):
     check_grad("dv", grads[0][2], dv)
 
 
-@pytest.mark.parametrize("handoff", ["1", "0"])
 @pytest.mark.parametrize("sq,sk,k_sel", [([300], [4500], 12), ([1500, 700], [1500, 700], 6), ([130], [130], 3)])
-def test_ds_handoff_and_recompute_agree_with_oracle(ops, monkeypatch, handoff, sq, sk, k_sel):
-    """With a top-k mask and INFLLMV2_BWD_HANDOFF=1 the dK/dV kernel hands its dS tiles to the dQ kernel (slot = rank of the block in the token's
-    mask row; [300] x [4500] has rows of two 64-bit words, so ranks continue across a word boundary);
-    without INFLLMV2_BWD_HANDOFF=1 (the default) the dQ kernel recomputes S and dP.  Both must meet the oracle."""
-    monkeypatch.setenv("INFLLMV2_BWD_HANDOFF", handoff)
+def test_wide_rows_and_packed_sequences_agree_with_oracle(ops, sq, sk, k_sel):
+    """[300] x [4500] has mask rows of two 64-bit words; two packed sequences; one short one."""
     run_case(ops, sq, sk, 2, k_sel, True, seed=21)
 
 
-def test_ds_handoff_with_duplicate_and_missing_indices(ops, monkeypatch):
-    """Rows with fewer set bits than the announced bound (-1 entries and repeated blocks) leave slots unused."""
-    monkeypatch.setenv("INFLLMV2_BWD_HANDOFF", "1")
+def test_backward_with_duplicate_and_missing_indices(ops):
+    """Rows with -1 entries and repeated blocks: fewer set bits than the row is wide."""
     dev = torch.device("cuda:0")
     q, k, v, cu_q, cu_k, idx = make_case(23, [700], [700], 2, 5, dev)
     idx[:, ::3, 1] = idx[:, ::3, 0]
@@ -158,31 +153,3 @@ def test_ds_handoff_with_duplicate_and_missing_indices(ops, monkeypatch):
     check_grad("dv", vg.grad, dv)
 
 
-def test_ds_handoff_falls_back_when_its_workspace_does_not_fit(ops, monkeypatch):
-    """The dS tiles need (k + 1) * 2 KiB per token and KV head; when that allocation fails the backward takes the
-    dQ kernel that recomputes S and dP.  The failure is simulated on the host: the first workspace request of the
-    backward raises torch's out-of-memory error."""
-    monkeypatch.setenv("INFLLMV2_BWD_HANDOFF", "1")
-    dev = torch.device("cuda:0")
-    q, k, v, cu_q, cu_k, idx = make_case(31, [700], [700], 2, 5, dev)
-    dout = torch.randn(q.shape, generator=torch.Generator(device="cpu").manual_seed(32)).to(torch.bfloat16).to(dev)
-    qg, kg, vg = [t.clone().requires_grad_(True) for t in (q, k, v)]
-    out = ops.infllmv2_attn_varlen_func(qg, kg, vg, cu_q, cu_k, 700, 700, causal=True, topk_idx=idx)
-    real_empty, state = torch.empty, {"armed": True, "raised": 0}
-
-    def empty(*args, **kwargs):
-        if state["armed"] and kwargs.get("dtype") == torch.uint8:
-            state["armed"] = False
-            state["raised"] += 1
-            raise torch.cuda.OutOfMemoryError("simulated")
-        return real_empty(*args, **kwargs)
-    monkeypatch.setattr(torch, "empty", empty)
-    out.backward(dout)
-    monkeypatch.setattr(torch, "empty", real_empty)
-    assert state["raised"] == 1
-    words = O.topk_to_uint64(idx.cpu().numpy(), 700, 64)[0]
-    dq, dk, dv = O.stage2_backward(bf16_np(q), bf16_np(k), bf16_np(v), bf16_np(dout), cu_q.cpu().numpy(),
-                                   cu_k.cpu().numpy(), words, 128 ** -0.5, True)
-    check_grad("dq", qg.grad, dq)
-    check_grad("dk", kg.grad, dk)
-    check_grad("dv", vg.grad, dv)
