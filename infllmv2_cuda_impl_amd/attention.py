@@ -241,7 +241,7 @@ def infllmv2_attn_varlen_func(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q,
     windows and paged KV are rejected exactly as the reference build rejects them.
     ``block_mask`` (not in the reference's signature) is the packed form of the same selection, int64
     ``(nheads_k, total_q, ceil(ceil(max_seqlen_k / 64) / 64))`` as ``topk_to_uint64`` / ``topk_blocks(return_mask=True)``
-    produce it; when given it is used as is and ``topk_idx`` only bounds the blocks per row for the backward.
+    produce it; when given it is used as is and ``topk_idx`` is ignored.
     Head sizes below 128 are served by zero padding (see :func:`pad_head_dim`); ``softmax_scale`` then defaults to
     the caller's head size ``** -0.5``, as in the reference.
     """
