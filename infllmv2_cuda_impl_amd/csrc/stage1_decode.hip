@@ -178,20 +178,46 @@ __device__ __forceinline__ void s1d_lse_run(const S1DecodeParams& p, const S1Dec
     }
 }
 
-// log-sum-exp (log2 units) of head 4g + e from `count` partial records {max x 16, sum x 16}: lane (n, g) merges the
-// records n, n + 16, ... for its four heads, then the 16 lanes of a row merge among themselves (the merge of (max,
-// sum) pairs is associative and commutative up to rounding, and every lane of a row ends with the same bits because
-// the butterfly combines the same pairs in the same order on both sides).
-__device__ __forceinline__ void s1d_merge_partials(const float* part, int count, int n, int g, int group, float (&lse2)[4]) {
+// The partial records {max x 16, sum x 16} of one (sequence, head) as a lane needs them: lane (n, g) takes the records
+// n, n + 16, n + 32, n + 48 (at most 64 runs) for its four heads, two 16-byte loads per record.  The number of loads
+// does not depend on the data (an index beyond the last record reads the last one again and is ignored later), so that
+// the loads requested after these can stay in flight while these are waited for.
+struct S1DRecords {
+    floatx4 m[4], l[4];
+};
+__device__ __forceinline__ void s1d_load_records(S1DRecords& r, const float* part, int count, int n, int g) {
+    auto fetch = [&](int k) {
+        int s = n + 16 * k;
+        s = s < count ? s : count - 1;
+        r.m[k] = *reinterpret_cast<const floatx4*>(part + s * 32 + 4 * g);
+        r.l[k] = *reinterpret_cast<const floatx4*>(part + s * 32 + 16 + 4 * g);
+    };
+    fetch(0);
+    if (count > 16) {                                          // uniform
+#pragma unroll
+        for (int k = 1; k < 4; ++k) fetch(k);
+    }
+}
+// log-sum-exp (log2 units) of head 4g + e from those records: each lane folds its own in run order, then the 16 lanes
+// of a row merge among themselves (the merge of (max, sum) pairs is associative and commutative up to rounding, and
+// every lane of a row ends with the same bits because the butterfly combines the same pairs in the same order on both
+// sides).
+__device__ __forceinline__ void s1d_merge_records(const S1DRecords& r, int count, int n, int g, int group, float (&lse2)[4]) {
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         float mm = -INFINITY, ll = 0.f;
-        for (int s = n; s < count; s += 16) {
-            const float mo = part[s * 32 + 4 * g + e], lo = part[s * 32 + 16 + 4 * g + e];
+        auto fold = [&](int k) {
+            const bool have = n + 16 * k < count;              // a record that is not there is the neutral element
+            const float mo = have ? r.m[k][e] : -INFINITY, lo = have ? r.l[k][e] : 0.f;
             const float mn = fmaxf(mm, mo);
             const float mu = (mn == -INFINITY) ? 0.f : mn;
             ll = ll * __builtin_amdgcn_exp2f(mm - mu) + lo * __builtin_amdgcn_exp2f(mo - mu);
             mm = mn;
+        };
+        fold(0);
+        if (count > 16) {                                      // uniform
+#pragma unroll
+            for (int k = 1; k < 4; ++k) fold(k);
         }
 #pragma unroll
         for (int off = 1; off < 16; off <<= 1) {
@@ -248,11 +274,22 @@ __device__ __forceinline__ float s1d_quad_xor2(float x) {
     return __uint_as_float(__builtin_amdgcn_mov_dpp(__float_as_uint(x), 0x4E, 0xF, 0xF, false));
 }
 
+// The 16 keys before tile t0 (the last group of tile t0 - 1), whose last key opens the first pooling window of a run
+// that does not start the row; with t0 == 0 the request goes to the row's first keys and is ignored.
+__device__ __forceinline__ void s1d_load_group_before(elem8 (&t4)[4], const S1DecodeSeq& sq, int64_t row_stride, int t0, int n, int g) {
+    int row = (t0 > 0 ? t0 * 64 - 16 : 0) + n;
+    row = row < sq.Lk ? row : sq.Lk - 1;
+    const elem_bits* src = sq.kbase + row * row_stride + 8 * g;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) t4[c] = *reinterpret_cast<const elem8*>(src + 32 * c);
+}
+
 // Scores (or pooled block scores) of the fine tiles [t0, t1) of one sequence and KV head, by one wavefront; ta / tb
-// hold tiles t0 and t0 + 1 already (requested by the caller before it waited for the log-sum-exp).
+// hold tiles t0 and t0 + 1 already and before4 the 16 keys before tile t0 (all requested by the caller before it
+// waited for the log-sum-exp).
 template <bool kPool>
 __device__ __forceinline__ void s1d_score_run(const S1DecodeParams& p, const S1DecodeSeq& sq, const elem8 (&qf)[4],
-                                              const float (&lse2)[4], elem8 (&ta)[16], elem8 (&tb)[16], int vis_f,
+                                              const float (&lse2)[4], const elem8 (&before4)[4], elem8 (&ta)[16], elem8 (&tb)[16], int vis_f,
                                               int tiles, int t0, int t1, bool owns_tail, int b, int h, int lane) {
     const int n = lane & 15, g = lane >> 4;
     const int64_t out_row = static_cast<int64_t>(h) * p.out_head_stride + static_cast<int64_t>(sq.q_row) * p.out_row_stride;
@@ -278,12 +315,7 @@ __device__ __forceinline__ void s1d_score_run(const S1DecodeParams& p, const S1D
 
     float carry = 0.f;                                         // score of the last key before the current tile
     if (kPool && t0 > 0 && t0 < t1) {
-        elem8 t4[4];
-        const int row = t0 * 64 - 16 + n;                      // keys of the last group of tile t0 - 1: all exist
-        const elem_bits* src = sq.kbase + row * p.k_row_stride + 8 * g;
-#pragma unroll
-        for (int c = 0; c < 4; ++c) t4[c] = *reinterpret_cast<const elem8*>(src + 32 * c);
-        const float part3 = group_part(t4);
+        const float part3 = group_part(before4);               // keys of the last group of tile t0 - 1: all exist
         float prev = s1d_fold_rows32(s1d_fold_rows16(0.f, 0.f), s1d_fold_rows16(0.f, part3));
         prev = (t0 * 64 - 64 + lane < vis_f) ? prev : 0.f;
         carry = __shfl(prev, 63);
@@ -352,18 +384,24 @@ void stage1_decode_score_kernel(const S1DecodeParams p) {
     const bool owns_tail = tiles == 0 ? split == 0 : (t0 < t1 && t1 == tiles);
     if (t0 >= t1 && !owns_tail) return;
 
-    elem8 qf[4];
-    s1d_load_q(qf, p, sq, h, n, g);
-    // the first two tiles are requested before anything waits on memory
-    elem8 ta[16], tb[16];
-    if (t0 < t1) s1d_load_tile(ta, sq.kbase, p.k_row_stride, t0 * 64, sq.Lk, n, g);
-    if (t0 + 1 < t1) s1d_load_tile(tb, sq.kbase, p.k_row_stride, (t0 + 1) * 64, sq.Lk, n, g);
-    // log-sum-exp of head 4g + e: the partials of the coarse runs merged in run order
-    float lse2[4];
+    // Everything this run reads is requested before anything waits on memory, in the order in which it is needed:
+    // the partial records of the log-sum-exp (merged while the keys are still on their way), the query, two tiles.
+    // A run has one or two tiles (more only when a sequence has over 128 of them); with one, the second request
+    // repeats the first, so that the number of requests in flight is the same on every path.
     int records = (((vis_c + 63) >> 6) + p.run_c - 1) / p.run_c;                    // the coarse runs of this sequence
     records = records < 1 ? 1 : records;
-    s1d_merge_partials(p.partial + (static_cast<int64_t>(b) * gridDim.y + h) * p.splits_c * 32, records, n, g, p.group, lse2);
-    s1d_score_run<kPool>(p, sq, qf, lse2, ta, tb, vis_f, tiles, t0, t1, owns_tail, b, h, lane);
+    S1DRecords rec;
+    elem8 qf[4], before4[4], ta[16], tb[16];
+    float lse2[4] = {0.f, 0.f, 0.f, 0.f};
+    if (t0 < t1) {                                             // uniform; otherwise this run only fills the row's tail
+        s1d_load_records(rec, p.partial + (static_cast<int64_t>(b) * gridDim.y + h) * p.splits_c * 32, records, n, g);
+        s1d_load_q(qf, p, sq, h, n, g);
+        if (kPool) s1d_load_group_before(before4, sq, p.k_row_stride, t0, n, g);
+        s1d_load_tile(ta, sq.kbase, p.k_row_stride, t0 * 64, sq.Lk, n, g);
+        s1d_load_tile(tb, sq.kbase, p.k_row_stride, (t0 + 1 < t1 ? t0 + 1 : t0) * 64, sq.Lk, n, g);
+        s1d_merge_records(rec, records, n, g, p.group, lse2);
+    }
+    s1d_score_run<kPool>(p, sq, qf, lse2, before4, ta, tb, vis_f, tiles, t0, t1, owns_tail, b, h, lane);
 }
 
 }  // namespace IV2_NS
