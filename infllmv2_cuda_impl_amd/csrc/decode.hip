@@ -104,7 +104,8 @@ __device__ __forceinline__ uint4 rotary_chunk(const DecodeParams& p, const elem_
     return make_uint4(pack_elem2(y[0], y[1]), pack_elem2(y[2], y[3]), pack_elem2(y[4], y[5]), pack_elem2(y[6], y[7]));
 }
 
-constexpr int kVtPitch = kHeadDim + 8;                         // LDS row pitch (elements) of the V tile
+constexpr int kVtPitch = kHeadDim + 16;                        // LDS row pitch (elements) of the V tile: rows 8 banks apart, so the
+                                                               // transposing reads of four rows at a time do not collide
 
 __global__ __launch_bounds__(256)
 void decode_append_kernel(const DecodeParams p) {
@@ -138,6 +139,13 @@ void decode_rotate_q_kernel(const DecodeParams p) {
     const int pos = p.cache_seqlens ? p.cache_seqlens[b] : 0;
     *reinterpret_cast<uint4*>(p.q_rot + (static_cast<int64_t>(b) * heads + head) * kHeadDim + chunk * 8) =
         rotary_chunk(p, p.q + b * p.q_batch + head * p.q_head, chunk, pos);
+}
+
+typedef short short4d __attribute__((ext_vector_type(4)));
+// 16 lanes x 4 halfwords, transposed (ds_read_b64_tr_b16): lane 16 g + r receives element r % 4 of the four-halfword
+// rows offered by lanes 16 g + r / 4 + {0, 4, 8, 12}
+__device__ __forceinline__ short4d lds_read_tr(const elem_bits* ptr) {
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4d*)(ptr));
 }
 
 template <bool kDirect>
@@ -190,13 +198,14 @@ void decode_split_kernel(const DecodeParams p) {
 
     int j = -1;
     for (int skip = 0; skip <= begin && count > 0; ++skip) j = walk.next();   // ordinal `begin` of the row
-    for (int it = 0; it < count && j >= 0; ++it) {
-        const int key0 = j * kBlockN;
-        // a block never straddles two pages (page_size is a multiple of 64 and paged caches have no left padding)
+    // K rows as A operands and the V rows of block jb, requested together; rows past the end are clamped to a valid row
+    // (K is masked below, P is zero there).  A block never straddles two pages (page_size is a multiple of 64 and
+    // paged caches have no left padding).
+    elem8 kreg[16], vreg[16];
+    auto request = [&](int jb) {
+        const int key0 = jb * kBlockN;
         const elem_bits* kbase = p.kcache + cache_row_offset(p, b, lp + key0, p.kc_batch, p.kc_row) + h * p.kc_head;
         const elem_bits* vbase = p.vcache + cache_row_offset(p, b, lp + key0, p.vc_batch, p.vc_row) + h * p.vc_head;
-        // K rows as A operands; rows past the end are clamped to a valid row and masked below
-        elem8 kreg[16];
 #pragma unroll
         for (int kt = 0; kt < 4; ++kt) {
             int key = key0 + 16 * kt + n;
@@ -205,27 +214,42 @@ void decode_split_kernel(const DecodeParams p) {
 #pragma unroll
             for (int c = 0; c < 4; ++c) kreg[kt * 4 + c] = *reinterpret_cast<const elem8*>(src + 32 * c);
         }
-        // V tile -> LDS, row-major
-        uint4 vreg[16];
 #pragma unroll
         for (int u = 0; u < 16; ++u) {
             const int unit = lane + 64 * u;
             int key = key0 + (unit >> 4);
             key = key < L ? key : L - 1;
-            vreg[u] = *reinterpret_cast<const uint4*>(vbase + static_cast<int64_t>(key - key0) * p.vc_row + (unit & 15) * 8);
+            vreg[u] = *reinterpret_cast<const elem8*>(vbase + static_cast<int64_t>(key - key0) * p.vc_row + (unit & 15) * 8);
         }
+    };
+    // One loop turn: S and the V tile of the block whose rows are in the registers (j), then - both register sets
+    // being free again - the request for the next block (j_req), then the softmax and P V of block j while those
+    // rows travel.  The first turn only requests.
+    int j_req = count > 0 ? j : -1, issued = 0;
+    j = -1;
+    for (;;) {
+        const int key0 = j * kBlockN;
         floatx4 s[4];
+        if (j >= 0) {
 #pragma unroll
-        for (int kt = 0; kt < 4; ++kt) {
-            s[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
+            for (int kt = 0; kt < 4; ++kt) {
+                s[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int c = 0; c < 4; ++c)
-                s[kt] = IV2_MFMA(kreg[kt * 4 + c], qf[c], s[kt], 0, 0, 0);
+                for (int c = 0; c < 4; ++c)
+                    s[kt] = IV2_MFMA(kreg[kt * 4 + c], qf[c], s[kt], 0, 0, 0);
+            }
+#pragma unroll
+            for (int u = 0; u < 16; ++u) {
+                const int unit = lane + 64 * u;
+                *reinterpret_cast<elem8*>(&vt[(unit >> 4) * kVtPitch + (unit & 15) * 8]) = vreg[u];
+            }
         }
-#pragma unroll
-        for (int u = 0; u < 16; ++u) {
-            const int unit = lane + 64 * u;
-            *reinterpret_cast<uint4*>(&vt[(unit >> 4) * kVtPitch + (unit & 15) * 8]) = vreg[u];
+        if (j_req >= 0) { request(j_req); ++issued; }
+        if (j < 0) {                                           // first turn: nothing to work on yet
+            if (j_req < 0) break;
+            j = j_req;
+            j_req = issued < count ? walk.next() : -1;
+            continue;
         }
         const int lim = L - 1 - key0;                           // in-block index of the last valid key
         if (lim < kBlockN - 1) {
@@ -268,27 +292,28 @@ void decode_split_kernel(const DecodeParams p) {
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __builtin_amdgcn_s_barrier();                          // single-wavefront workgroup: orders the LDS tile
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        // A operand of O^T += V^T P^T: lane (n, g) needs V[32 cc + 4 g + {0..3}, 32 cc + 16 + 4 g + {0..3}][16 dt + n], the
+        // keys in the order in which the lane holds P.  One transposing read hands a lane four rows' worth of one
+        // column: within 16 lanes, lane i offers the four columns 16 dt + 4 (i % 4) .. of key 4 g + i / 4 (+ 32 cc),
+        // and lane n receives column 16 dt + n of the keys 4 g + {0, 1, 2, 3}.
+        const elem_bits* tr_base = vt + (4 * g + (n >> 2)) * kVtPitch + 4 * (n & 3);
 #pragma unroll
         for (int dt = 0; dt < 8; ++dt)
 #pragma unroll
             for (int cc = 0; cc < 2; ++cc) {
-                const int d = 16 * dt + n;
-                uint32_t w[4];
-#pragma unroll
-                for (int jj = 0; jj < 8; jj += 2) {
-                    const int key = 32 * cc + (jj < 4 ? 4 * g + jj : 16 + 4 * g + jj - 4);
-                    w[jj >> 1] = static_cast<uint32_t>(vt[key * kVtPitch + d]) |
-                                 (static_cast<uint32_t>(vt[(key + 1) * kVtPitch + d]) << 16);
-                }
-                const uint4 raw = make_uint4(w[0], w[1], w[2], w[3]);
+                const short4d lo = lds_read_tr(tr_base + (32 * cc) * kVtPitch + 16 * dt);
+                const short4d hi = lds_read_tr(tr_base + (32 * cc + 16) * kVtPitch + 16 * dt);
                 elem8 vf;
-                __builtin_memcpy(&vf, &raw, 16);
+                __builtin_memcpy(&vf, &lo, 8);
+                __builtin_memcpy(reinterpret_cast<unsigned char*>(&vf) + 8, &hi, 8);
                 o[dt] = IV2_MFMA(vf, pf[cc], o[dt], 0, 0, 0);
             }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __builtin_amdgcn_s_barrier();                          // tile consumed before the next block overwrites it
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-        j = walk.next();
+        if (j_req < 0) break;
+        j = j_req;
+        j_req = issued < count ? walk.next() : -1;
     }
 
     const float l_tot = wave_sum_over_g(l);
