@@ -290,8 +290,8 @@ def decode_bench(torch, ops, dev):
     idx = ops.topk_blocks(pooled, topk).unsqueeze(2)
     s1_ms = event_ms(torch, s1, 20)
     topk_ms = event_ms(torch, lambda: ops.topk_blocks(pooled, topk, return_mask=True, by_index=True), 20)
-    append_ms = event_ms(torch, lambda: (ops.compress_keys_cache(kc, L, 32, 16, out=fine, old_lens=pos, max_new_rows=1),
-                                         ops.compress_keys_cache(kc, L, 128, 64, out=coarse, old_lens=pos, max_new_rows=1)), 20)
+    append = lambda: ops.compress_keys_cache_pair(kc, L, (32, 16, fine), (128, 64, coarse), old_lens=pos, max_new_rows=1)
+    append_ms = event_ms(torch, append, 20)
     s2_ms = event_ms(torch, lambda: ops.infllmv2_attn_with_kvcache(q, kc, vc, cache_seqlens=L, topk_idx=idx), 20)
     _, bm = ops.topk_blocks(pooled, topk, return_mask=True, by_index=True)
     bm = bm.unsqueeze(2)
@@ -303,11 +303,10 @@ def decode_bench(torch, ops, dev):
         return ops.infllmv2_attn_with_kvcache(q, kc, vc, cache_seqlens=L, block_mask=m.unsqueeze(2))
     step_ms = event_ms(torch, step, 20)
 
-    # the same step with the two compressed-key appends in front, once launched call by call and once as one captured
+    # the same step with the append to both compressed-key caches (one launch) in front, once launched call by call and once as one captured
     # HIP graph (a serving loop replays the graph: the gaps between the step's ten small launches disappear)
     def full_step():
-        ops.compress_keys_cache(kc, L, 32, 16, out=fine, old_lens=pos, max_new_rows=1)
-        ops.compress_keys_cache(kc, L, 128, 64, out=coarse, old_lens=pos, max_new_rows=1)
+        append()
         return step()
     full_ms = event_ms(torch, full_step, 20)
     graph = torch.cuda.CUDAGraph()

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define INFLLMV2_ABI_VERSION 10
+#define INFLLMV2_ABI_VERSION 11
 
 /* ---- library ------------------------------------------------------------------------------ */
 
@@ -147,6 +147,16 @@ int infllmv2_compress_keys_cache(void* stream, const void* kcache, void* out_cac
                                  int num_heads_k, int head_dim, const int64_t* kcache_strides,
                                  const int64_t* out_strides, int kernel_size, int stride, int kcache_rows,
                                  int out_rows);
+/* Two compressed caches of the same key cache in one call - the fine (kernel_size_a / stride_a) and the coarse
+ * (kernel_size_b / stride_b) keys that Stage 1 reads, which a decode step extends together: the same results as two
+ * calls of infllmv2_compress_keys_cache with the same lengths, in one launch when both are appends of a few rows. */
+int infllmv2_compress_keys_cache_pair(void* stream, const void* kcache, void* out_cache_a, void* out_cache_b,
+                                      const int32_t* old_lens, const int32_t* new_lens, int32_t* out_lens_a,
+                                      int32_t* out_lens_b, int batch, int max_new_rows_a, int max_new_rows_b,
+                                      int num_heads_k, int head_dim, const int64_t* kcache_strides,
+                                      const int64_t* out_strides_a, const int64_t* out_strides_b, int kernel_size_a,
+                                      int stride_a, int kernel_size_b, int stride_b, int kcache_rows, int out_rows_a,
+                                      int out_rows_b);
 
 /* ---- Stage 1: scoring over compressed keys --------------------------------------------------- */
 
@@ -349,6 +359,13 @@ int infllmv2_compress_keys_cache_f16(void* stream, const void* kcache, void* out
                                      int num_heads_k, int head_dim, const int64_t* kcache_strides,
                                      const int64_t* out_strides, int kernel_size, int stride, int kcache_rows,
                                      int out_rows);
+int infllmv2_compress_keys_cache_pair_f16(void* stream, const void* kcache, void* out_cache_a, void* out_cache_b,
+                                          const int32_t* old_lens, const int32_t* new_lens, int32_t* out_lens_a,
+                                          int32_t* out_lens_b, int batch, int max_new_rows_a, int max_new_rows_b,
+                                          int num_heads_k, int head_dim, const int64_t* kcache_strides,
+                                          const int64_t* out_strides_a, const int64_t* out_strides_b,
+                                          int kernel_size_a, int stride_a, int kernel_size_b, int stride_b,
+                                          int kcache_rows, int out_rows_a, int out_rows_b);
 int infllmv2_varlen_fwd_stage1_f16(void* stream, const void* q, const void* k, const void* v, void* score,
                                    const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
                                    const int32_t* cu_seqlens_v, int batch, int64_t total_q, int num_heads,

@@ -8,7 +8,7 @@ __version__ = "0.1.0"
 
 from .masks import blockmask_to_uint64, topk_to_uint64, uint64_to_bool, transpose_blockmask
 from .pooling import max_pooling_1d, max_pooling_1d_varlen
-from .selection import topk_blocks, compress_keys, compress_keys_cache, select_blocks
+from .selection import topk_blocks, compress_keys, compress_keys_cache, compress_keys_cache_pair, select_blocks
 from .attention import (
     infllmv2_attn_varlen_func,
     infllmv2_attn_stage1,
@@ -22,7 +22,7 @@ from .layer import BatchCache, InfLLMv2Attention, SequenceCache
 __all__ = [
     "BatchCache", "InfLLMv2Attention", "SequenceCache",
     "blockmask_to_uint64", "topk_to_uint64", "uint64_to_bool", "transpose_blockmask",
-    "max_pooling_1d", "max_pooling_1d_varlen", "topk_blocks", "compress_keys", "compress_keys_cache",
+    "max_pooling_1d", "max_pooling_1d_varlen", "topk_blocks", "compress_keys", "compress_keys_cache", "compress_keys_cache_pair",
     "select_blocks",
     "infllmv2_attn_varlen_func", "infllmv2_attn_stage1", "infllmv2_attn_stage1_pooled",
     "infllmv2_attn_stage1_kvcache",    "infllmv2_attn_with_kvcache",

@@ -11,7 +11,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libinfllmv2_hip.so")
 
-ABI_VERSION = 10
+ABI_VERSION = 11
 
 _p, _i, _i64, _sz, _f = C.c_void_p, C.c_int, C.c_int64, C.c_size_t, C.c_float
 
@@ -31,6 +31,7 @@ SIGNATURES = {
     "infllmv2_topk_select": [_p, _p, _i64, _i, _p, _p, _i64, _i, _i, _i, _i, _i],
     "infllmv2_compress_keys": [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i64, _i64, _i, _i, _i],
     "infllmv2_compress_keys_cache": [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _p, _p, _i, _i, _i, _i],
+    "infllmv2_compress_keys_cache_pair": [_p] * 8 + [_i] * 5 + [_p] * 3 + [_i] * 7,
     "infllmv2_varlen_fwd_stage1": [_p, _p, _p, _p, _p, _p, _p, _p, _i, _i64, _i, _i, _i, _i, _i, _p, _p, _p, _i64, _i64, _f, _i],
     "infllmv2_varlen_fwd_stage1_pooled": [_p] * 9 + [_i, _i, _i64, _i, _i, _i, _i, _i, _p, _p, _p, _i, _f] + [_i] * 7,
     "infllmv2_stage1_decode": [_p] * 11 + [_sz] + [_i] * 6 + [_p] * 3 + [_i64, _i64, _f, _i, _i, _p] + [_i] * 8,
@@ -42,7 +43,7 @@ SIGNATURES = {
     "infllmv2_pack_kv": [_p, _p, _p, _p, _p, _sz, _i, _i64, _i, _i, _i, _p, _p],
 }
 # entry points that exist once per element type: the plain name takes bfloat16, name + "_f16" IEEE half
-PER_ELEMENT_TYPE = ["infllmv2_compress_keys", "infllmv2_compress_keys_cache", "infllmv2_varlen_fwd_stage1",
+PER_ELEMENT_TYPE = ["infllmv2_compress_keys", "infllmv2_compress_keys_cache", "infllmv2_compress_keys_cache_pair", "infllmv2_varlen_fwd_stage1",
                     "infllmv2_varlen_fwd_stage1_pooled", "infllmv2_stage1_decode", "infllmv2_varlen_fwd",
                     "infllmv2_varlen_bwd", "infllmv2_fwd_kvcache"]
 for _name in PER_ELEMENT_TYPE:

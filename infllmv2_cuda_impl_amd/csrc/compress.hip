@@ -151,14 +151,13 @@ void compress_keys_cache_kernel(const CompressCacheParams p) {
 constexpr int kAppendUnits = 32;
 constexpr int kAppendMaxLds = 65536;
 
-__global__ __launch_bounds__(256)
-void compress_keys_cache_append_kernel(const CompressCacheParams p) {
-    extern __shared__ uint4 window[];                          // [kernel_size][kAppendUnits]
+// new_row: which of the sequence's new rows this workgroup takes
+__device__ __forceinline__ void append_one_row(const CompressCacheParams& p, int new_row, uint4* window) {
     const int b = blockIdx.y;
     int first, rows;
     cache_row_range(p, b, first, rows);
-    if (blockIdx.x == 0 && blockIdx.z == 0 && threadIdx.x == 0 && p.out_lens) p.out_lens[b] = rows;
-    const int j = first + blockIdx.x;
+    if (new_row == 0 && blockIdx.z == 0 && threadIdx.x == 0 && p.out_lens) p.out_lens[b] = rows;
+    const int j = first + new_row;
     if (j >= rows) return;                                     // uniform per workgroup
     const int u0 = blockIdx.z * kAppendUnits;
     const int nu = p.units_per_row - u0 < kAppendUnits ? p.units_per_row - u0 : kAppendUnits;
@@ -182,6 +181,20 @@ void compress_keys_cache_append_kernel(const CompressCacheParams p) {
     const int u = u0 + uu;
     p.out[b * p.o_batch + static_cast<int64_t>(j) * p.o_row + (u / p.units_per_head) * p.o_head + (u % p.units_per_head) * 8 + e] =
         f32_to_elem(acc / n);
+}
+
+__global__ __launch_bounds__(256)
+void compress_keys_cache_append_kernel(const CompressCacheParams p) {
+    extern __shared__ uint4 window[];                          // [kernel_size][kAppendUnits]
+    append_one_row(p, blockIdx.x, window);
+}
+// the appends to two compressed caches of the same key cache (the fine and the coarse keys of a decode step) in one
+// launch: the first rows_a workgroups of a sequence belong to cache a
+__global__ __launch_bounds__(256)
+void compress_keys_cache_append_pair_kernel(const CompressCacheParams pa, const CompressCacheParams pb, int rows_a) {
+    extern __shared__ uint4 window[];                          // [the larger kernel_size][kAppendUnits]
+    if (static_cast<int>(blockIdx.x) < rows_a) append_one_row(pa, blockIdx.x, window);
+    else append_one_row(pb, blockIdx.x - rows_a, window);
 }
 
 }  // namespace IV2_NS
@@ -218,21 +231,23 @@ extern "C" int IV2_ENTRY(infllmv2_compress_keys)(void* stream, const void* k, vo
     return 0;
 }
 
-extern "C" int IV2_ENTRY(infllmv2_compress_keys_cache)(void* stream, const void* kcache, void* out_cache, const int32_t* old_lens,
-                                            const int32_t* new_lens, int32_t* out_lens, int batch, int max_new_rows,
-                                            int num_heads_k, int head_dim, const int64_t* kcache_strides,
-                                            const int64_t* out_strides, int kernel_size, int stride,
-                                            int kcache_rows, int out_rows) {
-    IV2_CHECK(batch > 0 && batch <= 65535 && max_new_rows >= 0, "compress_keys_cache: bad batch or max_new_rows");
-    IV2_CHECK(kcache_rows >= 0 && out_rows >= 0, "compress_keys_cache: negative cache capacity");
-    IV2_CHECK(kernel_size > 0 && stride > 0, "compress_keys_cache: kernel_size and stride must be positive");
-    IV2_CHECK(kcache && out_cache && new_lens, "compress_keys_cache: null pointer");
-    IV2_CHECK(head_dim > 0 && head_dim % 8 == 0 && num_heads_k > 0, "compress_keys_cache: head_dim must be a multiple of 8");
+namespace {
+
+// checks and parameters of one compressed cache; 0 or an error code
+int cache_params(const char* who, CompressCacheParams& p, const void* kcache, void* out_cache, const int32_t* old_lens,
+                 const int32_t* new_lens, int32_t* out_lens, int batch, int max_new_rows, int num_heads_k, int head_dim,
+                 const int64_t* kcache_strides, const int64_t* out_strides, int kernel_size, int stride, int kcache_rows,
+                 int out_rows) {
+    IV2_CHECK(batch > 0 && batch <= 65535 && max_new_rows >= 0, "%s: bad batch or max_new_rows", who);
+    IV2_CHECK(kcache_rows >= 0 && out_rows >= 0, "%s: negative cache capacity", who);
+    IV2_CHECK(kernel_size > 0 && stride > 0, "%s: kernel_size and stride must be positive", who);
+    IV2_CHECK(kcache && out_cache && new_lens, "%s: null pointer", who);
+    IV2_CHECK(head_dim > 0 && head_dim % 8 == 0 && num_heads_k > 0, "%s: head_dim must be a multiple of 8", who);
     IV2_CHECK(reinterpret_cast<uintptr_t>(kcache) % 16 == 0 && reinterpret_cast<uintptr_t>(out_cache) % 16 == 0,
-              "compress_keys_cache: caches must be 16-byte aligned");
+              "%s: caches must be 16-byte aligned", who);
     for (int s = 0; s < 3; ++s)
-        IV2_CHECK(kcache_strides[s] % 8 == 0 && out_strides[s] % 8 == 0, "compress_keys_cache: strides must be multiples of 8 elements");
-    CompressCacheParams p{};
+        IV2_CHECK(kcache_strides[s] % 8 == 0 && out_strides[s] % 8 == 0, "%s: strides must be multiples of 8 elements", who);
+    p = CompressCacheParams{};
     p.k = static_cast<const elem_bits*>(kcache);
     p.out = static_cast<elem_bits*>(out_cache);
     p.old_lens = old_lens; p.new_lens = new_lens; p.out_lens = out_lens;
@@ -241,17 +256,65 @@ extern "C" int IV2_ENTRY(infllmv2_compress_keys_cache)(void* stream, const void*
     p.units_per_row = num_heads_k * head_dim / 8; p.units_per_head = head_dim / 8;
     p.kernel_size = kernel_size; p.stride = stride;
     p.k_capacity = kcache_rows; p.out_capacity = out_rows; p.max_new_rows = max_new_rows;
-    const size_t window_bytes = static_cast<size_t>(kernel_size) * kAppendUnits * 16;
-    if (max_new_rows >= 1 && max_new_rows <= 8 && window_bytes <= kAppendMaxLds) {
-        // a decode step's append: one workgroup per new row and 32 units
-        const dim3 grid(max_new_rows, batch, (p.units_per_row + kAppendUnits - 1) / kAppendUnits);
-        hipLaunchKernelGGL(compress_keys_cache_append_kernel, grid, dim3(256), window_bytes, static_cast<hipStream_t>(stream), p);
+    return 0;
+}
+size_t append_window_bytes(const CompressCacheParams& p) { return static_cast<size_t>(p.kernel_size) * kAppendUnits * 16; }
+// a decode step's append: one workgroup per new row and 32 units
+bool append_shaped(const CompressCacheParams& p) {
+    return p.max_new_rows >= 1 && p.max_new_rows <= 8 && append_window_bytes(p) <= kAppendMaxLds;
+}
+int launch_cache(hipStream_t st, const CompressCacheParams& p, int batch) {
+    if (append_shaped(p)) {
+        const dim3 grid(p.max_new_rows, batch, (p.units_per_row + kAppendUnits - 1) / kAppendUnits);
+        hipLaunchKernelGGL(compress_keys_cache_append_kernel, grid, dim3(256), append_window_bytes(p), st, p);
         IV2_LAUNCH_CHECK();
         return 0;
     }
     // at least one workgroup per sequence so that out_lens is always written
-    const int groups = max_new_rows > 0 ? (max_new_rows + kCompressRowsPerWg - 1) / kCompressRowsPerWg : 1;
-    hipLaunchKernelGGL(compress_keys_cache_kernel, dim3(groups, batch), dim3(256), 0, static_cast<hipStream_t>(stream), p);
+    const int groups = p.max_new_rows > 0 ? (p.max_new_rows + kCompressRowsPerWg - 1) / kCompressRowsPerWg : 1;
+    hipLaunchKernelGGL(compress_keys_cache_kernel, dim3(groups, batch), dim3(256), 0, st, p);
     IV2_LAUNCH_CHECK();
     return 0;
+}
+
+}  // namespace
+
+extern "C" int IV2_ENTRY(infllmv2_compress_keys_cache)(void* stream, const void* kcache, void* out_cache, const int32_t* old_lens,
+                                            const int32_t* new_lens, int32_t* out_lens, int batch, int max_new_rows,
+                                            int num_heads_k, int head_dim, const int64_t* kcache_strides,
+                                            const int64_t* out_strides, int kernel_size, int stride,
+                                            int kcache_rows, int out_rows) {
+    CompressCacheParams p;
+    if (int rc = cache_params("compress_keys_cache", p, kcache, out_cache, old_lens, new_lens, out_lens, batch, max_new_rows,
+                              num_heads_k, head_dim, kcache_strides, out_strides, kernel_size, stride, kcache_rows, out_rows))
+        return rc;
+    return launch_cache(static_cast<hipStream_t>(stream), p, batch);
+}
+
+extern "C" int IV2_ENTRY(infllmv2_compress_keys_cache_pair)(void* stream, const void* kcache, void* out_cache_a, void* out_cache_b,
+                                                 const int32_t* old_lens, const int32_t* new_lens, int32_t* out_lens_a,
+                                                 int32_t* out_lens_b, int batch, int max_new_rows_a, int max_new_rows_b,
+                                                 int num_heads_k, int head_dim, const int64_t* kcache_strides,
+                                                 const int64_t* out_strides_a, const int64_t* out_strides_b,
+                                                 int kernel_size_a, int stride_a, int kernel_size_b, int stride_b,
+                                                 int kcache_rows, int out_rows_a, int out_rows_b) {
+    CompressCacheParams pa, pb;
+    if (int rc = cache_params("compress_keys_cache_pair", pa, kcache, out_cache_a, old_lens, new_lens, out_lens_a, batch,
+                              max_new_rows_a, num_heads_k, head_dim, kcache_strides, out_strides_a, kernel_size_a, stride_a,
+                              kcache_rows, out_rows_a))
+        return rc;
+    if (int rc = cache_params("compress_keys_cache_pair", pb, kcache, out_cache_b, old_lens, new_lens, out_lens_b, batch,
+                              max_new_rows_b, num_heads_k, head_dim, kcache_strides, out_strides_b, kernel_size_b, stride_b,
+                              kcache_rows, out_rows_b))
+        return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (append_shaped(pa) && append_shaped(pb)) {
+        const size_t lds = append_window_bytes(pa) > append_window_bytes(pb) ? append_window_bytes(pa) : append_window_bytes(pb);
+        const dim3 grid(pa.max_new_rows + pb.max_new_rows, batch, (pa.units_per_row + kAppendUnits - 1) / kAppendUnits);
+        hipLaunchKernelGGL(compress_keys_cache_append_pair_kernel, grid, dim3(256), lds, st, pa, pb, pa.max_new_rows);
+        IV2_LAUNCH_CHECK();
+        return 0;
+    }
+    if (int rc = launch_cache(st, pa, batch)) return rc;
+    return launch_cache(st, pb, batch);
 }

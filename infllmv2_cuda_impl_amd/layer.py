@@ -27,7 +27,7 @@ import torch
 from .attention import (infllmv2_attn_stage1_kvcache, infllmv2_attn_stage1_pooled, infllmv2_attn_varlen_func,
                         infllmv2_attn_with_kvcache)
 from .pooling import max_pooling_1d_varlen
-from .selection import compress_keys, compress_keys_cache, select_blocks, topk_blocks
+from .selection import compress_keys, compress_keys_cache, compress_keys_cache_pair, select_blocks, topk_blocks
 
 
 @dataclass
@@ -202,9 +202,9 @@ class InfLLMv2Attention(torch.nn.Module):
         new = old + 1
         # the selection needs the new key inside the compressed keys; the decode kernel's own append rewrites the row
         cache.k[torch.arange(batch, device=q.device), old.long()] = k_new[:, 0]
-        for buf, lens, ks, st in ((cache.k_fine, cache.fine_lens, self.kernel_size, self.stride),
-                                  (cache.k_coarse, cache.coarse_lens, 4 * self.kernel_size, 4 * self.stride)):
-            compress_keys_cache(cache.k, new, ks, st, out=buf, old_lens=old, max_new_rows=1, out_lens=lens)
+        compress_keys_cache_pair(cache.k, new, (self.kernel_size, self.stride, cache.k_fine),
+                                 (4 * self.kernel_size, 4 * self.stride, cache.k_coarse), old_lens=old, max_new_rows=1,
+                                 out_lens=(cache.fine_lens, cache.coarse_lens))
         mask = None
         if self.selection == "window" and cache.max_length + 1 > self.dense_len:
             cu_one = torch.arange(batch + 1, dtype=torch.int32, device=q.device)

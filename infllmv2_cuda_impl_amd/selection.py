@@ -117,6 +117,44 @@ def compress_keys_cache(k_cache: torch.Tensor, new_lens: torch.Tensor, kernel_si
     return out_lens
 
 
+def compress_keys_cache_pair(k_cache: torch.Tensor, new_lens: torch.Tensor, fine, coarse, old_lens: torch.Tensor | None = None,
+                             max_new_rows: int | None = None, out_lens=(None, None)):
+    """:func:`compress_keys_cache` for the two compressed caches Stage 1 reads, in one call (one launch when both are
+    appends of a few rows, as in a decode step): ``fine`` and ``coarse`` are ``(kernel_size, stride, out)`` triples, e.g.
+    ``(32, 16, k_fine)`` and ``(128, 64, k_coarse)``.  Same results as two separate calls.  Returns the two ``out_lens``."""
+    require_gpu(k_cache, "k_cache")
+    (ks_a, st_a, out_a), (ks_b, st_b, out_b) = fine, coarse
+    if k_cache.dtype not in (torch.float16, torch.bfloat16) or out_a.dtype != k_cache.dtype or out_b.dtype != k_cache.dtype:
+        raise RuntimeError("FlashAttention only support fp16 and bf16 data type")
+    for out in (out_a, out_b):
+        if k_cache.dim() != 4 or out.dim() != 4 or k_cache.stride(-1) != 1 or out.stride(-1) != 1 or \
+                out.shape[0] != k_cache.shape[0] or tuple(out.shape[2:]) != tuple(k_cache.shape[2:]):
+            raise RuntimeError("k_cache and out must have shapes (batch, capacity, num_heads_k, head_size) and "
+                               "(batch, rows, num_heads_k, head_size)")
+    batch, cap, Hk, d = k_cache.shape
+    for name, t in (("new_lens", new_lens), ("old_lens", old_lens)):
+        if t is not None and (t.dtype != torch.int32 or tuple(t.shape) != (batch,) or not t.is_contiguous()):
+            raise RuntimeError(f"{name} must be a contiguous int32 tensor of shape (batch_size)")
+    rows = []
+    for ks, st, out in ((ks_a, st_a, out_a), (ks_b, st_b, out_b)):
+        if max_new_rows is None:
+            if (cap - ks) // st + 1 > out.shape[1]:
+                raise RuntimeError("out has fewer rows than the key cache has windows")
+            rows.append(out.shape[1])
+        elif max_new_rows < 0:
+            raise RuntimeError("max_new_rows must not be negative")
+        else:
+            rows.append(int(max_new_rows))
+    lens_a, lens_b = [torch.empty(batch, dtype=torch.int32, device=k_cache.device) if t is None else t for t in out_lens]
+    s3 = lambda t: _lib.i64_array([t.stride(0), t.stride(1), t.stride(2)])
+    with torch.cuda.device(k_cache.device):
+        _lib.call_for(k_cache.dtype, "infllmv2_compress_keys_cache_pair", stream_ptr(k_cache.device), k_cache.data_ptr(),
+                      out_a.data_ptr(), out_b.data_ptr(), None if old_lens is None else old_lens.data_ptr(), new_lens.data_ptr(),
+                      lens_a.data_ptr(), lens_b.data_ptr(), batch, rows[0], rows[1], Hk, d, s3(k_cache), s3(out_a), s3(out_b),
+                      ks_a, st_a, ks_b, st_b, cap, out_a.shape[1], out_b.shape[1])
+    return lens_a, lens_b
+
+
 def select_blocks(q: torch.Tensor, k: torch.Tensor, cu_seqlens_q: torch.Tensor, cu_seqlens_k: torch.Tensor,
                   max_seqlen_q: int, max_seqlen_k: int, topk: int, local_blocks: int, init_blocks: int,
                   cache_lens: torch.Tensor | None = None, max_cache_len: int | None = None, softmax_scale=None,

@@ -171,6 +171,33 @@ def test_append_of_a_few_rows_equals_the_full_build(ops, dtype, Hk, d, ks, st, j
     assert torch.equal(inc, full)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_both_compressed_caches_in_one_call(ops, dtype):
+    """compress_keys_cache_pair == two compress_keys_cache calls, bit for bit: the full build (two launches inside), a
+    one-token step and a step of a few tokens (one launch for both caches), undersized second cache included."""
+    lens = [0, 31, 32, 127, 128, 129, 1000, 47, 640]
+    B, cap = len(lens), 1100
+    g = torch.Generator(device="cpu").manual_seed(23)
+    kcache = torch.randn(B, cap, 2, 128, generator=g).to(dtype).to(DEV)
+    L = torch.tensor(lens, dtype=torch.int32, device=DEV)
+    shapes = ((32, 16, cap // 16 + 1), (128, 64, 12))          # the coarse cache holds 12 rows only
+    mk = lambda: [torch.full((B, r, 2, 128), 7.0, dtype=dtype, device=DEV) for _, _, r in shapes]
+    one, two = mk(), mk()
+    la, lb = ops.compress_keys_cache_pair(kcache, L, (32, 16, one[0]), (128, 64, one[1]), max_new_rows=cap)
+    ra = ops.compress_keys_cache(kcache, L, 32, 16, out=two[0], max_new_rows=cap)
+    rb = ops.compress_keys_cache(kcache, L, 128, 64, out=two[1], max_new_rows=cap)
+    assert torch.equal(la, ra) and torch.equal(lb, rb) and torch.equal(one[0], two[0]) and torch.equal(one[1], two[1])
+    for jump in (1, 1, 1, 40, 1, 100):
+        new = L + jump
+        la, lb = ops.compress_keys_cache_pair(kcache, new, (32, 16, one[0]), (128, 64, one[1]), old_lens=L, max_new_rows=7)
+        ra = ops.compress_keys_cache(kcache, new, 32, 16, out=two[0], old_lens=L, max_new_rows=7)
+        rb = ops.compress_keys_cache(kcache, new, 128, 64, out=two[1], old_lens=L, max_new_rows=7)
+        assert torch.equal(la, ra) and torch.equal(lb, rb)
+        assert torch.equal(one[0], two[0]) and torch.equal(one[1], two[1])
+        L = new
+    assert int(lb.max()) == 12 and int(la.max()) == O.compressed_len(cap, 32, 16)     # 1144 tokens read as the capacity
+
+
 def test_compressed_cache_capacity_bounds_what_is_written(ops):
     """An undersized compressed cache, or a step that completes more windows than max_new_rows covers: nothing is
     written beyond the cache's rows, and out_lens counts only rows the call did write (the kernels get both
