@@ -55,6 +55,8 @@ def batch_inputs(seed, lens, Hk=2, exact=False):
     ([20000], False, False),                                   # one sequence: many runs per (sequence, head)
     ([5000, 700], False, True),                                # exact softmax: the log-sum-exp over the fine keys themselves
     ([64 * 17 + 5] * 40, False, False),                       # more (sequence, head) pairs than runs wanted: short runs
+    ([140000, 300], False, False),                            # over 128 fine tiles: runs of three tiles
+    ([140000], True, True),                                    # ... and, the log-sum-exp over the same keys, coarse runs of three
 ])
 def test_scores_pooled_and_layouts(ops, lens, causal, exact):
     q, k, cu, kf, cu_f, kc, cu_c = batch_inputs(1, lens, exact=exact)
