@@ -340,7 +340,10 @@ void decode_split_kernel(const DecodeParams p) {
     }
 }
 
-// merge the per-split partials: one workgroup per (sequence, KV head); thread t -> head t / 16, 8 columns
+// merge the per-split partials: one workgroup per (sequence, KV head); thread t -> head t / 16, 8 columns.
+// kSplits > 0: the split count is known at compile time, so every partial is requested before the first is used
+// (one round trip to memory instead of one per split); 0: any count.
+template <int kSplits>
 __global__ __launch_bounds__(256)
 void decode_combine_kernel(const DecodeParams p) {
     const int h = blockIdx.x, b = blockIdx.y;
@@ -348,21 +351,44 @@ void decode_combine_kernel(const DecodeParams p) {
     const int head = tid >> 4, d0 = (tid & 15) * 8;
     if (head >= p.group) return;                               // partial rows that only filled the MFMA tile
     const int64_t slot0 = (static_cast<int64_t>(b) * p.num_heads_k + h) * p.splits;
-    float mx = -INFINITY;
-    for (int s = 0; s < p.splits; ++s) mx = fmaxf(mx, p.lse_part[(slot0 + s) * 16 + head]);
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    float wsum = 0.f;
-    if (mx != -INFINITY) {
-        for (int s = 0; s < p.splits; ++s) {
-            const float ls = p.lse_part[(slot0 + s) * 16 + head];
-            if (ls == -INFINITY) continue;
-            const float w = expf(ls - mx);
-            wsum += w;
+    float wsum = 0.f, mx = -INFINITY;
+    if constexpr (kSplits > 0) {
+        float ls[kSplits];
+        float4 a[kSplits], c[kSplits];
+#pragma unroll
+        for (int s = 0; s < kSplits; ++s) ls[s] = p.lse_part[(slot0 + s) * 16 + head];
+#pragma unroll
+        for (int s = 0; s < kSplits; ++s) {
             const float* src = p.o_part + ((slot0 + s) * 16 + head) * kHeadDim + d0;
-            const float4 a = *reinterpret_cast<const float4*>(src);
-            const float4 c = *reinterpret_cast<const float4*>(src + 4);
-            acc[0] += w * a.x; acc[1] += w * a.y; acc[2] += w * a.z; acc[3] += w * a.w;
-            acc[4] += w * c.x; acc[5] += w * c.y; acc[6] += w * c.z; acc[7] += w * c.w;
+            a[s] = *reinterpret_cast<const float4*>(src);
+            c[s] = *reinterpret_cast<const float4*>(src + 4);
+        }
+#pragma unroll
+        for (int s = 0; s < kSplits; ++s) mx = fmaxf(mx, ls[s]);
+        if (mx != -INFINITY) {
+#pragma unroll
+            for (int s = 0; s < kSplits; ++s) {
+                const float w = ls[s] == -INFINITY ? 0.f : expf(ls[s] - mx);       // a split without blocks: zeros and -inf
+                wsum += w;
+                acc[0] += w * a[s].x; acc[1] += w * a[s].y; acc[2] += w * a[s].z; acc[3] += w * a[s].w;
+                acc[4] += w * c[s].x; acc[5] += w * c[s].y; acc[6] += w * c[s].z; acc[7] += w * c[s].w;
+            }
+        }
+    } else {
+        for (int s = 0; s < p.splits; ++s) mx = fmaxf(mx, p.lse_part[(slot0 + s) * 16 + head]);
+        if (mx != -INFINITY) {
+            for (int s = 0; s < p.splits; ++s) {
+                const float ls = p.lse_part[(slot0 + s) * 16 + head];
+                if (ls == -INFINITY) continue;
+                const float w = expf(ls - mx);
+                wsum += w;
+                const float* src = p.o_part + ((slot0 + s) * 16 + head) * kHeadDim + d0;
+                const float4 a = *reinterpret_cast<const float4*>(src);
+                const float4 c = *reinterpret_cast<const float4*>(src + 4);
+                acc[0] += w * a.x; acc[1] += w * a.y; acc[2] += w * a.z; acc[3] += w * a.w;
+                acc[4] += w * c.x; acc[5] += w * c.y; acc[6] += w * c.z; acc[7] += w * c.w;
+            }
         }
     }
     const float inv = wsum > 0.f ? 1.f / wsum : 0.f;
@@ -501,7 +527,14 @@ static int fwd_kvcache_impl(void* stream, const void* q, void* kcache, void* vca
         p.lse_part = ws + static_cast<size_t>(batch) * num_heads_k * num_splits * 16 * kHeadDim;
         hipLaunchKernelGGL(decode_split_kernel<false>, grid, dim3(64), 0, st, p);
         IV2_LAUNCH_CHECK();
-        hipLaunchKernelGGL(decode_combine_kernel, dim3(num_heads_k, batch), dim3(256), 0, st, p);
+        const dim3 cgrid(num_heads_k, batch);
+        switch (num_splits) {
+            case 2: hipLaunchKernelGGL(decode_combine_kernel<2>, cgrid, dim3(256), 0, st, p); break;
+            case 4: hipLaunchKernelGGL(decode_combine_kernel<4>, cgrid, dim3(256), 0, st, p); break;
+            case 8: hipLaunchKernelGGL(decode_combine_kernel<8>, cgrid, dim3(256), 0, st, p); break;
+            case 16: hipLaunchKernelGGL(decode_combine_kernel<16>, cgrid, dim3(256), 0, st, p); break;
+            default: hipLaunchKernelGGL(decode_combine_kernel<0>, cgrid, dim3(256), 0, st, p); break;
+        }
         IV2_LAUNCH_CHECK();
     }
     return 0;
