@@ -103,11 +103,36 @@ def make_inputs(torch, S, dev, seed=0):
     return q, k, v, kf, kc, mk(S), mk(kf.shape[0]), mk(kc.shape[0])
 
 
+_SLEEP_CYCLES_PER_MS = None
+
+
+def hold_device(torch, ms):
+    """Keep the stream busy for about `ms` milliseconds (a spinning kernel), so that the launches enqueued after it are
+    all queued by the time the device gets to them: what is timed behind it is device time, not how fast this process
+    can issue launches.  No-op when torch has no spin kernel."""
+    global _SLEEP_CYCLES_PER_MS
+    sleep = getattr(torch.cuda, "_sleep", None)
+    if sleep is None:
+        return
+    if _SLEEP_CYCLES_PER_MS is None:                           # the spin kernel's clock differs between devices: measure it once
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        sleep(1000)
+        torch.cuda.synchronize()
+        e0.record()
+        sleep(200000)
+        e1.record()
+        torch.cuda.synchronize()
+        _SLEEP_CYCLES_PER_MS = 200000 / max(e0.elapsed_time(e1), 1e-3)
+    sleep(int(ms * _SLEEP_CYCLES_PER_MS))
+
+
 def event_ms(torch, fn, iters, warmup=2):
+    """Device time per call of fn, HIP events around `iters` back-to-back calls queued behind a short spin."""
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    hold_device(torch, 0.5 + 0.1 * iters)
     e0.record()
     for _ in range(iters):
         fn()
