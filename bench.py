@@ -123,7 +123,7 @@ def hold_device(torch, ms):
         e1.record()
         torch.cuda.synchronize()
         _SLEEP_CYCLES_PER_MS = 200000 / max(e0.elapsed_time(e1), 1e-3)
-    sleep(int(ms * _SLEEP_CYCLES_PER_MS))
+    sleep(int(min(ms, 5.0) * min(_SLEEP_CYCLES_PER_MS, 5e6)))   # bounded whatever the calibration read: at most 5 ms of a 5 GHz clock
 
 
 def event_ms(torch, fn, iters, warmup=2):
