@@ -162,7 +162,16 @@ def copy_bandwidth(torch, dev):
     src = torch.ones(1 << 30, dtype=torch.uint8, device=dev)
     dst = torch.empty_like(src)
     ms = event_ms(torch, lambda: dst.copy_(src), 10)
-    return {"gbs": 2 * src.numel() / ms / 1e6, "ms": ms, "what": "torch copy_ of 1 GiB, read + write bytes"}
+    out = {"gbs": 2 * src.numel() / ms / 1e6, "ms": ms, "what": "torch copy_ of 1 GiB, read + write bytes"}
+    del dst
+    # what a read-only stream gets: a library reduction over 1 GiB (HBM) and over 184 MiB, the size of the decode
+    # step's compressed keys, which the last-level cache partly holds between the timed calls
+    f32 = src.view(torch.float32)
+    for name, t in (("read_only_1gib_gbs", f32), ("read_only_184mib_gbs", f32[:184 << 18])):
+        ms_r = event_ms(torch, t.sum, 10)
+        out[name] = t.numel() * 4 / ms_r / 1e6
+    out["read_only_what"] = "torch sum over fp32, bytes read"
+    return out
 
 
 def sharing_stats(torch, ops, dev):
